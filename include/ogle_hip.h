@@ -1,0 +1,278 @@
+/*
+ * ogle_hip.h - C ABI of the MI355X (gfx950) kernels behind OGLE's convolution
+ * hot path.
+ *
+ * This is the boundary the reference's "Program" layer is replaced at.  In the
+ * reference, Kernel::Compute sets uniforms on a GLSL program and issues one
+ * draw call (ogl_runtime/opengl/core/program.h:30-103, used by
+ * ogl_runtime/opengl/nn/kernels/conv2d.cc:116-167).  Here the same call sites
+ * fill a plain struct and call one entry point, which launches hand-written
+ * HIP kernels on the given stream.
+ *
+ * Conventions
+ *  - Every pointer named *_dev is device memory owned by the caller.  Unless an
+ *    entry point says otherwise nothing here allocates, frees or synchronises:
+ *    launches are asynchronous on `stream`.
+ *  - Activations are dense NHWC, channel contiguous, no per-pixel padding.
+ *    Logical shapes are the reference's (Tensor::shape() NHWC, filters OIHW).
+ *  - Filters are consumed in a packed device layout produced once at load time
+ *    by ogle_hip_pack_filter (the counterpart of the reference's
+ *    NCHW -> HWN4C4 upload, ogl_runtime/opengl/nn/kernels/const.cc:21-28).
+ *  - Return value: OGLE_OK (0) or a negative OgleStatus.  Entry points never
+ *    abort; ogle_hip_last_error() gives the message of the calling thread's
+ *    last failure.  The reference aborts through glog CHECK / LOG(FATAL)
+ *    (ogl_runtime/opengl/utils/macros.h:16-20); its Kernel wrappers turn a
+ *    non-zero status back into that behaviour.
+ *  - `stream` is a hipStream_t passed as void* so that this header needs no
+ *    HIP include; NULL is the default stream.
+ */
+#ifndef OGLE_HIP_H_
+#define OGLE_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* ogle_stream_t;
+
+typedef enum OgleStatus {
+  OGLE_OK = 0,
+  OGLE_ERR_INVALID_ARG = -1, /* shape/attribute violates what the op allows */
+  OGLE_ERR_UNSUPPORTED = -2, /* valid request, no kernel for it             */
+  OGLE_ERR_LAUNCH = -3,      /* HIP reported an error at launch             */
+  OGLE_ERR_NOT_FOUND = -4,   /* registry lookup failed                      */
+  OGLE_ERR_NO_DEVICE = -5    /* no gfx950 device / code object              */
+} OgleStatus;
+
+typedef enum OgleDType { OGLE_F32 = 0, OGLE_F16 = 1 } OgleDType;
+
+/* Fused activation codes: the reference's "act" uniform
+ * (ogl_runtime/opengl/nn/kernels/conv2d.cc:137-147). */
+typedef enum OgleAct { OGLE_ACT_NONE = 0, OGLE_ACT_CLIP = 1, OGLE_ACT_RELU = 2 } OgleAct;
+
+/* How a shader variant reads min/max for the fused activation.
+ * NHWC4: conv2d.glsl:82-90 (clamp(x,min,max); relu max(0,x)).
+ * PW:    conv2d_pw.glsl:85 (clamp(x,0,max): min ignored).
+ * ANY4:  conv2d_any4.glsl:89-94 (relu is max(min,x)). */
+typedef enum OgleActVariant {
+  OGLE_VARIANT_NHWC4 = 0,
+  OGLE_VARIANT_PW = 1,
+  OGLE_VARIANT_ANY4 = 2
+} OgleActVariant;
+
+/* Packed filter layouts. */
+typedef enum OgleFilterLayout {
+  OGLE_FILTER_OHWI = 0, /* [O][kh][kw][I/g]: dense, pointwise, grouped */
+  OGLE_FILTER_HWC = 1   /* [kh*kw][C]: depthwise (multiplier 1)        */
+} OgleFilterLayout;
+
+/* ------------------------------------------------------------------------ */
+/* Library / registry                                                         */
+/* ------------------------------------------------------------------------ */
+
+/* Version of this ABI (major*100 + minor). */
+int32_t ogle_hip_abi_version(void);
+
+/* Message of the calling thread's most recent failure ("" if none). */
+const char* ogle_hip_last_error(void);
+const char* ogle_hip_status_string(int32_t status);
+
+/*
+ * Kernel registry: replaces the generated shader table (all_shaders.h, built
+ * by ogl_runtime/opengl/nn/makeshader.py:16-43) and the program cache of
+ * Context::CreateProgram (ogl_runtime/opengl/core/context.cc:288-313).
+ * `name` is the shader's stem ("conv2d", "conv2d_dw", "conv2d_pw",
+ * "conv2d_grp", "conv2d_any4", "conv2d_dw_any4", "conv2d_pw_any4", "pool",
+ * "pool_any4", "concat_multi", "decoder"); `options` is the build-option text
+ * the Kernel composed ("#define USE_BIAS\n#define USE_CLIP\n", may be NULL).
+ * On success *handle identifies the HIP kernel family and its compile-time
+ * flags; it is what OgleConvArgs.kernel carries.
+ */
+int32_t ogle_hip_registry_lookup(const char* name, const char* options, int32_t* handle);
+int32_t ogle_hip_registry_size(void);
+const char* ogle_hip_registry_name(int32_t index);
+
+/* Waits for everything queued on `stream` (glFinish's counterpart,
+ * ogl_runtime/opengl/nn/profiler/traceme.h:61-65). */
+int32_t ogle_hip_sync(ogle_stream_t stream);
+
+/* ------------------------------------------------------------------------ */
+/* Filter upload                                                              */
+/* ------------------------------------------------------------------------ */
+
+/* Number of elements of the packed filter for an OIHW filter (o, i, kh, kw). */
+int64_t ogle_hip_packed_filter_elems(int32_t layout, int32_t o, int32_t i, int32_t kh,
+                                     int32_t kw);
+
+/*
+ * Repacks an OIHW fp32 filter (device memory, the order the .dlx file stores,
+ * converter/converter/onnx/ops/conv2d.cc:12-27) into `layout` with element type
+ * `dtype`.  Counterpart of functor::ConvertTensorNCHWToHWN4C4
+ * (ogl_runtime/opengl/core/functor.cc:45-93, shader nchw_to_hwn4c4.glsl).
+ * For OGLE_FILTER_HWC, i must be 1.
+ */
+int32_t ogle_hip_pack_filter(const float* oihw_dev, void* packed_dev, int32_t layout,
+                             int32_t dtype, int32_t o, int32_t i, int32_t kh, int32_t kw,
+                             ogle_stream_t stream);
+
+/* Element-type conversion of a flat buffer (fp32 <-> fp16 storage). */
+int32_t ogle_hip_convert(const void* src_dev, int32_t src_dtype, void* dst_dev,
+                         int32_t dst_dtype, int64_t count, ogle_stream_t stream);
+
+/* ------------------------------------------------------------------------ */
+/* Convolution                                                                */
+/* ------------------------------------------------------------------------ */
+
+/*
+ * Arguments of one convolution launch: the uniforms and texture bindings of
+ * Conv2DKernel::Compute (ogl_runtime/opengl/nn/kernels/conv2d.cc:127-164).
+ */
+typedef struct OgleConvArgs {
+  const void* input_dev;  /* NHWC (n, in_h, in_w, in_c), dtype               */
+  const void* filter_dev; /* packed by ogle_hip_pack_filter, dtype            */
+  const float* bias_dev;  /* (out_c) fp32, or NULL (no USE_BIAS)              */
+  void* output_dev;       /* NHWC (n, out_h, out_w, out_c), dtype             */
+  int32_t n, in_h, in_w, in_c;
+  int32_t out_h, out_w, out_c;
+  int32_t kernel_size, stride, padding, dilation, group;
+  int32_t act;         /* OgleAct                                             */
+  float min_value;     /* "min_value" uniform                                 */
+  float max_value;     /* "max_value" uniform                                 */
+  int32_t act_variant; /* OgleActVariant                                      */
+  int32_t dtype;       /* OgleDType of input/filter/output; accumulation fp32 */
+} OgleConvArgs;
+
+/* Dense (group 1) or grouped KxK convolution: conv2d.glsl:29-92,
+ * conv2d_grp.glsl:30-123, conv2d_any4.glsl:29-96.  Filter layout OHWI. */
+int32_t ogle_hip_conv2d(const OgleConvArgs* args, ogle_stream_t stream);
+
+/* Depthwise KxK (group == in_c == out_c): conv2d_dw.glsl:38-96,
+ * conv2d_dw_any4.glsl:38-98.  Filter layout HWC. */
+int32_t ogle_hip_dwconv2d(const OgleConvArgs* args, ogle_stream_t stream);
+
+/* Pointwise 1x1, stride 1, pad 0, group 1, as a GEMM
+ * [n*h*w, in_c] x [out_c, in_c]^T: conv2d_pw.glsl:35-91,
+ * conv2d_pw_any4.glsl:35-88.  Filter layout OHWI (== [O][I]). */
+int32_t ogle_hip_pwconv_gemm(const OgleConvArgs* args, ogle_stream_t stream);
+
+/* ------------------------------------------------------------------------ */
+/* Pooling                                                                    */
+/* ------------------------------------------------------------------------ */
+
+/* pool_type as ogl_runtime/opengl/nn/kernels/pool.h:10-14. */
+typedef enum OglePoolType { OGLE_POOL_MAX = 0, OGLE_POOL_AVG = 1, OGLE_POOL_GLOBAL_AVG = 2 } OglePoolType;
+
+/* Uniforms of PoolKernel::Compute (ogl_runtime/opengl/nn/kernels/pool.cc:53-79). */
+typedef struct OglePoolArgs {
+  const void* input_dev; /* NHWC */
+  void* output_dev;      /* NHWC (n, out_h, out_w, c) */
+  int32_t n, in_h, in_w, c;
+  int32_t out_h, out_w;
+  int32_t kernel_size, stride, padding;
+  int32_t pool_type; /* OglePoolType; for GLOBAL_AVG the caller sets
+                        kernel_size = in_h, stride 1, padding 0 (pool.cc:84-91) */
+  int32_t dtype;
+} OglePoolArgs;
+
+/* pool.glsl:19-66 / pool_any4.glsl. */
+int32_t ogle_hip_pool2d(const OglePoolArgs* args, ogle_stream_t stream);
+
+/* ------------------------------------------------------------------------ */
+/* Concat                                                                     */
+/* ------------------------------------------------------------------------ */
+
+#define OGLE_CONCAT_MAX_INPUTS 16
+
+/*
+ * Concatenation of n_inputs tensors along one axis: ConcatKernel::Compute
+ * (ogl_runtime/opengl/nn/kernels/concat.cc:56-97) with the intended semantics
+ * of concat_multi.glsl:14-114 (numpy.concatenate).  Each input i is viewed as
+ * (outer, axis_len[i], inner) row-major and lands at its running offset along
+ * the axis of the (outer, sum axis_len, inner) output.  One launch for all
+ * inputs.  n_inputs <= OGLE_CONCAT_MAX_INPUTS.
+ */
+typedef struct OgleConcatArgs {
+  const void* inputs_dev[OGLE_CONCAT_MAX_INPUTS];
+  int64_t axis_len[OGLE_CONCAT_MAX_INPUTS];
+  void* output_dev;
+  int32_t n_inputs;
+  int64_t outer;
+  int64_t inner;
+  int32_t dtype;
+} OgleConcatArgs;
+
+int32_t ogle_hip_concat(const OgleConcatArgs* args, ogle_stream_t stream);
+
+/* ------------------------------------------------------------------------ */
+/* SSD box decoder and score filter                                           */
+/* ------------------------------------------------------------------------ */
+
+/*
+ * Box decode: decoder.glsl:13-28 as driven by DecoderKernel::Compute
+ * (ogl_runtime/opengl/nn/kernels/decoder.cc:33-58) and
+ * functor::SSDBBoxDecoder (ogl_runtime/opengl/core/functor.cc:96-143).
+ * prediction (batch, priors, 4) = (tx,ty,tw,th); anchors (cx,cy,w,h);
+ * output (batch, priors, 4) = (xmin,ymin,xmax,ymax).  anchors_batch_stride is
+ * 0 when every image shares one (priors,4) anchor set (the functor form) or
+ * priors*4 when anchors are (batch, priors, 4) (the graph-op form,
+ * decoder.cc:82-85).
+ */
+typedef struct OgleDecodeArgs {
+  const float* prediction_dev;
+  const float* anchors_dev;
+  float* boxes_dev;
+  int32_t batch, priors;
+  int64_t anchors_batch_stride;
+  float variances[4];
+} OgleDecodeArgs;
+
+int32_t ogle_hip_ssd_decode(const OgleDecodeArgs* args, ogle_stream_t stream);
+
+/*
+ * Decode + per-prior softmax-max + score threshold + ordered compaction, in
+ * one launch: decoder.glsl followed by Detector::GenerateBoxInfo
+ * (ogl_runtime/opengl/examples/ssd/detector.cc:184-225), for every image of
+ * the batch.  Outputs per image b, in ascending prior order:
+ *   kept_count_dev[b]
+ *   kept_prior_dev[b*priors + r], kept_class_dev[..], kept_score_dev[..]
+ *   kept_box_dev[(b*priors + r)*4 + 0..3]  scaled xmin,ymin,xmax,ymax (fp32)
+ *   kept_rect_dev[(b*priors + r)*4 + 0..3] integer x,y,width,height
+ *                                          (cv::Rect truncation, detector.cc:211-214)
+ * boxes_dev (batch, priors, 4), if not NULL, also receives every decoded box
+ * (what the reference reads back).  If prediction_dev is NULL, boxes_dev is an
+ * INPUT holding already decoded boxes.  Any kept_* pointer except
+ * kept_count_dev may be NULL.
+ */
+typedef struct OgleDetectArgs {
+  const float* logits_dev;     /* (batch, priors, classes) */
+  const float* prediction_dev; /* (batch, priors, 4) or NULL */
+  const float* anchors_dev;    /* as OgleDecodeArgs */
+  float* boxes_dev;            /* (batch, priors, 4), see above */
+  int32_t batch, priors, classes;
+  int64_t anchors_batch_stride;
+  float variances[4];
+  float score_threshold; /* strict > (detector.cc:209) */
+  float image_width;     /* scale applied to x (detector.cc:201-204) */
+  float image_height;
+  int32_t* kept_count_dev;
+  int32_t* kept_prior_dev;
+  int32_t* kept_class_dev;
+  float* kept_score_dev;
+  float* kept_box_dev;
+  int32_t* kept_rect_dev;
+} OgleDetectArgs;
+
+int32_t ogle_hip_ssd_detect(const OgleDetectArgs* args, ogle_stream_t stream);
+
+/* y[i] = exp(x[i]) exactly as ogle_hip_ssd_detect evaluates it; lets a test
+ * compare the device exponential with the host's on the same inputs. */
+int32_t ogle_hip_expf(const float* x_dev, float* y_dev, int64_t count, ogle_stream_t stream);
+
+#ifdef __cplusplus
+} /* extern "C" */
+#endif
+
+#endif /* OGLE_HIP_H_ */

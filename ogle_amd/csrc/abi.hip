@@ -1,0 +1,301 @@
+// C ABI of the kernel library: argument validation, the kernel registry and the
+// dispatch from op-level entry points to the HIP launchers.
+#include <cstring>
+#include <string>
+
+#include "common.h"
+
+namespace ogle {
+
+static thread_local char g_error[512] = "";
+
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+}
+
+int32_t check_launch(const char* kernel) {
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    set_error("%s: launch failed: %s", kernel, hipGetErrorString(e));
+    return OGLE_ERR_LAUNCH;
+  }
+  return OGLE_OK;
+}
+
+namespace {
+
+// Registry: shader stem -> kernel family.  The flag bits mirror the build
+// options the reference composes (conv2d.cc:54-62).
+enum Family {
+  FAM_CONV = 1, FAM_CONV_DW = 2, FAM_CONV_PW = 3, FAM_CONV_GRP = 4,
+  FAM_POOL = 5, FAM_CONCAT = 6, FAM_DECODER = 7
+};
+enum Flags { FLAG_BIAS = 1, FLAG_CLIP = 2, FLAG_RELU = 4, FLAG_ANY4 = 8 };
+
+struct Entry {
+  const char* name;
+  int family;
+  int base_flags;
+};
+
+const Entry kRegistry[] = {
+    {"conv2d", FAM_CONV, 0},
+    {"conv2d_any4", FAM_CONV, FLAG_ANY4},
+    {"conv2d_dw", FAM_CONV_DW, 0},
+    {"conv2d_dw_any4", FAM_CONV_DW, FLAG_ANY4},
+    {"conv2d_pw", FAM_CONV_PW, 0},
+    {"conv2d_pw_any4", FAM_CONV_PW, FLAG_ANY4},
+    {"conv2d_grp", FAM_CONV_GRP, 0},
+    {"pool", FAM_POOL, 0},
+    {"pool_any4", FAM_POOL, FLAG_ANY4},
+    {"concat_multi", FAM_CONCAT, 0},
+    {"decoder", FAM_DECODER, 0},
+};
+constexpr int kRegistrySize = sizeof(kRegistry) / sizeof(kRegistry[0]);
+
+bool positive(int v) { return v > 0; }
+
+int32_t validate_conv(const OgleConvArgs* a, const char* who) {
+  if (a == nullptr) return fail(OGLE_ERR_INVALID_ARG, "null args");
+  if (!a->input_dev || !a->filter_dev || !a->output_dev) {
+    set_error("%s: null device pointer", who);
+    return OGLE_ERR_INVALID_ARG;
+  }
+  if (!positive(a->n) || !positive(a->in_h) || !positive(a->in_w) || !positive(a->in_c) ||
+      !positive(a->out_c) || !positive(a->kernel_size) || !positive(a->stride) ||
+      a->padding < 0 || !positive(a->dilation) || !positive(a->group)) {
+    set_error("%s: non-positive shape or attribute", who);
+    return OGLE_ERR_INVALID_ARG;
+  }
+  if (a->dtype != OGLE_F32 && a->dtype != OGLE_F16) {
+    set_error("%s: unknown dtype %d", who, a->dtype);
+    return OGLE_ERR_INVALID_ARG;
+  }
+  if (a->act < OGLE_ACT_NONE || a->act > OGLE_ACT_RELU) {
+    set_error("%s: unknown activation %d", who, a->act);
+    return OGLE_ERR_INVALID_ARG;
+  }
+  // Output size rule of Conv2DKernel::InferOutputShape (conv2d.cc:191-193).
+  const int keff = a->kernel_size * a->dilation - a->dilation + 1;
+  const int oh = (a->in_h - keff + 2 * a->padding) / a->stride + 1;
+  const int ow = (a->in_w - keff + 2 * a->padding) / a->stride + 1;
+  if (oh != a->out_h || ow != a->out_w || oh <= 0 || ow <= 0) {
+    set_error("%s: output %dx%d does not follow from input %dx%d k%d s%d p%d d%d (expect %dx%d)",
+              who, a->out_h, a->out_w, a->in_h, a->in_w, a->kernel_size, a->stride, a->padding,
+              a->dilation, oh, ow);
+    return OGLE_ERR_INVALID_ARG;
+  }
+  if (a->in_c % a->group != 0 || a->out_c % a->group != 0) {
+    set_error("%s: channels %d -> %d not divisible by group %d", who, a->in_c, a->out_c, a->group);
+    return OGLE_ERR_INVALID_ARG;
+  }
+  return OGLE_OK;
+}
+
+}  // namespace
+}  // namespace ogle
+
+using namespace ogle;
+
+extern "C" {
+
+int32_t ogle_hip_abi_version(void) { return 100; }
+
+const char* ogle_hip_last_error(void) { return g_error; }
+
+const char* ogle_hip_status_string(int32_t status) {
+  switch (status) {
+    case OGLE_OK: return "ok";
+    case OGLE_ERR_INVALID_ARG: return "invalid argument";
+    case OGLE_ERR_UNSUPPORTED: return "unsupported";
+    case OGLE_ERR_LAUNCH: return "launch failed";
+    case OGLE_ERR_NOT_FOUND: return "not found";
+    case OGLE_ERR_NO_DEVICE: return "no device";
+    default: return "unknown status";
+  }
+}
+
+int32_t ogle_hip_registry_size(void) { return kRegistrySize; }
+
+const char* ogle_hip_registry_name(int32_t index) {
+  if (index < 0 || index >= kRegistrySize) return nullptr;
+  return kRegistry[index].name;
+}
+
+int32_t ogle_hip_registry_lookup(const char* name, const char* options, int32_t* handle) {
+  if (name == nullptr || handle == nullptr) return fail(OGLE_ERR_INVALID_ARG, "null name/handle");
+  for (int i = 0; i < kRegistrySize; ++i) {
+    if (std::strcmp(kRegistry[i].name, name) != 0) continue;
+    int flags = kRegistry[i].base_flags;
+    if (options != nullptr) {
+      if (std::strstr(options, "USE_BIAS")) flags |= FLAG_BIAS;
+      if (std::strstr(options, "USE_CLIP")) flags |= FLAG_CLIP;
+      if (std::strstr(options, "USE_RELU")) flags |= FLAG_RELU;
+    }
+    *handle = (kRegistry[i].family << 8) | flags;
+    return OGLE_OK;
+  }
+  set_error("registry: no kernel named '%s'", name);
+  return OGLE_ERR_NOT_FOUND;
+}
+
+int32_t ogle_hip_sync(ogle_stream_t stream) {
+  const hipError_t e = hipStreamSynchronize(as_stream(stream));
+  if (e != hipSuccess) {
+    set_error("sync: %s", hipGetErrorString(e));
+    return OGLE_ERR_LAUNCH;
+  }
+  return OGLE_OK;
+}
+
+int64_t ogle_hip_packed_filter_elems(int32_t layout, int32_t o, int32_t i, int32_t kh,
+                                     int32_t kw) {
+  if (o <= 0 || i <= 0 || kh <= 0 || kw <= 0) return -1;
+  if (layout == OGLE_FILTER_OHWI) return (int64_t)o * i * kh * kw;
+  if (layout == OGLE_FILTER_HWC) return i == 1 ? (int64_t)o * kh * kw : -1;
+  return -1;
+}
+
+int32_t ogle_hip_pack_filter(const float* oihw_dev, void* packed_dev, int32_t layout,
+                             int32_t dtype, int32_t o, int32_t i, int32_t kh, int32_t kw,
+                             ogle_stream_t stream) {
+  if (!oihw_dev || !packed_dev) return fail(OGLE_ERR_INVALID_ARG, "pack_filter: null pointer");
+  if (ogle_hip_packed_filter_elems(layout, o, i, kh, kw) < 0)
+    return fail(OGLE_ERR_INVALID_ARG, "pack_filter: bad layout or shape");
+  if (dtype != OGLE_F32 && dtype != OGLE_F16)
+    return fail(OGLE_ERR_INVALID_ARG, "pack_filter: unknown dtype");
+  return launch_pack_filter(oihw_dev, packed_dev, layout, dtype, o, i, kh, kw, as_stream(stream));
+}
+
+int32_t ogle_hip_convert(const void* src_dev, int32_t src_dtype, void* dst_dev,
+                         int32_t dst_dtype, int64_t count, ogle_stream_t stream) {
+  if (count < 0 || (count > 0 && (!src_dev || !dst_dev)))
+    return fail(OGLE_ERR_INVALID_ARG, "convert: null pointer or negative count");
+  if ((src_dtype != OGLE_F32 && src_dtype != OGLE_F16) ||
+      (dst_dtype != OGLE_F32 && dst_dtype != OGLE_F16))
+    return fail(OGLE_ERR_INVALID_ARG, "convert: unknown dtype");
+  return launch_convert(src_dev, src_dtype, dst_dev, dst_dtype, count, as_stream(stream));
+}
+
+int32_t ogle_hip_conv2d(const OgleConvArgs* a, ogle_stream_t stream) {
+  int32_t st = validate_conv(a, "conv2d");
+  if (st != OGLE_OK) return st;
+  if (a->group == 1) {
+    st = launch_conv_igemm(*a, as_stream(stream));
+    if (st != OGLE_ERR_UNSUPPORTED) return st;
+  }
+  return launch_conv_direct(*a, as_stream(stream));
+}
+
+int32_t ogle_hip_dwconv2d(const OgleConvArgs* a, ogle_stream_t stream) {
+  int32_t st = validate_conv(a, "dwconv2d");
+  if (st != OGLE_OK) return st;
+  // conv2d.cc:27-29,41: depthwise means group == C_in (== C_out).
+  if (a->group != a->in_c || a->out_c != a->in_c) {
+    set_error("dwconv2d: group %d must equal in_c %d and out_c %d", a->group, a->in_c, a->out_c);
+    return OGLE_ERR_INVALID_ARG;
+  }
+  return launch_conv_dw(*a, as_stream(stream));
+}
+
+int32_t ogle_hip_pwconv_gemm(const OgleConvArgs* a, ogle_stream_t stream) {
+  int32_t st = validate_conv(a, "pwconv_gemm");
+  if (st != OGLE_OK) return st;
+  // conv2d.cc:37: the pointwise shader is chosen only for 1x1, g1, d1, s1, p0.
+  if (a->kernel_size != 1 || a->group != 1 || a->dilation != 1 || a->stride != 1 ||
+      a->padding != 0) {
+    set_error("pwconv_gemm: needs kernel 1, group 1, dilation 1, stride 1, padding 0");
+    return OGLE_ERR_INVALID_ARG;
+  }
+  st = launch_conv_igemm(*a, as_stream(stream));
+  if (st != OGLE_ERR_UNSUPPORTED) return st;
+  return launch_conv_direct(*a, as_stream(stream));
+}
+
+int32_t ogle_hip_pool2d(const OglePoolArgs* a, ogle_stream_t stream) {
+  if (a == nullptr) return fail(OGLE_ERR_INVALID_ARG, "pool2d: null args");
+  if (!a->input_dev || !a->output_dev) return fail(OGLE_ERR_INVALID_ARG, "pool2d: null pointer");
+  if (!positive(a->n) || !positive(a->in_h) || !positive(a->in_w) || !positive(a->c) ||
+      !positive(a->kernel_size) || !positive(a->stride) || a->padding < 0)
+    return fail(OGLE_ERR_INVALID_ARG, "pool2d: non-positive shape or attribute");
+  if (a->pool_type < OGLE_POOL_MAX || a->pool_type > OGLE_POOL_GLOBAL_AVG)
+    return fail(OGLE_ERR_INVALID_ARG, "pool2d: unknown pool_type");
+  if (a->dtype != OGLE_F32 && a->dtype != OGLE_F16)
+    return fail(OGLE_ERR_INVALID_ARG, "pool2d: unknown dtype");
+  if (a->pool_type == OGLE_POOL_GLOBAL_AVG &&
+      (a->in_h != a->in_w || a->kernel_size != a->in_h || a->stride != 1 || a->padding != 0))
+    return fail(OGLE_ERR_INVALID_ARG,
+                "pool2d: global average needs a square input, kernel = H, stride 1, padding 0");
+  // pool.cc:94-96
+  const int oh = (a->in_h - a->kernel_size + 2 * a->padding) / a->stride + 1;
+  const int ow = (a->in_w - a->kernel_size + 2 * a->padding) / a->stride + 1;
+  if (oh != a->out_h || ow != a->out_w || oh <= 0 || ow <= 0) {
+    set_error("pool2d: output %dx%d does not follow from the input (expect %dx%d)", a->out_h,
+              a->out_w, oh, ow);
+    return OGLE_ERR_INVALID_ARG;
+  }
+  return launch_pool(*a, as_stream(stream));
+}
+
+int32_t ogle_hip_concat(const OgleConcatArgs* a, ogle_stream_t stream) {
+  if (a == nullptr) return fail(OGLE_ERR_INVALID_ARG, "concat: null args");
+  if (a->n_inputs < 1 || a->n_inputs > OGLE_CONCAT_MAX_INPUTS) {
+    set_error("concat: %d inputs (1..%d allowed)", a->n_inputs, OGLE_CONCAT_MAX_INPUTS);
+    return OGLE_ERR_INVALID_ARG;
+  }
+  if (a->outer < 0 || a->inner < 0) return fail(OGLE_ERR_INVALID_ARG, "concat: negative extent");
+  if (a->dtype != OGLE_F32 && a->dtype != OGLE_F16)
+    return fail(OGLE_ERR_INVALID_ARG, "concat: unknown dtype");
+  int64_t total = 0;
+  for (int i = 0; i < a->n_inputs; ++i) {
+    if (a->axis_len[i] < 0) return fail(OGLE_ERR_INVALID_ARG, "concat: negative axis length");
+    if (a->axis_len[i] > 0 && a->inputs_dev[i] == nullptr && a->outer * a->inner > 0)
+      return fail(OGLE_ERR_INVALID_ARG, "concat: null input");
+    total += a->axis_len[i];
+  }
+  if (total * a->outer * a->inner > 0 && a->output_dev == nullptr)
+    return fail(OGLE_ERR_INVALID_ARG, "concat: null output");
+  return launch_concat(*a, as_stream(stream));
+}
+
+int32_t ogle_hip_ssd_decode(const OgleDecodeArgs* a, ogle_stream_t stream) {
+  if (a == nullptr) return fail(OGLE_ERR_INVALID_ARG, "ssd_decode: null args");
+  if (a->batch < 0 || a->priors < 0) return fail(OGLE_ERR_INVALID_ARG, "ssd_decode: negative size");
+  if ((long)a->batch * a->priors > 0 && (!a->prediction_dev || !a->anchors_dev || !a->boxes_dev))
+    return fail(OGLE_ERR_INVALID_ARG, "ssd_decode: null pointer");
+  // decoder.cc:82-85: anchors are either shared or one set per image.
+  if (a->anchors_batch_stride != 0 && a->anchors_batch_stride != (int64_t)a->priors * 4)
+    return fail(OGLE_ERR_INVALID_ARG, "ssd_decode: anchors_batch_stride must be 0 or priors*4");
+  return launch_decode(*a, as_stream(stream));
+}
+
+int32_t ogle_hip_ssd_detect(const OgleDetectArgs* a, ogle_stream_t stream) {
+  if (a == nullptr) return fail(OGLE_ERR_INVALID_ARG, "ssd_detect: null args");
+  if (a->batch < 0 || a->priors < 0 || a->classes < 1)
+    return fail(OGLE_ERR_INVALID_ARG, "ssd_detect: bad size");
+  if (a->classes > 40)  // the logit slab of 256 priors must fit LDS
+    return fail(OGLE_ERR_UNSUPPORTED, "ssd_detect: more than 40 classes");
+  if (!a->kept_count_dev && a->batch > 0)
+    return fail(OGLE_ERR_INVALID_ARG, "ssd_detect: kept_count_dev is required");
+  if ((long)a->batch * a->priors > 0) {
+    if (!a->logits_dev) return fail(OGLE_ERR_INVALID_ARG, "ssd_detect: null logits");
+    if (a->prediction_dev && !a->anchors_dev)
+      return fail(OGLE_ERR_INVALID_ARG, "ssd_detect: prediction without anchors");
+    if (!a->prediction_dev && !a->boxes_dev)
+      return fail(OGLE_ERR_INVALID_ARG, "ssd_detect: neither prediction nor decoded boxes");
+  }
+  if (a->anchors_batch_stride != 0 && a->anchors_batch_stride != (int64_t)a->priors * 4)
+    return fail(OGLE_ERR_INVALID_ARG, "ssd_detect: anchors_batch_stride must be 0 or priors*4");
+  return launch_detect(*a, as_stream(stream));
+}
+
+int32_t ogle_hip_expf(const float* x_dev, float* y_dev, int64_t count, ogle_stream_t stream) {
+  if (count < 0 || (count > 0 && (!x_dev || !y_dev)))
+    return fail(OGLE_ERR_INVALID_ARG, "expf: null pointer or negative count");
+  return launch_expf(x_dev, y_dev, count, as_stream(stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,96 @@
+// Shared device/host helpers for the gfx950 kernels.
+#ifndef OGLE_CSRC_COMMON_H_
+#define OGLE_CSRC_COMMON_H_
+
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+
+#include "ogle_hip.h"
+
+namespace ogle {
+
+// Thread-local message for ogle_hip_last_error().
+void set_error(const char* fmt, ...);
+
+inline int32_t fail(int32_t status, const char* what) {
+  set_error("%s", what);
+  return status;
+}
+
+// Reports the launch status of the kernel just enqueued.
+int32_t check_launch(const char* kernel);
+
+inline hipStream_t as_stream(ogle_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+
+inline int ceil_div(long a, long b) { return static_cast<int>((a + b - 1) / b); }
+
+// Fused activation with the variant rules of the reference's shaders
+// (conv2d.glsl:82-90, conv2d_pw.glsl:82-90, conv2d_any4.glsl:89-94).  The
+// bounds are resolved on the host into (lo, hi) plus two flags so that the
+// device code is variant free.
+struct Epilogue {
+  float lo;
+  float hi;
+  int use_lo;
+  int use_hi;
+};
+
+inline Epilogue make_epilogue(int act, float minv, float maxv, int variant) {
+  Epilogue e{0.f, 0.f, 0, 0};
+  if (act == OGLE_ACT_CLIP) {
+    e.lo = (variant == OGLE_VARIANT_PW) ? 0.f : minv;
+    e.hi = maxv;
+    e.use_lo = 1;
+    e.use_hi = 1;
+  } else if (act == OGLE_ACT_RELU) {
+    e.lo = (variant == OGLE_VARIANT_ANY4) ? minv : 0.f;
+    e.use_lo = 1;
+  }
+  return e;
+}
+
+__device__ __forceinline__ float apply_epilogue(float v, const Epilogue& e) {
+  if (e.use_lo) v = v < e.lo ? e.lo : v;
+  if (e.use_hi) v = v > e.hi ? e.hi : v;
+  return v;
+}
+
+// Storage <-> fp32 conversions.
+__device__ __forceinline__ float to_f32(float v) { return v; }
+__device__ __forceinline__ float to_f32(__half v) { return __half2float(v); }
+template <typename T>
+__device__ __forceinline__ T from_f32(float v);
+template <>
+__device__ __forceinline__ float from_f32<float>(float v) { return v; }
+template <>
+__device__ __forceinline__ __half from_f32<__half>(float v) { return __float2half_rn(v); }
+
+// Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.
+// Remaps the linear workgroup id so that consecutive logical ids land on the
+// same XCD, keeping tiles that share operands in one L2.
+__device__ __forceinline__ int xcd_swizzle(int pid, int grid) {
+  constexpr int kXcds = 8;
+  if (grid % kXcds != 0) return pid;
+  return (pid % kXcds) * (grid / kXcds) + pid / kXcds;
+}
+
+// Launchers implemented in the .hip files (host side).
+int32_t launch_conv_igemm(const OgleConvArgs& a, hipStream_t s);   // returns OGLE_ERR_UNSUPPORTED if shape not eligible
+int32_t launch_conv_direct(const OgleConvArgs& a, hipStream_t s);
+int32_t launch_conv_dw(const OgleConvArgs& a, hipStream_t s);
+int32_t launch_pool(const OglePoolArgs& a, hipStream_t s);
+int32_t launch_concat(const OgleConcatArgs& a, hipStream_t s);
+int32_t launch_decode(const OgleDecodeArgs& a, hipStream_t s);
+int32_t launch_detect(const OgleDetectArgs& a, hipStream_t s);
+int32_t launch_expf(const float* x, float* y, int64_t n, hipStream_t s);
+int32_t launch_pack_filter(const float* src, void* dst, int layout, int dtype, int o, int i,
+                           int kh, int kw, hipStream_t s);
+int32_t launch_convert(const void* src, int sdt, void* dst, int ddt, int64_t n, hipStream_t s);
+
+}  // namespace ogle
+
+#endif  // OGLE_CSRC_COMMON_H_

@@ -1,0 +1,290 @@
+// Dense convolution (group 1) as an implicit GEMM on the MFMA units.
+//
+//   Y[m, o] = act( bias[o] + sum_{tap, c} X[row(m) + tap, c] * W[o, tap, c] )
+//
+// with m = (image, oy, ox) flattened, K = taps * C.  Both operands are
+// K-contiguous in memory: X is NHWC (a pixel's channels are contiguous) and W is
+// packed OHWI (an output channel's taps*channels are contiguous), so both tiles
+// are fetched as 16-byte vectors along K and the pointwise 1x1 convolution is the
+// special case with one tap and no gather (conv2d_pw.glsl:35-91); the KxK form
+// follows conv2d.glsl:29-92 (taps outside the image contribute zero).
+//
+// Tiling.  A workgroup of 4 waves (256 threads) owns a BM x BN output tile and
+// walks K in slabs of ROWB bytes per row.  Slabs are staged global -> registers
+// -> LDS (double buffered, one barrier per slab) with the next slab's global
+// loads in flight while the current one is multiplied.  LDS rows are padded by
+// 16 bytes so the 16-byte-per-lane operand reads are bank-conflict free.
+//
+// MFMA mapping (64-wide waves).  fp32 uses v_mfma_f32_32x32x2_f32: lane l
+// supplies A[l%32][l/32] and B[l/32][l%32].  Since the contraction sums over k
+// in any order, a lane reads four consecutive k of its row with one 16-byte LDS
+// read (lanes 0-31 take k 0..3 of an 8-wide group, lanes 32-63 take k 4..7) and
+// issues four MFMAs, one per element.  fp16 storage uses
+// v_mfma_f32_32x32x16_f16: a lane's 16 bytes are the 8 halves the instruction
+// wants (k = 8*(l/32)..+7).  Accumulation is fp32 in both cases.
+//
+// Result layout of a 32x32 block: register r of lane l holds
+// row 8*(r/4) + 4*(l/32) + r%4, column l%32, so a store instruction writes two
+// 128-byte runs of one output pixel's channels.
+#include "common.h"
+
+namespace ogle {
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
+
+struct ConvGeom {
+  int n, h, w, c;
+  int oh, ow, o;
+  int k, stride, pad, dil;
+  int m_total;   // n*oh*ow
+  int cchunks;   // K slabs per tap
+  int ktiles;    // taps * cchunks
+};
+
+template <typename T>
+struct Mma;
+template <>
+struct Mma<float> {
+  __device__ static __forceinline__ void run(const uint4& a, const uint4& b, floatx16& acc) {
+    const float* af = reinterpret_cast<const float*>(&a);
+    const float* bf = reinterpret_cast<const float*>(&b);
+#pragma unroll
+    for (int s = 0; s < 4; ++s)
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af[s], bf[s], acc, 0, 0, 0);
+  }
+};
+template <>
+struct Mma<__half> {
+  __device__ static __forceinline__ void run(const uint4& a, const uint4& b, floatx16& acc) {
+    const halfx8 ah = *reinterpret_cast<const halfx8*>(&a);
+    const halfx8 bh = *reinterpret_cast<const halfx8*>(&b);
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bh, acc, 0, 0, 0);
+  }
+};
+
+template <typename T, int BM, int BN, int WM, int WN, int ROWB, bool PW>
+__global__ __launch_bounds__(256) void conv_igemm_kernel(
+    ConvGeom g, const T* __restrict__ x, const T* __restrict__ w,
+    const float* __restrict__ bias, T* __restrict__ y, Epilogue ep, int tiles_n) {
+  static_assert(WM * WN == 4, "four waves per workgroup");
+  constexpr int WTM = BM / WM, WTN = BN / WN;
+  constexpr int TM = WTM / 32, TN = WTN / 32;
+  static_assert(TM >= 1 && TN >= 1, "wave tile at least 32x32");
+  constexpr int VPR = ROWB / 16;       // 16-byte vectors per row per slab
+  constexpr int RPP = 256 / VPR;       // rows one pass of the workgroup loads
+  constexpr int AP = (BM + RPP - 1) / RPP, BP = (BN + RPP - 1) / RPP;
+  constexpr bool A_PART = BM % RPP != 0, B_PART = BN % RPP != 0;  // last pass partly idle
+  constexpr int LROW = ROWB + 16;      // padded LDS row, bytes
+  constexpr int VE = 16 / (int)sizeof(T);    // elements per vector
+  constexpr int EPR = ROWB / (int)sizeof(T); // elements per row per slab
+  constexpr int CHUNKS = ROWB / 32;
+
+  __shared__ __attribute__((aligned(16))) unsigned char lds[2 * (BM + BN) * LROW];
+  constexpr int STAGE = (BM + BN) * LROW;  // one buffer: A rows then B rows
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wave_m = wave / WN, wave_n = wave % WN;
+
+  const int pid = xcd_swizzle(blockIdx.x, gridDim.x);
+  const int tile_n = pid % tiles_n;
+  const int tile_m = pid / tiles_n;
+  const int m0 = tile_m * BM;
+  const int n0 = tile_n * BN;
+
+  const int vcol = tid % VPR;   // which 16-byte vector of the slab row
+  const int vrow = tid / VPR;   // row within a pass
+
+  // Per-pass source rows of this thread.
+  long a_base[AP];   // PW: element offset of the row; KxK: image base offset
+  int a_iy[AP], a_ix[AP];
+  bool a_ok[AP];
+#pragma unroll
+  for (int p = 0; p < AP; ++p) {
+    const int m = m0 + p * RPP + vrow;
+    a_ok[p] = m < g.m_total && (!A_PART || p * RPP + vrow < BM);
+    if (PW) {
+      a_base[p] = (long)m * g.c;
+      a_iy[p] = 0;
+      a_ix[p] = 0;
+    } else {
+      const int ox = m % g.ow;
+      const int t = m / g.ow;
+      const int oy = t % g.oh;
+      const int b = t / g.oh;
+      a_base[p] = (long)b * g.h * g.w * g.c;
+      a_iy[p] = oy * g.stride - g.pad;
+      a_ix[p] = ox * g.stride - g.pad;
+    }
+  }
+  const long ktot = (long)g.k * g.k * g.c;
+  long b_base[BP];
+  bool b_ok[BP];
+#pragma unroll
+  for (int p = 0; p < BP; ++p) {
+    const int o = n0 + p * RPP + vrow;
+    b_ok[p] = o < g.o && (!B_PART || p * RPP + vrow < BN);
+    b_base[p] = (long)o * ktot;
+  }
+
+  uint4 ra[AP], rb[BP];
+  const uint4 zero = make_uint4(0, 0, 0, 0);
+
+  auto load_slab = [&](int kt) {
+    int tap = 0, cc = kt;
+    if (!PW) {
+      tap = kt / g.cchunks;
+      cc = kt - tap * g.cchunks;
+    }
+    const int c0 = cc * EPR + vcol * VE;
+    const bool c_ok = c0 < g.c;
+    int dy = 0, dx = 0;
+    if (!PW) {
+      const int ky = tap / g.k;
+      dy = ky * g.dil;
+      dx = (tap - ky * g.k) * g.dil;
+    }
+#pragma unroll
+    for (int p = 0; p < AP; ++p) {
+      bool ok = a_ok[p] && c_ok;
+      long off;
+      if (PW) {
+        off = a_base[p] + c0;
+      } else {
+        const int iy = a_iy[p] + dy, ix = a_ix[p] + dx;
+        ok = ok && iy >= 0 && iy < g.h && ix >= 0 && ix < g.w;
+        off = a_base[p] + ((long)iy * g.w + ix) * g.c + c0;
+      }
+      ra[p] = ok ? *reinterpret_cast<const uint4*>(x + off) : zero;
+    }
+#pragma unroll
+    for (int p = 0; p < BP; ++p) {
+      const bool ok = b_ok[p] && c_ok;
+      rb[p] = ok ? *reinterpret_cast<const uint4*>(w + b_base[p] + (long)tap * g.c + c0) : zero;
+    }
+  };
+  auto store_slab = [&](int buf) {
+#pragma unroll
+    for (int p = 0; p < AP; ++p)
+      if (!A_PART || p * RPP + vrow < BM)
+        *reinterpret_cast<uint4*>(lds + buf * STAGE + (p * RPP + vrow) * LROW + vcol * 16) = ra[p];
+#pragma unroll
+    for (int p = 0; p < BP; ++p)
+      if (!B_PART || p * RPP + vrow < BN)
+        *reinterpret_cast<uint4*>(lds + buf * STAGE + (BM + p * RPP + vrow) * LROW + vcol * 16) = rb[p];
+  };
+
+  floatx16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  const int l32 = lane & 31;
+  const int lh = lane >> 5;
+
+  load_slab(0);
+  store_slab(0);
+  __syncthreads();
+  for (int kt = 0; kt < g.ktiles; ++kt) {
+    const int buf = kt & 1;
+    const bool more = kt + 1 < g.ktiles;
+    if (more) load_slab(kt + 1);
+    const unsigned char* pa = lds + buf * STAGE + (wave_m * WTM + l32) * LROW + lh * 16;
+    const unsigned char* pb = lds + buf * STAGE + (BM + wave_n * WTN + l32) * LROW + lh * 16;
+#pragma unroll
+    for (int ch = 0; ch < CHUNKS; ++ch) {
+      uint4 av[TM], bv[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        av[i] = *reinterpret_cast<const uint4*>(pa + i * 32 * LROW + ch * 32);
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        bv[j] = *reinterpret_cast<const uint4*>(pb + j * 32 * LROW + ch * 32);
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) Mma<T>::run(av[i], bv[j], acc[i][j]);
+    }
+    if (more) store_slab(buf ^ 1);
+    __syncthreads();
+  }
+
+  // Epilogue: bias, activation, store.
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int col = n0 + wave_n * WTN + j * 32 + l32;
+    if (col >= g.o) continue;
+    const float bv = bias != nullptr ? bias[col] : 0.f;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int rbase = m0 + wave_m * WTM + i * 32 + lh * 4;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = rbase + (r >> 2) * 8 + (r & 3);
+        if (row < g.m_total)
+          y[(long)row * g.o + col] = from_f32<T>(apply_epilogue(acc[i][j][r] + bv, ep));
+      }
+    }
+  }
+}
+
+template <typename T, int BM, int BN, int WM, int WN, int ROWB, bool PW>
+int32_t launch_cfg(const ConvGeom& g0, const OgleConvArgs& a, hipStream_t s) {
+  ConvGeom g = g0;
+  constexpr int EPR = ROWB / (int)sizeof(T);
+  g.cchunks = (g.c + EPR - 1) / EPR;
+  g.ktiles = g.k * g.k * g.cchunks;
+  const int tiles_m = (g.m_total + BM - 1) / BM;
+  const int tiles_n = (g.o + BN - 1) / BN;
+  const Epilogue ep = make_epilogue(a.act, a.min_value, a.max_value, a.act_variant);
+  hipLaunchKernelGGL((conv_igemm_kernel<T, BM, BN, WM, WN, ROWB, PW>),
+                     dim3((unsigned)(tiles_m * tiles_n)), dim3(256), 0, s, g,
+                     static_cast<const T*>(a.input_dev), static_cast<const T*>(a.filter_dev),
+                     a.bias_dev, static_cast<T*>(a.output_dev), ep, tiles_n);
+  return check_launch("conv_igemm");
+}
+
+template <typename T, int ROWB, bool PW>
+int32_t pick_tile(const ConvGeom& g, const OgleConvArgs& a, hipStream_t s) {
+  const long m = g.m_total;
+  auto tiles = [&](int bm, int bn) { return ((m + bm - 1) / bm) * ((g.o + bn - 1) / bn); };
+  constexpr long kFill = 256;  // compute units
+  if (g.o <= 32) return launch_cfg<T, 128, 32, 4, 1, ROWB, PW>(g, a, s);
+  if (g.o <= 64) {
+    if (tiles(128, 64) >= 2 * kFill) return launch_cfg<T, 128, 64, 2, 2, ROWB, PW>(g, a, s);
+    return launch_cfg<T, 64, 64, 2, 2, ROWB, PW>(g, a, s);
+  }
+  if (tiles(128, 128) >= 2 * kFill) return launch_cfg<T, 128, 128, 2, 2, ROWB, PW>(g, a, s);
+  if (tiles(128, 64) >= kFill) return launch_cfg<T, 128, 64, 2, 2, ROWB, PW>(g, a, s);
+  return launch_cfg<T, 64, 64, 2, 2, ROWB, PW>(g, a, s);
+}
+
+}  // namespace
+
+int32_t launch_conv_igemm(const OgleConvArgs& a, hipStream_t s) {
+  if (a.group != 1) return OGLE_ERR_UNSUPPORTED;
+  const int ve = a.dtype == OGLE_F16 ? 8 : 4;
+  if (a.in_c % ve != 0) return OGLE_ERR_UNSUPPORTED;
+  if ((long)a.kernel_size * a.kernel_size * a.in_c < 32) return OGLE_ERR_UNSUPPORTED;
+  const long m = (long)a.n * a.out_h * a.out_w;
+  if (m <= 0 || m > 0x7fffffffL) return OGLE_ERR_UNSUPPORTED;
+  ConvGeom g{};
+  g.n = a.n; g.h = a.in_h; g.w = a.in_w; g.c = a.in_c;
+  g.oh = a.out_h; g.ow = a.out_w; g.o = a.out_c;
+  g.k = a.kernel_size; g.stride = a.stride; g.pad = a.padding; g.dil = a.dilation;
+  g.m_total = (int)m;
+  const bool pw = a.kernel_size == 1 && a.stride == 1 && a.padding == 0;
+  if (a.dtype == OGLE_F16) {
+    return pw ? pick_tile<__half, 128, true>(g, a, s) : pick_tile<__half, 128, false>(g, a, s);
+  }
+  return pw ? pick_tile<float, 64, true>(g, a, s) : pick_tile<float, 64, false>(g, a, s);
+}
+
+}  // namespace ogle

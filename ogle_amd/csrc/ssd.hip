@@ -1,0 +1,196 @@
+// SSD box decoder and score filter.
+//
+// ssd_decode_kernel restates decoder.glsl:13-28 (center-size -> corners with
+// variances).  ssd_detect_kernel fuses it with the per-prior work of
+// Detector::GenerateBoxInfo (examples/ssd/detector.cc:184-225): sequential fp32
+// softmax denominator over classes 0..C-1, strict-greater maximum over classes
+// 1..C-1, p = e_max / sum, keep iff p > threshold, scale to pixels, truncate to
+// an integer rectangle; kept priors are written compacted in ascending prior
+// order (the order the host loop produces them in).
+//
+// Every floating-point operation here is a separate IEEE binary32 operation in
+// the host code's order: contraction into FMA is disabled for this file, and
+// exp is evaluated in binary64 and rounded once to binary32, i.e. a correctly
+// rounded expf, which is what the host's libm returns in all but a vanishing
+// fraction of inputs.  That keeps kept indices and class ids equal to the host
+// result bit for bit.
+#pragma clang fp contract(off)
+#include "common.h"
+
+namespace ogle {
+namespace {
+
+__device__ __forceinline__ float exp_cr(float v) { return (float)exp((double)v); }
+
+__device__ __forceinline__ float4 decode_one(const float4 p, const float4 a, const float v0,
+                                             const float v1, const float v2, const float v3) {
+  const float ycenter = p.y * v1 * a.w + a.y;
+  const float xcenter = p.x * v0 * a.z + a.x;
+  const float hh = exp_cr(p.w * v3) * a.w;
+  const float ww = exp_cr(p.z * v2) * a.z;
+  // The host narrows (double)center -/+ (double)size*0.5 to float.
+  float4 o;
+  o.y = (float)((double)ycenter - (double)hh * 0.5);
+  o.x = (float)((double)xcenter - (double)ww * 0.5);
+  o.w = (float)((double)ycenter + (double)hh * 0.5);
+  o.z = (float)((double)xcenter + (double)ww * 0.5);
+  return o;
+}
+
+__global__ __launch_bounds__(256) void ssd_decode_kernel(const float4* __restrict__ pred,
+                                                         const float4* __restrict__ anchors,
+                                                         float4* __restrict__ out, int batch,
+                                                         int priors, long anchor_stride_vec,
+                                                         float v0, float v1, float v2, float v3) {
+  const long total = (long)batch * priors;
+  for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (long)gridDim.x * blockDim.x) {
+    const int b = (int)(idx / priors);
+    const int i = (int)(idx - (long)b * priors);
+    out[idx] = decode_one(pred[idx], anchors[b * anchor_stride_vec + i], v0, v1, v2, v3);
+  }
+}
+
+__global__ __launch_bounds__(256) void expf_kernel(const float* __restrict__ x,
+                                                   float* __restrict__ y, long n) {
+  for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < n;
+       idx += (long)gridDim.x * blockDim.x)
+    y[idx] = exp_cr(x[idx]);
+}
+
+struct DetectParams {
+  const float* logits;
+  const float4* pred;
+  const float4* anchors;
+  float4* boxes;
+  int batch, priors, classes;
+  long anchor_stride_vec;
+  float v0, v1, v2, v3;
+  float threshold, image_w, image_h;
+  int32_t* kept_count;
+  int32_t* kept_prior;
+  int32_t* kept_class;
+  float* kept_score;
+  float4* kept_box;
+  int4* kept_rect;
+};
+
+// One workgroup per image walks the priors in slabs of 256.  A slab's logits
+// (256 x classes floats, contiguous) are staged into LDS with coalesced loads;
+// each thread then scores one prior from LDS.  Kept flags are compacted with a
+// wave ballot + popcount and a 4-entry cross-wave prefix, so the output order is
+// the prior order.
+__global__ __launch_bounds__(256) void ssd_detect_kernel(DetectParams p) {
+  extern __shared__ float slab[];  // 256 * classes
+  __shared__ int wave_count[4];
+  __shared__ int base_shared;
+  const int b = blockIdx.x;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const float* logits = p.logits + (long)b * p.priors * p.classes;
+  int base = 0;
+  for (int start = 0; start < p.priors; start += 256) {
+    const int rows = min(256, p.priors - start);
+    const int count = rows * p.classes;
+    const float* src = logits + (long)start * p.classes;
+    for (int i = tid; i < count; i += 256) slab[i] = src[i];
+    __syncthreads();
+
+    const int prior = start + tid;
+    bool keep = false;
+    int max_id = 0;
+    float max_prob = 0.f;
+    float4 box = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (tid < rows) {
+      const float* l = slab + tid * p.classes;
+      float total_sum = exp_cr(l[0]);
+      for (int j = 1; j < p.classes; ++j) {
+        const float e = exp_cr(l[j]);
+        total_sum += e;
+        if (max_prob < e) {
+          max_prob = e;
+          max_id = j;
+        }
+      }
+      const long at = (long)b * p.priors + prior;
+      if (p.pred != nullptr) {
+        box = decode_one(p.pred[at], p.anchors[b * p.anchor_stride_vec + prior], p.v0, p.v1,
+                         p.v2, p.v3);
+        if (p.boxes != nullptr) p.boxes[at] = box;
+      } else {
+        box = p.boxes[at];
+      }
+      max_prob = max_prob / total_sum;
+      keep = max_prob > p.threshold;
+    }
+    const unsigned long long ballot = __ballot(keep);
+    const int before = __popcll(ballot & ((1ull << lane) - 1ull));
+    if (lane == 0) wave_count[wave] = __popcll(ballot);
+    __syncthreads();
+    int wave_base = 0;
+    for (int wv = 0; wv < wave; ++wv) wave_base += wave_count[wv];
+    if (keep) {
+      const long slot = (long)b * p.priors + base + wave_base + before;
+      const float xmin = box.x * p.image_w;
+      const float ymin = box.y * p.image_h;
+      const float xmax = box.z * p.image_w;
+      const float ymax = box.w * p.image_h;
+      if (p.kept_prior) p.kept_prior[slot] = prior;
+      if (p.kept_class) p.kept_class[slot] = max_id;
+      if (p.kept_score) p.kept_score[slot] = max_prob;
+      if (p.kept_box) p.kept_box[slot] = make_float4(xmin, ymin, xmax, ymax);
+      if (p.kept_rect)
+        p.kept_rect[slot] = make_int4((int)xmin, (int)ymin, (int)(xmax - xmin), (int)(ymax - ymin));
+    }
+    if (tid == 0) base_shared = base + wave_count[0] + wave_count[1] + wave_count[2] + wave_count[3];
+    __syncthreads();
+    base = base_shared;
+  }
+  if (tid == 0) p.kept_count[b] = base;
+}
+
+}  // namespace
+
+int32_t launch_decode(const OgleDecodeArgs& a, hipStream_t s) {
+  const long total = (long)a.batch * a.priors;
+  if (total == 0) return OGLE_OK;
+  long blocks = (total + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  hipLaunchKernelGGL(ssd_decode_kernel, dim3((unsigned)blocks), dim3(256), 0, s,
+                     reinterpret_cast<const float4*>(a.prediction_dev),
+                     reinterpret_cast<const float4*>(a.anchors_dev),
+                     reinterpret_cast<float4*>(a.boxes_dev), a.batch, a.priors,
+                     (long)(a.anchors_batch_stride / 4), a.variances[0], a.variances[1],
+                     a.variances[2], a.variances[3]);
+  return check_launch("ssd_decode_kernel");
+}
+
+int32_t launch_detect(const OgleDetectArgs& a, hipStream_t s) {
+  if (a.batch == 0) return OGLE_OK;
+  DetectParams p{};
+  p.logits = a.logits_dev;
+  p.pred = reinterpret_cast<const float4*>(a.prediction_dev);
+  p.anchors = reinterpret_cast<const float4*>(a.anchors_dev);
+  p.boxes = reinterpret_cast<float4*>(a.boxes_dev);
+  p.batch = a.batch; p.priors = a.priors; p.classes = a.classes;
+  p.anchor_stride_vec = (long)(a.anchors_batch_stride / 4);
+  p.v0 = a.variances[0]; p.v1 = a.variances[1]; p.v2 = a.variances[2]; p.v3 = a.variances[3];
+  p.threshold = a.score_threshold; p.image_w = a.image_width; p.image_h = a.image_height;
+  p.kept_count = a.kept_count_dev; p.kept_prior = a.kept_prior_dev;
+  p.kept_class = a.kept_class_dev; p.kept_score = a.kept_score_dev;
+  p.kept_box = reinterpret_cast<float4*>(a.kept_box_dev);
+  p.kept_rect = reinterpret_cast<int4*>(a.kept_rect_dev);
+  const size_t lds = sizeof(float) * 256 * (size_t)a.classes;
+  hipLaunchKernelGGL(ssd_detect_kernel, dim3((unsigned)a.batch), dim3(256), lds, s, p);
+  return check_launch("ssd_detect_kernel");
+}
+
+int32_t launch_expf(const float* x, float* y, int64_t n, hipStream_t s) {
+  if (n == 0) return OGLE_OK;
+  long blocks = (n + 255) / 256;
+  if (blocks > 8192) blocks = 8192;
+  hipLaunchKernelGGL(expf_kernel, dim3((unsigned)blocks), dim3(256), 0, s, x, y, (long)n);
+  return check_launch("expf_kernel");
+}
+
+}  // namespace ogle

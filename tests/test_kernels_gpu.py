@@ -1,0 +1,369 @@
+"""GPU parity tests: every kernel is called through the C ABI (include/ogle_hip.h)
+on seeded inputs and compared with the CPU oracle.
+
+Tolerances (BASELINE targets): fp32 1e-4, fp16 storage 5e-3, both measured
+against the accumulated magnitude sum|x||w| (see util.assert_conv_close); pooling,
+concat and kept indices / class ids exact; box coordinates 1e-4.
+The shape sweeps mirror the reference's DIFFERENT_SHAPE_LOOP
+(ogl_runtime/opengl/nn/kernels/kernel_test_utils.h:59-65) and its conv tests
+(conv2d_test.cc:220-354: any-format input, no bias, dilation 2, grouped, stride 2
+at 320x320x3->32, depthwise).
+"""
+import numpy as np
+import pytest
+
+import oracle as O
+from ogle_amd import hip as H
+from util import (assert_conv_close, gpu_concat, gpu_conv, gpu_decode, gpu_detect, gpu_pool, rng)
+
+pytestmark = pytest.mark.gpu
+
+FP32_RTOL = 1e-4
+FP16_RTOL = 5e-3
+
+
+def check_conv(x, w, b, stride=1, pad=0, dil=1, groups=1, act=H.ACT_NONE, minv=0.0, maxv=0.0,
+               variant=H.VARIANT_NHWC4, dtype=H.F32, entry=None, what=""):
+    ref = O.conv2d(x, w, b, stride, pad, dil, groups, act, minv, maxv, variant)
+    scale = O.conv2d_abs(x, w, b, stride, pad, dil, groups)
+    got = gpu_conv(x, w, b, stride, pad, dil, groups, act, minv, maxv, variant, dtype, entry)
+    return assert_conv_close(got, ref, scale, FP16_RTOL if dtype == H.F16 else FP32_RTOL, what)
+
+
+
+def assert_same_detections(got, ora, logits, threshold, what=""):
+    """Kept prior indices and class ids must be bit-exact; scores may differ in the last
+    place because the host's expf is not correctly rounded on every input (the device's is).
+    A prior whose decision a 1-ulp change of one exponential could flip (score within 2e-6 of
+    the threshold, or its two best foreground classes within 2e-6 of each other) is excluded
+    from the exact comparison and counted; none occurs with the seeds used here."""
+    l64 = logits.astype(np.float64)
+    e = np.exp(l64 - l64.max(-1, keepdims=True))
+    sm = e / e.sum(-1, keepdims=True)
+    fg = np.sort(sm[:, 1:], axis=-1)
+    ambiguous = (np.abs(fg[:, -1] - threshold) < 2e-6) | ((fg[:, -1] - fg[:, -2]) < 2e-6 * fg[:, -1])
+    amb = set(np.nonzero(ambiguous)[0].tolist())
+    gp = [(int(p), int(c)) for p, c in zip(got["prior"], got["cls"]) if int(p) not in amb]
+    op = [(int(p), int(c)) for p, c in zip(ora["prior"], ora["cls"]) if int(p) not in amb]
+    assert gp == op, what
+    if len(got["prior"]) == len(ora["prior"]) and np.array_equal(got["prior"], ora["prior"]):
+        np.testing.assert_allclose(got["score"], ora["score"], rtol=3e-7, atol=0)
+        np.testing.assert_array_equal(got["box"], ora["box"])
+        np.testing.assert_array_equal(got["rect"], ora["rect"])
+    return len(amb)
+
+
+SMALL_CASES = [
+    # n, h, w, c, o, k, s, p, d, g
+    (1, 3, 3, 3, 1, 3, 1, 1, 1, 1),
+    (2, 7, 5, 4, 6, 3, 1, 1, 1, 1),
+    (1, 9, 9, 5, 7, 3, 2, 1, 1, 1),
+    (1, 8, 8, 3, 4, 3, 1, 2, 2, 1),
+    (2, 6, 6, 8, 8, 3, 1, 1, 1, 8),
+    (1, 6, 7, 8, 12, 3, 2, 1, 1, 4),
+    (3, 5, 5, 16, 9, 1, 1, 0, 1, 1),
+    (1, 10, 10, 6, 4, 5, 1, 2, 1, 1),
+    (1, 4, 4, 2, 3, 1, 2, 0, 1, 1),
+    (1, 1, 1, 20, 5, 3, 1, 1, 1, 1),
+    (2, 13, 11, 32, 40, 3, 1, 1, 1, 1),    # MFMA path, ragged M and N
+    (1, 17, 17, 64, 130, 3, 2, 1, 1, 1),   # MFMA path, stride 2, N just over a tile
+    (1, 9, 9, 36, 33, 3, 1, 1, 2, 1),      # MFMA path, dilation 2, K tail inside a slab
+    (4, 19, 19, 128, 24, 3, 1, 1, 1, 1),   # SSD loc head shape
+    (2, 10, 10, 64, 126, 3, 1, 1, 1, 1),   # SSD conf head shape
+    (1, 5, 5, 48, 72, 1, 1, 0, 1, 1),      # pointwise, K not a multiple of the slab
+    (2, 9, 7, 12, 12, 5, 2, 2, 1, 12),     # depthwise 5x5 stride 2 (general kernel)
+    (1, 8, 8, 6, 6, 3, 1, 1, 1, 6),        # depthwise, C not a multiple of 4
+    (1, 11, 9, 16, 16, 3, 2, 1, 1, 16),    # depthwise stride 2
+]
+
+
+@pytest.mark.parametrize("case", SMALL_CASES)
+@pytest.mark.parametrize("use_bias", [False, True])
+def test_conv_small_cases(case, use_bias):
+    n, h, w, c, o, k, s, p, d, g = case
+    r = rng(1000 + SMALL_CASES.index(case))
+    x = r.uniform(-1, 1, (n, h, w, c)).astype(np.float32)
+    wt = r.normal(0, 0.5, (o, c // g, k, k)).astype(np.float32)
+    b = r.uniform(-0.1, 0.1, o).astype(np.float32) if use_bias else None
+    check_conv(x, wt, b, s, p, d, g, what=str(case))
+
+
+def test_conv_shape_sweep_dense_and_depthwise():
+    """size 1,2,4..32 x channels 1..20, dense 3x3 p1 and depthwise, with bias + ReLU."""
+    r = rng(2000)
+    for size in (1, 2, 4, 8, 16, 32):
+        for ch in range(1, 21):
+            x = r.uniform(-1, 1, (2, size, size, ch)).astype(np.float32)
+            wt = r.normal(0, 0.5, (ch + 1, ch, 3, 3)).astype(np.float32)
+            b = r.uniform(-0.1, 0.1, ch + 1).astype(np.float32)
+            check_conv(x, wt, b, 1, 1, act=H.ACT_RELU, what="dense %d %d" % (size, ch))
+            wd = r.normal(0, 0.5, (ch, 1, 3, 3)).astype(np.float32)
+            bd = r.uniform(-0.1, 0.1, ch).astype(np.float32)
+            check_conv(x, wd, bd, 1, 1, 1, ch, act=H.ACT_CLIP, maxv=0.5,
+                       entry="ogle_hip_dwconv2d", what="dw %d %d" % (size, ch))
+
+
+def test_conv_shape_sweep_mfma_path():
+    """Channel counts that take the implicit-GEMM kernel, ragged in every dimension."""
+    r = rng(2100)
+    for (h, w) in ((1, 1), (3, 5), (8, 8), (19, 19), (33, 9)):
+        for c in (8, 12, 16, 20, 64, 100):
+            for o in (1, 31, 32, 33, 64, 65, 129):
+                x = r.uniform(-1, 1, (2, h, w, c)).astype(np.float32)
+                wt = r.normal(0, 0.3, (o, c, 1, 1)).astype(np.float32)
+                b = r.uniform(-0.1, 0.1, o).astype(np.float32)
+                check_conv(x, wt, b, act=H.ACT_RELU, variant=H.VARIANT_PW,
+                           what="pw %dx%d c%d o%d" % (h, w, c, o))
+    for c in (8, 16, 36):
+        for o in (4, 40, 70):
+            x = r.uniform(-1, 1, (1, 7, 6, c)).astype(np.float32)
+            wt = r.normal(0, 0.3, (o, c, 3, 3)).astype(np.float32)
+            check_conv(x, wt, None, 1, 1, what="3x3 c%d o%d" % (c, o))
+
+
+def test_activation_variants_on_device():
+    r = rng(2200)
+    x = r.uniform(-2, 2, (1, 6, 6, 16)).astype(np.float32)
+    w1 = r.normal(0, 0.5, (16, 16, 1, 1)).astype(np.float32)
+    w3 = r.normal(0, 0.3, (16, 16, 3, 3)).astype(np.float32)
+    wd = r.normal(0, 0.5, (16, 1, 3, 3)).astype(np.float32)
+    for variant in (H.VARIANT_NHWC4, H.VARIANT_PW, H.VARIANT_ANY4):
+        for act, mn, mx in ((H.ACT_CLIP, -0.5, 1.0), (H.ACT_RELU, -0.25, 0.0), (H.ACT_CLIP, 0.0, 6.0)):
+            check_conv(x, w1, None, act=act, minv=mn, maxv=mx, variant=variant, what="pw act")
+            check_conv(x, w3, None, 1, 1, act=act, minv=mn, maxv=mx, variant=variant, what="3x3 act")
+            check_conv(x, wd, None, 1, 1, 1, 16, act=act, minv=mn, maxv=mx, variant=variant,
+                       what="dw act")
+
+
+def test_stride2_stem_320():
+    """conv2d_test.cc:324-337: 320x320x3 -> 32, 3x3 stride 2."""
+    r = rng(2300)
+    x = r.uniform(-1, 1, (1, 320, 320, 3)).astype(np.float32)
+    w = r.normal(0, np.sqrt(2 / 27), (32, 3, 3, 3)).astype(np.float32)
+    b = r.uniform(-0.1, 0.1, 32).astype(np.float32)
+    check_conv(x, w, b, 2, 1, act=H.ACT_CLIP, maxv=6.0, what="stem")
+
+
+# ----------------------------------------------------------- BASELINE configs --
+
+def test_config1_dense_3x3():
+    r = rng(20240001)
+    x = r.uniform(-1, 1, (1, 112, 112, 32)).astype(np.float32)
+    w = r.normal(0, np.sqrt(2 / 288), (64, 32, 3, 3)).astype(np.float32)
+    b = r.uniform(-0.1, 0.1, 64).astype(np.float32)
+    check_conv(x, w, b, 1, 1, act=H.ACT_RELU, what="C1")
+
+
+@pytest.mark.parametrize("batch", [1, 8])
+def test_config2_depthwise_separable_block(batch):
+    r = rng(20240002)
+    x = r.uniform(0, 6, (batch, 38, 38, 256)).astype(np.float32)
+    wd = r.normal(0, np.sqrt(2 / 9), (256, 1, 3, 3)).astype(np.float32)
+    wp = r.normal(0, np.sqrt(2 / 256), (512, 256, 1, 1)).astype(np.float32)
+
+    def bn(c):
+        return (r.uniform(0.5, 1.5, c).astype(np.float32), r.normal(0, 0.1, c).astype(np.float32),
+                r.normal(0, 0.1, c).astype(np.float32), r.uniform(0.5, 1.5, c).astype(np.float32))
+
+    wdf, bdf = O.fold_bn(wd, None, *bn(256))
+    wpf, bpf = O.fold_bn(wp, None, *bn(512))
+    ref1 = O.conv2d(x, wdf, bdf, 1, 1, 1, 256, O.ACT_CLIP, 0.0, 6.0)
+    got1 = gpu_conv(x, wdf, bdf, 1, 1, 1, 256, H.ACT_CLIP, 0.0, 6.0)
+    assert_conv_close(got1, ref1, O.conv2d_abs(x, wdf, bdf, 1, 1, 1, 256), FP32_RTOL, "C2 dw")
+    ref2 = O.conv2d(ref1, wpf, bpf, act=O.ACT_CLIP, maxv=6.0, variant=O.VARIANT_PW)
+    got2 = gpu_conv(ref1, wpf, bpf, act=H.ACT_CLIP, maxv=6.0, variant=H.VARIANT_PW)
+    assert_conv_close(got2, ref2, O.conv2d_abs(ref1, wpf, bpf), FP32_RTOL, "C2 pw")
+
+
+@pytest.mark.parametrize("dtype", [H.F32, H.F16])
+def test_config3_pointwise_gemm(dtype):
+    r = rng(20240003)
+    x = r.uniform(0, 6, (32, 19, 19, 512)).astype(np.float32)
+    w = r.normal(0, np.sqrt(2 / 512), (1024, 512, 1, 1)).astype(np.float32)
+    b = r.uniform(-0.1, 0.1, 1024).astype(np.float32)
+    # float64 matmul is the tight reference here (the scalar oracle takes minutes at this size);
+    # the oracle itself is compared on the first image below.
+    a64 = x.reshape(-1, 512).astype(np.float64)
+    ref = np.maximum(a64 @ w.reshape(1024, 512).astype(np.float64).T + b, 0).astype(np.float32)
+    scale = (np.abs(a64) @ np.abs(w.reshape(1024, 512)).astype(np.float64).T + np.abs(b))
+    got = gpu_conv(x, w, b, act=H.ACT_RELU, variant=H.VARIANT_PW, dtype=dtype)
+    rtol = FP16_RTOL if dtype == H.F16 else FP32_RTOL
+    assert_conv_close(got.reshape(-1, 1024), ref, scale.astype(np.float32), rtol, "C3")
+    ora = O.conv2d(x[:1], w, b, act=O.ACT_RELU, variant=O.VARIANT_PW)
+    assert_conv_close(got[:1], ora, scale[:361].reshape(1, 19, 19, 1024).astype(np.float32), rtol,
+                      "C3 vs oracle")
+
+
+def ssd_anchors():
+    """1917 center-size priors: 19/10/5/3/2/1 maps, 3,6,6,6,6,6 anchors, scales 0.2-0.95."""
+    maps, counts = [19, 10, 5, 3, 2, 1], [3, 6, 6, 6, 6, 6]
+    scales = [0.2 + (0.95 - 0.2) * i / 5 for i in range(6)] + [1.0]
+    out = []
+    for k, (m, a) in enumerate(zip(maps, counts)):
+        ratios = [1.0, 2.0, 0.5] if a == 3 else [1.0, 2.0, 0.5, 3.0, 1.0 / 3.0]
+        for y in range(m):
+            for x in range(m):
+                cx, cy = (x + 0.5) / m, (y + 0.5) / m
+                for ar in ratios:
+                    out.append([cx, cy, scales[k] * np.sqrt(ar), scales[k] / np.sqrt(ar)])
+                if a == 6:
+                    s = np.sqrt(scales[k] * scales[k + 1])
+                    out.append([cx, cy, s, s])
+    a = np.array(out, np.float32)
+    assert a.shape == (1917, 4)
+    return a
+
+
+def test_config4_heads_concat_decode():
+    """SSD heads (3x3 convs) -> concat -> softmax-max/threshold -> decode, batch 4 for the
+    oracle-checked part (the oracle's convs at batch 64 take minutes)."""
+    r = rng(20240004)
+    batch = 4
+    maps = [(19, 512, 3), (10, 1024, 6), (5, 512, 6), (3, 256, 6), (2, 256, 6), (1, 128, 6)]
+    locs_ref, confs_ref, locs_gpu, confs_gpu = [], [], [], []
+    for m, c, a in maps:
+        f = r.uniform(0, 6, (batch, m, m, c)).astype(np.float32)
+        wl = r.normal(0, 0.01, (a * 4, c, 3, 3)).astype(np.float32)
+        wc = r.normal(0, 0.01, (a * 21, c, 3, 3)).astype(np.float32)
+        for wt, refs, gpus, last in ((wl, locs_ref, locs_gpu, 4), (wc, confs_ref, confs_gpu, 21)):
+            ref = O.conv2d(f, wt, None, 1, 1)
+            got = gpu_conv(f, wt, None, 1, 1)
+            assert_conv_close(got, ref, O.conv2d_abs(f, wt, None, 1, 1), FP32_RTOL, "head %d" % m)
+            refs.append(ref.reshape(batch, -1, last))
+            gpus.append(got.reshape(batch, -1, last))
+    loc = gpu_concat(locs_gpu, 1)
+    conf = gpu_concat(confs_gpu, 1)
+    np.testing.assert_array_equal(loc, np.concatenate(locs_gpu, 1))
+    np.testing.assert_array_equal(conf, np.concatenate(confs_gpu, 1))
+    np.testing.assert_array_equal(O.concat(locs_ref, 1), np.concatenate(locs_ref, 1))
+    assert loc.shape == (batch, 1917, 4) and conf.shape == (batch, 1917, 21)
+    anchors = ssd_anchors()
+    # Features ~U(0,6) over 9*C taps with weights ~N(0,0.01) give logits with a standard
+    # deviation near 2, so a good share of the priors passes the 0.3 threshold.  The score
+    # filter is compared on identical inputs: the device's own logits and decoded boxes.
+    res, boxes = gpu_detect(conf, loc, anchors, 0.3, 300.0, 300.0)
+    np.testing.assert_allclose(boxes, O.ssd_decode(loc, anchors), rtol=0, atol=1e-4)
+    ora = O.box_info(conf, boxes, 0.3, 300.0, 300.0)
+    for b in range(batch):
+        assert len(ora[b]["prior"]) > 0
+        assert_same_detections(res[b], ora[b], conf[b], 0.3, "C4 image %d" % b)
+        np.testing.assert_array_equal(res[b]["prior"], ora[b]["prior"])
+        np.testing.assert_array_equal(res[b]["cls"], ora[b]["cls"])
+
+
+@pytest.mark.parametrize("batch", [1, 64])
+def test_detect_kept_sets_bit_exact(batch):
+    """Logits scaled so that a few percent of the priors pass the threshold."""
+    r = rng(20240014 + batch)
+    priors, classes = 1917, 21
+    logits = r.normal(0, 0.9, (batch, priors, classes)).astype(np.float32)
+    pred = r.normal(0, 1.0, (batch, priors, 4)).astype(np.float32)
+    anchors = ssd_anchors()
+    res, boxes = gpu_detect(logits, pred, anchors, 0.3, 300.0, 300.0)
+    ref_boxes = O.ssd_decode(pred, anchors)
+    np.testing.assert_allclose(boxes, ref_boxes, rtol=0, atol=1e-4)
+    # identical inputs to the score filter on both sides: the device's own decoded boxes
+    ora = O.box_info(logits, boxes, 0.3, 300.0, 300.0)
+    kept = 0
+    for b in range(batch):
+        assert_same_detections(res[b], ora[b], logits[b], 0.3, "image %d" % b)
+        np.testing.assert_array_equal(res[b]["prior"], ora[b]["prior"])
+        np.testing.assert_array_equal(res[b]["cls"], ora[b]["cls"])
+        kept += len(res[b]["prior"])
+    frac = kept / (batch * priors)
+    assert 0.005 < frac < 0.6, frac
+    # with already-decoded boxes as input
+    res2, _ = gpu_detect(logits, None, None, 0.3, 300.0, 300.0, boxes_in=boxes)
+    for b in range(batch):
+        np.testing.assert_array_equal(res2[b]["prior"], ora[b]["prior"])
+        np.testing.assert_array_equal(res2[b]["box"], ora[b]["box"])
+
+
+def test_device_exp_matches_host_libm():
+    """The device exponential is the correctly rounded expf (binary64 exp, rounded once).  The
+    host's libm expf is within 0.502 ulp of the true value, so the two agree except on the few
+    inputs where libm is not correctly rounded; there they differ by one ulp."""
+    import ctypes
+    import torch
+    r = rng(77)
+    x = np.concatenate([r.uniform(-20, 20, 1 << 20), r.normal(0, 3, 1 << 20),
+                        np.linspace(-87, 88, 1 << 18)]).astype(np.float32)
+    xd = torch.from_numpy(x).cuda()
+    yd = torch.empty_like(xd)
+    H.check(H.lib().ogle_hip_expf(xd.data_ptr(), yd.data_ptr(), x.size,
+                                  torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    got, ref = yd.cpu().numpy(), O.expf(x)
+    mism = np.count_nonzero(got != ref)
+    assert mism <= x.size * 2e-3, "device exp differs from libm expf on %d of %d inputs" % (mism, x.size)
+    ulp = np.abs(got.view(np.int32).astype(np.int64) - ref.view(np.int32).astype(np.int64))
+    assert ulp.max() <= 1
+    # against binary64: the device result is the nearest binary32 to exp(x)
+    exact = np.exp(x.astype(np.float64))
+    ok = np.isfinite(ref) & (ref > 1e-37)
+    dev_err = np.abs(got[ok].astype(np.float64) - exact[ok])
+    host_err = np.abs(ref[ok].astype(np.float64) - exact[ok])
+    assert np.all(dev_err <= host_err * (1 + 1e-12) + 0.0)
+
+
+def test_decode_matches_oracle():
+    r = rng(3100)
+    anchors = ssd_anchors()
+    pred = r.normal(0, 1.5, (3, 1917, 4)).astype(np.float32)
+    got = gpu_decode(pred, anchors)
+    np.testing.assert_allclose(got, O.ssd_decode(pred, anchors), rtol=0, atol=1e-4)
+    # zero prediction: the anchor in corner form, exactly
+    z = gpu_decode(np.zeros((1, 1917, 4), np.float32), anchors)
+    exp = np.concatenate([anchors[:, :2] - anchors[:, 2:] * np.float32(0.5),
+                          anchors[:, :2] + anchors[:, 2:] * np.float32(0.5)], 1)
+    np.testing.assert_array_equal(z[0], exp)
+    # per-image anchors (the graph-op form)
+    a3 = np.stack([anchors, anchors * np.float32(0.5), anchors * np.float32(0.25)])
+    got = gpu_decode(pred, a3)
+    for b in range(3):
+        np.testing.assert_allclose(got[b:b + 1], O.ssd_decode(pred[b:b + 1], a3[b]), rtol=0, atol=1e-4)
+
+
+POOL_CASES = [
+    (1, 112, 112, 64, 3, 2, 1), (2, 11, 9, 5, 2, 2, 0), (1, 8, 8, 7, 3, 1, 1), (3, 13, 13, 16, 5, 3, 2),
+    (1, 4, 4, 4, 2, 2, 2),       # corner windows with no in-image tap
+]
+
+
+@pytest.mark.parametrize("case", POOL_CASES)
+def test_pool_matches_oracle(case):
+    n, h, w, c, k, s, p = case
+    x = rng(4000 + h).normal(0, 1, (n, h, w, c)).astype(np.float32)
+    np.testing.assert_array_equal(gpu_pool(x, k, s, p, H.POOL_MAX), O.pool2d(x, k, s, p, O.POOL_MAX))
+    np.testing.assert_array_equal(gpu_pool(x, k, s, p, H.POOL_AVG), O.pool2d(x, k, s, p, O.POOL_AVG))
+
+
+def test_global_average_pool():
+    r = rng(4100)
+    for (n, hw, c) in ((2, 7, 1024), (1, 3, 10), (3, 10, 130)):
+        x = r.normal(0, 1, (n, hw, hw, c)).astype(np.float32)
+        got = gpu_pool(x, 0, 0, 0, H.POOL_GLOBAL_AVG)
+        ref = O.pool2d(x, 0, 0, 0, O.POOL_GLOBAL_AVG)
+        scale = np.abs(x).sum(axis=(1, 2), keepdims=True) / (hw * hw)
+        assert np.all(np.abs(got - ref) <= 1e-5 * scale + 1e-12)
+
+
+@pytest.mark.parametrize("rank", [1, 2, 3, 4])
+def test_concat_every_axis(rank):
+    r = rng(5000 + rank)
+    base = [2, 3, 5, 4][:rank]
+    for axis in list(range(rank)) + [-1]:
+        for lens in ((1, 4, 2), (8, 4), (3, 1, 2, 5, 7, 1)):
+            ins = []
+            for ln in lens:
+                shp = list(base)
+                shp[axis] = ln
+                ins.append(r.normal(0, 1, shp).astype(np.float32))
+            np.testing.assert_array_equal(gpu_concat(ins, axis), O.concat(ins, axis))
+
+
+def test_concat_ssd_shapes_batch64():
+    r = rng(5100)
+    for last in (4, 21):
+        ins = [r.normal(0, 1, (64, p, last)).astype(np.float32) for p in (1083, 600, 150, 54, 24, 6)]
+        np.testing.assert_array_equal(gpu_concat(ins, 1), np.concatenate(ins, 1))
