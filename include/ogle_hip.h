@@ -207,6 +207,27 @@ typedef struct OgleConcatArgs {
 int32_t ogle_hip_concat(const OgleConcatArgs* args, ogle_stream_t stream);
 
 /* ------------------------------------------------------------------------ */
+/* Transpose                                                                  */
+/* ------------------------------------------------------------------------ */
+
+/*
+ * Permutation of a rank-4 row-major tensor: output dimension d is input
+ * dimension perm[d] (out_shape[d] == in_shape[perm[d]]).  Uniforms of
+ * TransposeKernel::Compute (ogl_runtime/opengl/nn/kernels/transpose.cc:71-89,
+ * shaders transpose.glsl / transpose_any4.glsl); lower ranks are left-padded with
+ * 1s by the caller as AmendShape / AmendPerm do (transpose.cc:13-31).
+ */
+typedef struct OgleTransposeArgs {
+  const void* input_dev;
+  void* output_dev;
+  int32_t in_shape[4];
+  int32_t perm[4];
+  int32_t dtype;
+} OgleTransposeArgs;
+
+int32_t ogle_hip_transpose(const OgleTransposeArgs* args, ogle_stream_t stream);
+
+/* ------------------------------------------------------------------------ */
 /* SSD box decoder and score filter                                           */
 /* ------------------------------------------------------------------------ */
 

@@ -1,0 +1,129 @@
+/*
+ * ogle_runtime.h - C ABI of the graph runtime (libogle_runtime.so).
+ *
+ * The runtime itself is C++ and keeps the reference's classes (opengl::Kernel,
+ * KernelRegistry, FBOSession, Tensor, Context, Detector; headers under
+ * ogle_amd/runtime/opengl).  These entry points expose FBOSession's public
+ * interface (ogl_runtime/opengl/core/fbo_session.h:20-51) and the SSD Detector
+ * (ogl_runtime/opengl/examples/ssd/detector.h:28-79) to callers that cannot link
+ * C++: tests and benchmarks drive the executor through them from Python.
+ *
+ * A fatal condition (the reference's CHECK / LOG(FATAL) abort) surfaces here as a
+ * negative return value; ogle_rt_last_error() holds its "file:line message".
+ */
+#ifndef OGLE_RUNTIME_H_
+#define OGLE_RUNTIME_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct OgleSession OgleSession; /* an opengl::FBOSession plus its Context */
+
+const char* ogle_rt_last_error(void);
+
+/* FBOSession(): one context (one HIP stream) per session. */
+OgleSession* ogle_rt_session_create(void);
+void ogle_rt_session_destroy(OgleSession* s);
+
+/* FBOSession::LoadGraph(path) / LoadGraph(ModelProto) from serialized bytes
+ * (fbo_session.cc:62-124). */
+int32_t ogle_rt_load_file(OgleSession* s, const char* path);
+int32_t ogle_rt_load_bytes(OgleSession* s, const void* data, size_t size);
+
+/*
+ * FBOSession::Run(NamedTensorList) (fbo_session.cc:127-165).  Input i is a host
+ * float buffer named names[i] of shape dims[i][0..ranks[i]) whose element order is
+ * dformats[i] ("NHWC", "NCHW" or "ANY").  The first call allocates every tensor.
+ */
+int32_t ogle_rt_run(OgleSession* s, int32_t n_inputs, const char* const* names,
+                    const float* const* data, const int32_t* const* dims, const int32_t* ranks,
+                    const char* const* dformats);
+
+/* One pass over the kernels with inputs already resident on the device. */
+int32_t ogle_rt_compute(OgleSession* s);
+/* The same pass as one captured hipGraph (captured on the first call). */
+int32_t ogle_rt_compute_graph(OgleSession* s);
+int32_t ogle_rt_sync(OgleSession* s);
+
+/*
+ * Times `iters` passes (after `warmup` untimed ones) with HIP events recorded on
+ * the session's stream; inputs stay resident.  use_graph selects ogle_rt_compute
+ * or ogle_rt_compute_graph.  ms_each (may be NULL) receives one duration per pass,
+ * each pass bracketed by its own event pair; *total_ms the span of all passes.
+ */
+int32_t ogle_rt_time_compute(OgleSession* s, int32_t warmup, int32_t iters, int32_t use_graph,
+                             float* ms_each, float* total_ms);
+
+/*
+ * One pass with an event pair around every node (the reference's per-node TraceMe
+ * with sync, fbo_session.cc:140-153).  Returns the number of nodes timed, or a
+ * negative status.  ogle_rt_profile_entry then reads entry i: its
+ * "<node>#<type>#" label, op type and milliseconds.
+ */
+int32_t ogle_rt_profile(OgleSession* s);
+int32_t ogle_rt_profile_entry(OgleSession* s, int32_t i, const char** label, const char** type,
+                              float* ms);
+
+/* Shape of a tensor by name (FindTensorByName): writes up to 8 dims, returns rank. */
+int32_t ogle_rt_tensor_shape(OgleSession* s, const char* name, int32_t* dims);
+/* Layout tag of a tensor as a TensorProto.DataFormat value (dlxnet.proto:7-30), or negative. */
+int32_t ogle_rt_tensor_dformat(OgleSession* s, const char* name);
+/* Device address of a tensor's first element (for zero-copy consumers), or NULL. */
+void* ogle_rt_tensor_device_ptr(OgleSession* s, const char* name);
+/* The session's hipStream_t. */
+void* ogle_rt_stream(OgleSession* s);
+
+/*
+ * FBOSession::GetOutputs for one tensor (fbo_session.cc:276-300): copies it to
+ * `dst` (capacity in floats) converted to `dformat`; the sync point.  Returns the
+ * element count.
+ */
+int64_t ogle_rt_get_output(OgleSession* s, const char* name, const char* dformat, float* dst,
+                           int64_t capacity);
+
+/*
+ * Parses a serialized ModelProto with the runtime's own wire codec and serializes
+ * it again into `out` (capacity bytes): returns the size written, or negative.  Lets
+ * a test check the hand-written .dlx codec against another protobuf implementation.
+ * ogle_rt_model_debug_string does the same into the text form of DebugString().
+ */
+int64_t ogle_rt_reserialize(const void* data, size_t size, void* out, int64_t capacity);
+int64_t ogle_rt_model_debug_string(const void* data, size_t size, char* out, int64_t capacity);
+
+/* Number of kernels the loaded graph created, and registered op-type names. */
+int32_t ogle_rt_num_kernels(OgleSession* s);
+int32_t ogle_rt_registered_kernel_count(void);
+const char* ogle_rt_registered_kernel_name(int32_t i);
+
+/* One detection, as BoxInfo (examples/ssd/common.h:29-45). */
+typedef struct OgleDetection {
+  int32_t image;      /* index in the batch */
+  int32_t prior;      /* BoxInfo.index */
+  int32_t class_id;   /* BoxInfo.class_name */
+  float score;
+  int32_t x, y, width, height; /* BoxInfo.box (integer rectangle) */
+  float cx, cy;
+} OgleDetection;
+
+/*
+ * Detector::Detect (examples/ssd/detector.cc:275-295) on a loaded session: runs the
+ * graph on `images` (host NHWC floats, already preprocessed), decodes and filters
+ * on the device, then top-k and NMS.  Tensor names are cls_logits / box_preds /
+ * anchors unless overridden (NULL keeps the default).  Writes up to `capacity`
+ * detections, returns how many there are in total.
+ */
+int64_t ogle_rt_detect(OgleSession* s, const float* images, const int32_t* dims /* n,h,w,c */,
+                       const char* input_name, const char* cls_name, const char* box_name,
+                       const char* anchors_name, float score_threshold, float nms_threshold,
+                       int32_t topk, int32_t raw_width, int32_t raw_height, OgleDetection* out,
+                       int64_t capacity);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* OGLE_RUNTIME_H_ */

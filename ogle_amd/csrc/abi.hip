@@ -31,7 +31,7 @@ namespace {
 // options the reference composes (conv2d.cc:54-62).
 enum Family {
   FAM_CONV = 1, FAM_CONV_DW = 2, FAM_CONV_PW = 3, FAM_CONV_GRP = 4,
-  FAM_POOL = 5, FAM_CONCAT = 6, FAM_DECODER = 7
+  FAM_POOL = 5, FAM_CONCAT = 6, FAM_DECODER = 7, FAM_TRANSPOSE = 8, FAM_RESHAPE = 9
 };
 enum Flags { FLAG_BIAS = 1, FLAG_CLIP = 2, FLAG_RELU = 4, FLAG_ANY4 = 8 };
 
@@ -53,6 +53,10 @@ const Entry kRegistry[] = {
     {"pool_any4", FAM_POOL, FLAG_ANY4},
     {"concat_multi", FAM_CONCAT, 0},
     {"decoder", FAM_DECODER, 0},
+    {"transpose", FAM_TRANSPOSE, 0},
+    {"transpose_any4", FAM_TRANSPOSE, FLAG_ANY4},
+    {"reshape", FAM_RESHAPE, 0},
+    {"reshape_any4", FAM_RESHAPE, FLAG_ANY4},
 };
 constexpr int kRegistrySize = sizeof(kRegistry) / sizeof(kRegistry[0]);
 
@@ -259,6 +263,24 @@ int32_t ogle_hip_concat(const OgleConcatArgs* a, ogle_stream_t stream) {
   if (total * a->outer * a->inner > 0 && a->output_dev == nullptr)
     return fail(OGLE_ERR_INVALID_ARG, "concat: null output");
   return launch_concat(*a, as_stream(stream));
+}
+
+int32_t ogle_hip_transpose(const OgleTransposeArgs* a, ogle_stream_t stream) {
+  if (a == nullptr) return fail(OGLE_ERR_INVALID_ARG, "transpose: null args");
+  if (a->dtype != OGLE_F32 && a->dtype != OGLE_F16)
+    return fail(OGLE_ERR_INVALID_ARG, "transpose: unknown dtype");
+  int seen = 0;
+  int64_t total = 1;
+  for (int d = 0; d < 4; ++d) {
+    if (a->perm[d] < 0 || a->perm[d] > 3 || a->in_shape[d] < 0)
+      return fail(OGLE_ERR_INVALID_ARG, "transpose: bad perm or shape");
+    seen |= 1 << a->perm[d];
+    total *= a->in_shape[d];
+  }
+  if (seen != 15) return fail(OGLE_ERR_INVALID_ARG, "transpose: perm is not a permutation");
+  if (total > 0 && (!a->input_dev || !a->output_dev))
+    return fail(OGLE_ERR_INVALID_ARG, "transpose: null pointer");
+  return launch_transpose(*a, as_stream(stream));
 }
 
 int32_t ogle_hip_ssd_decode(const OgleDecodeArgs* a, ogle_stream_t stream) {

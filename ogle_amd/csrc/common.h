@@ -84,6 +84,7 @@ int32_t launch_conv_direct(const OgleConvArgs& a, hipStream_t s);
 int32_t launch_conv_dw(const OgleConvArgs& a, hipStream_t s);
 int32_t launch_pool(const OglePoolArgs& a, hipStream_t s);
 int32_t launch_concat(const OgleConcatArgs& a, hipStream_t s);
+int32_t launch_transpose(const OgleTransposeArgs& a, hipStream_t s);
 int32_t launch_decode(const OgleDecodeArgs& a, hipStream_t s);
 int32_t launch_detect(const OgleDetectArgs& a, hipStream_t s);
 int32_t launch_expf(const float* x, float* y, int64_t n, hipStream_t s);

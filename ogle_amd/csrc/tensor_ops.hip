@@ -124,6 +124,30 @@ __global__ __launch_bounds__(256) void concat_kernel(ConcatPlan p, E* __restrict
   }
 }
 
+// -------------------------------------------------------------- transpose --
+struct TransposePlan {
+  int out_shape[4];
+  long in_stride[4];  // input stride (elements) of output dimension d
+  long total;
+};
+
+// One thread per output element, output order; an identity permutation is a copy
+// and is done with 16-byte vectors by the launcher instead.
+template <typename E>
+__global__ __launch_bounds__(256) void transpose_kernel(TransposePlan p, const E* __restrict__ in,
+                                                        E* __restrict__ out) {
+  for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < p.total;
+       idx += (long)gridDim.x * blockDim.x) {
+    long t = idx;
+    const int d3 = (int)(t % p.out_shape[3]); t /= p.out_shape[3];
+    const int d2 = (int)(t % p.out_shape[2]); t /= p.out_shape[2];
+    const int d1 = (int)(t % p.out_shape[1]); t /= p.out_shape[1];
+    const int d0 = (int)t;
+    out[idx] = in[d0 * p.in_stride[0] + d1 * p.in_stride[1] + d2 * p.in_stride[2] +
+                  d3 * p.in_stride[3]];
+  }
+}
+
 // ------------------------------------------------------------ filter pack --
 // OIHW fp32 -> OHWI (layout 0) or [kh*kw][O] for depthwise (layout 1, I == 1).
 template <typename T>
@@ -235,6 +259,53 @@ int32_t launch_concat(const OgleConcatArgs& a, hipStream_t s) {
                        static_cast<uint16_t*>(a.output_dev));
   }
   return check_launch("concat_kernel");
+}
+
+int32_t launch_transpose(const OgleTransposeArgs& a, hipStream_t s) {
+  TransposePlan p{};
+  long stride[4];
+  stride[3] = 1;
+  for (int d = 2; d >= 0; --d) stride[d] = stride[d + 1] * a.in_shape[d + 1];
+  p.total = 1;
+  bool identity = true;
+  for (int d = 0; d < 4; ++d) {
+    p.out_shape[d] = a.in_shape[a.perm[d]];
+    p.in_stride[d] = stride[a.perm[d]];
+    p.total *= p.out_shape[d];
+    // moving a dimension of extent 1 does not change the element order
+    if (a.perm[d] != d) identity = false;
+  }
+  if (p.total == 0) return OGLE_OK;
+  if (!identity) {
+    // Equivalent to a copy when the non-unit dimensions keep their relative order.
+    int last = -1;
+    identity = true;
+    for (int d = 0; d < 4; ++d) {
+      if (p.out_shape[d] == 1) continue;
+      if (a.perm[d] < last) identity = false;
+      last = a.perm[d];
+    }
+  }
+  const int esz = a.dtype == OGLE_F16 ? 2 : 4;
+  if (identity) {
+    const hipError_t e = hipMemcpyAsync(a.output_dev, a.input_dev, (size_t)p.total * esz,
+                                        hipMemcpyDeviceToDevice, s);
+    if (e != hipSuccess) {
+      set_error("transpose: copy failed: %s", hipGetErrorString(e));
+      return OGLE_ERR_LAUNCH;
+    }
+    return OGLE_OK;
+  }
+  if (esz == 4) {
+    hipLaunchKernelGGL((transpose_kernel<uint32_t>), dim3(grid_for(p.total)), dim3(256), 0, s, p,
+                       static_cast<const uint32_t*>(a.input_dev),
+                       static_cast<uint32_t*>(a.output_dev));
+  } else {
+    hipLaunchKernelGGL((transpose_kernel<uint16_t>), dim3(grid_for(p.total)), dim3(256), 0, s, p,
+                       static_cast<const uint16_t*>(a.input_dev),
+                       static_cast<uint16_t*>(a.output_dev));
+  }
+  return check_launch("transpose_kernel");
 }
 
 int32_t launch_pack_filter(const float* src, void* dst, int layout, int dtype, int o, int i,

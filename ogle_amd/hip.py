@@ -25,7 +25,7 @@ SYMBOLS = [
     "ogle_hip_sync", "ogle_hip_packed_filter_elems", "ogle_hip_pack_filter",
     "ogle_hip_convert", "ogle_hip_conv2d", "ogle_hip_dwconv2d", "ogle_hip_pwconv_gemm",
     "ogle_hip_pool2d", "ogle_hip_concat", "ogle_hip_ssd_decode", "ogle_hip_ssd_detect",
-    "ogle_hip_expf",
+    "ogle_hip_expf", "ogle_hip_transpose",
 ]
 
 
@@ -65,6 +65,13 @@ class ConcatArgs(ctypes.Structure):
         ("axis_len", ctypes.c_int64 * CONCAT_MAX_INPUTS),
         ("output_dev", ctypes.c_void_p), ("n_inputs", ctypes.c_int32),
         ("outer", ctypes.c_int64), ("inner", ctypes.c_int64), ("dtype", ctypes.c_int32),
+    ]
+
+
+class TransposeArgs(ctypes.Structure):
+    _fields_ = [
+        ("input_dev", ctypes.c_void_p), ("output_dev", ctypes.c_void_p),
+        ("in_shape", ctypes.c_int32 * 4), ("perm", ctypes.c_int32 * 4), ("dtype", ctypes.c_int32),
     ]
 
 
@@ -118,7 +125,8 @@ def lib():
         for name, typ in (("ogle_hip_conv2d", ConvArgs), ("ogle_hip_dwconv2d", ConvArgs),
                           ("ogle_hip_pwconv_gemm", ConvArgs), ("ogle_hip_pool2d", PoolArgs),
                           ("ogle_hip_concat", ConcatArgs), ("ogle_hip_ssd_decode", DecodeArgs),
-                          ("ogle_hip_ssd_detect", DetectArgs)):
+                          ("ogle_hip_ssd_detect", DetectArgs),
+                          ("ogle_hip_transpose", TransposeArgs)):
             getattr(l, name).argtypes = [ctypes.POINTER(typ), ctypes.c_void_p]
         l.ogle_hip_expf.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64,
                                     ctypes.c_void_p]

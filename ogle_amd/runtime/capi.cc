@@ -1,0 +1,324 @@
+// C ABI over the C++ graph runtime (include/ogle_runtime.h).
+#include "ogle_runtime.h"
+
+#include <hip/hip_runtime_api.h>
+
+#include <cstring>
+#include <exception>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "opengl/core/fbo_session.h"
+#include "opengl/core/kernel_registry.h"
+#include "opengl/core/tensor.h"
+#include "opengl/examples/ssd/detector.h"
+
+using opengl::FBOSession;
+using opengl::Tensor;
+
+struct OgleSession {
+  std::unique_ptr<opengl::Context> context;
+  std::unique_ptr<FBOSession> session;
+  std::vector<opengl::NodeTiming> timings;
+  std::unique_ptr<opengl::Detector> detector;
+};
+
+namespace {
+thread_local std::string g_error;
+
+template <typename F>
+int64_t Guard(F&& f) {
+  try {
+    return f();
+  } catch (const std::exception& e) {
+    g_error = e.what();
+    return -1;
+  } catch (...) {
+    g_error = "unknown exception";
+    return -1;
+  }
+}
+}  // namespace
+
+extern "C" {
+
+const char* ogle_rt_last_error(void) { return g_error.c_str(); }
+
+OgleSession* ogle_rt_session_create(void) {
+  OgleSession* s = nullptr;
+  Guard([&]() -> int64_t {
+    std::unique_ptr<OgleSession> p(new OgleSession);
+    p->context.reset(new opengl::Context);
+    p->session.reset(new FBOSession(p->context.get()));
+    s = p.release();
+    return 0;
+  });
+  return s;
+}
+
+void ogle_rt_session_destroy(OgleSession* s) {
+  if (s == nullptr) return;
+  Guard([&]() -> int64_t {
+    s->detector.reset();
+    s->session.reset();
+    s->context.reset();
+    return 0;
+  });
+  delete s;
+}
+
+int32_t ogle_rt_load_file(OgleSession* s, const char* path) {
+  return (int32_t)Guard([&]() -> int64_t {
+    s->session->LoadGraph(std::string(path));
+    return 0;
+  });
+}
+
+int32_t ogle_rt_load_bytes(OgleSession* s, const void* data, size_t size) {
+  return (int32_t)Guard([&]() -> int64_t {
+    dlxnet::ModelProto model;
+    if (!model.ParseFromArray(data, size)) {
+      g_error = "not a .dlx model";
+      return -1;
+    }
+    s->session->LoadGraph(model);
+    return 0;
+  });
+}
+
+int32_t ogle_rt_run(OgleSession* s, int32_t n_inputs, const char* const* names,
+                    const float* const* data, const int32_t* const* dims, const int32_t* ranks,
+                    const char* const* dformats) {
+  return (int32_t)Guard([&]() -> int64_t {
+    std::vector<std::unique_ptr<Tensor>> owned;
+    opengl::NamedTensorList inputs;
+    for (int i = 0; i < n_inputs; ++i) {
+      opengl::IntList shape(dims[i], dims[i] + ranks[i]);
+      owned.emplace_back(new Tensor(Tensor::DT_FLOAT, shape, data[i], opengl::StrToFormat(dformats[i])));
+      inputs.emplace_back(names[i], owned.back().get());
+    }
+    s->session->Run(inputs);
+    return 0;
+  });
+}
+
+int32_t ogle_rt_compute(OgleSession* s) {
+  return (int32_t)Guard([&]() -> int64_t {
+    s->session->Compute();
+    return 0;
+  });
+}
+
+int32_t ogle_rt_compute_graph(OgleSession* s) {
+  return (int32_t)Guard([&]() -> int64_t {
+    if (!s->session->graph_captured()) s->session->CaptureGraph();
+    s->session->LaunchGraph();
+    return 0;
+  });
+}
+
+int32_t ogle_rt_sync(OgleSession* s) {
+  return (int32_t)Guard([&]() -> int64_t {
+    s->context->Finish();
+    return 0;
+  });
+}
+
+int32_t ogle_rt_time_compute(OgleSession* s, int32_t warmup, int32_t iters, int32_t use_graph,
+                             float* ms_each, float* total_ms) {
+  return (int32_t)Guard([&]() -> int64_t {
+    hipStream_t st = static_cast<hipStream_t>(s->context->stream());
+    auto pass = [&]() {
+      if (use_graph) {
+        if (!s->session->graph_captured()) s->session->CaptureGraph();
+        s->session->LaunchGraph();
+      } else {
+        s->session->Compute();
+      }
+    };
+    for (int i = 0; i < warmup; ++i) pass();
+    s->context->Finish();
+    std::vector<hipEvent_t> ev(iters + 1);
+    for (auto& e : ev)
+      if (hipEventCreate(&e) != hipSuccess) LOG(FATAL) << "hipEventCreate failed";
+    (void)hipEventRecord(ev[0], st);
+    for (int i = 0; i < iters; ++i) {
+      pass();
+      (void)hipEventRecord(ev[i + 1], st);
+    }
+    s->context->Finish();
+    float total = 0.f;
+    (void)hipEventElapsedTime(&total, ev[0], ev[iters]);
+    if (total_ms) *total_ms = total;
+    if (ms_each)
+      for (int i = 0; i < iters; ++i) (void)hipEventElapsedTime(&ms_each[i], ev[i], ev[i + 1]);
+    for (auto& e : ev) (void)hipEventDestroy(e);
+    return 0;
+  });
+}
+
+int32_t ogle_rt_profile(OgleSession* s) {
+  return (int32_t)Guard([&]() -> int64_t {
+    s->session->RunProfiled(&s->timings);
+    return (int64_t)s->timings.size();
+  });
+}
+
+int32_t ogle_rt_profile_entry(OgleSession* s, int32_t i, const char** label, const char** type,
+                              float* ms) {
+  if (i < 0 || i >= (int32_t)s->timings.size()) {
+    g_error = "profile entry out of range";
+    return -1;
+  }
+  if (label) *label = s->timings[i].name.c_str();
+  if (type) *type = s->timings[i].type.c_str();
+  if (ms) *ms = s->timings[i].ms;
+  return 0;
+}
+
+int32_t ogle_rt_tensor_shape(OgleSession* s, const char* name, int32_t* dims) {
+  return (int32_t)Guard([&]() -> int64_t {
+    Tensor* t = s->session->FindTensorByName(name);
+    if (t == nullptr) {
+      g_error = std::string("tensor '") + name + "' is not allocated";
+      return -1;
+    }
+    const auto& shape = t->shape();
+    for (size_t i = 0; i < shape.size() && i < 8; ++i) dims[i] = shape[i];
+    return (int64_t)shape.size();
+  });
+}
+
+int32_t ogle_rt_tensor_dformat(OgleSession* s, const char* name) {
+  return (int32_t)Guard([&]() -> int64_t {
+    Tensor* t = s->session->FindTensorByName(name);
+    if (t == nullptr) {
+      g_error = std::string("tensor '") + name + "' is not allocated";
+      return -1;
+    }
+    return (int64_t)t->dformat();
+  });
+}
+
+void* ogle_rt_tensor_device_ptr(OgleSession* s, const char* name) {
+  void* p = nullptr;
+  Guard([&]() -> int64_t {
+    Tensor* t = s->session->FindTensorByName(name);
+    p = t ? t->device_ptr() : nullptr;
+    return 0;
+  });
+  return p;
+}
+
+void* ogle_rt_stream(OgleSession* s) {
+  void* p = nullptr;
+  Guard([&]() -> int64_t {
+    p = s->context->stream();
+    return 0;
+  });
+  return p;
+}
+
+int64_t ogle_rt_get_output(OgleSession* s, const char* name, const char* dformat, float* dst,
+                           int64_t capacity) {
+  return Guard([&]() -> int64_t {
+    opengl::TensorList outs;
+    s->session->GetOutputs({name}, {dformat}, &outs);
+    std::unique_ptr<Tensor> host(outs[0]);
+    const int64_t n = (int64_t)host->num_elements();
+    if (n > capacity) {
+      g_error = "output buffer too small";
+      return -1;
+    }
+    std::memcpy(dst, host->host(), n * sizeof(float));
+    return n;
+  });
+}
+
+int64_t ogle_rt_reserialize(const void* data, size_t size, void* out, int64_t capacity) {
+  return Guard([&]() -> int64_t {
+    dlxnet::ModelProto model;
+    if (!model.ParseFromArray(data, size)) {
+      g_error = "not a .dlx model";
+      return -1;
+    }
+    const std::string bytes = model.SerializeAsString();
+    if ((int64_t)bytes.size() > capacity) {
+      g_error = "output buffer too small";
+      return -1;
+    }
+    std::memcpy(out, bytes.data(), bytes.size());
+    return (int64_t)bytes.size();
+  });
+}
+
+int64_t ogle_rt_model_debug_string(const void* data, size_t size, char* out, int64_t capacity) {
+  return Guard([&]() -> int64_t {
+    dlxnet::ModelProto model;
+    if (!model.ParseFromArray(data, size)) {
+      g_error = "not a .dlx model";
+      return -1;
+    }
+    const std::string text = model.DebugString();
+    if ((int64_t)text.size() + 1 > capacity) {
+      g_error = "output buffer too small";
+      return -1;
+    }
+    std::memcpy(out, text.c_str(), text.size() + 1);
+    return (int64_t)text.size();
+  });
+}
+
+int32_t ogle_rt_num_kernels(OgleSession* s) { return s->session->num_kernels(); }
+
+int32_t ogle_rt_registered_kernel_count(void) {
+  return (int32_t)opengl::KernelRegistry::Global()->RegisteredNames().size();
+}
+
+const char* ogle_rt_registered_kernel_name(int32_t i) {
+  static thread_local std::string name;
+  const auto names = opengl::KernelRegistry::Global()->RegisteredNames();
+  if (i < 0 || i >= (int32_t)names.size()) return nullptr;
+  name = names[i];
+  return name.c_str();
+}
+
+int64_t ogle_rt_detect(OgleSession* s, const float* images, const int32_t* dims,
+                       const char* input_name, const char* cls_name, const char* box_name,
+                       const char* anchors_name, float score_threshold, float nms_threshold,
+                       int32_t topk, int32_t raw_width, int32_t raw_height, OgleDetection* out,
+                       int64_t capacity) {
+  return Guard([&]() -> int64_t {
+    opengl::DetectorOptions opt;
+    if (input_name) opt.input_names = {input_name};
+    if (cls_name) opt.output_names[0] = cls_name;
+    if (box_name) opt.output_names[1] = box_name;
+    if (anchors_name) opt.output_names[2] = anchors_name;
+    opt.score_threshold = score_threshold;
+    opt.nms_threshold = nms_threshold;
+    opt.topk = topk;
+    s->detector = opengl::Detector::Create(s->session.get(), opt);
+    opengl::IntList shape(dims, dims + 4);
+    Tensor input(Tensor::DT_FLOAT, shape, images, dlxnet::TensorProto::NHWC);
+    std::vector<std::vector<opengl::BoxInfo>> result;
+    s->detector->Detect(&input, raw_width, raw_height, &result);
+    int64_t n = 0;
+    for (size_t b = 0; b < result.size(); ++b)
+      for (const auto& info : result[b]) {
+        if (n < capacity) {
+          OgleDetection& d = out[n];
+          d.image = (int32_t)b;
+          d.prior = info.index;
+          d.class_id = info.class_name;
+          d.score = info.score;
+          d.x = info.box.x; d.y = info.box.y; d.width = info.box.width; d.height = info.box.height;
+          d.cx = info.cx; d.cy = info.cy;
+        }
+        ++n;
+      }
+    return n;
+  });
+}
+
+}  // extern "C"

@@ -1,0 +1,135 @@
+#include "opengl/core/context.h"
+
+#include <hip/hip_runtime_api.h>
+
+#include <vector>
+
+namespace opengl {
+
+#define OGLE_HIP_CALL(expr)                                                       \
+  do {                                                                            \
+    const hipError_t e__ = (expr);                                                \
+    if (e__ != hipSuccess) LOG(FATAL) << #expr << ": " << hipGetErrorString(e__); \
+  } while (0)
+
+Context::Context() {}
+
+void* Context::stream() {
+  if (stream_ == nullptr) {
+    hipStream_t s = nullptr;
+    OGLE_HIP_CALL(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+    stream_ = s;
+  }
+  return stream_;
+}
+
+Context::~Context() {
+  if (stream_ != nullptr) (void)hipStreamDestroy(static_cast<hipStream_t>(stream_));
+}
+
+Program* Context::CreateProgram(const std::string& kernel_fname, const std::string& build_options) {
+  if (kernel_fname.empty()) return nullptr;  // ops without device code (Const)
+  const std::string key = kernel_fname + "\n" + build_options;
+  auto it = programs_.find(key);
+  if (it != programs_.end()) return it->second.get();
+  int32_t handle = 0;
+  const int32_t st = ogle_hip_registry_lookup(kernel_fname.c_str(), build_options.c_str(), &handle);
+  if (st != OGLE_OK) LOG(FATAL) << "CreateProgram: " << ogle_hip_last_error();
+  Program* p = new Program(kernel_fname, build_options, handle, this);
+  programs_[key].reset(p);
+  return p;
+}
+
+namespace {
+// NCHW <-> NHWC on the host, rank 4 only.
+void Permute4(const float* src, float* dst, const IntList& nhwc, bool to_nhwc = false) {
+  const int n = nhwc[0], h = nhwc[1], w = nhwc[2], c = nhwc[3];
+  for (int b = 0; b < n; ++b)
+    for (int y = 0; y < h; ++y)
+      for (int x = 0; x < w; ++x)
+        for (int ch = 0; ch < c; ++ch) {
+          const size_t i_nhwc = ((static_cast<size_t>(b) * h + y) * w + x) * c + ch;
+          const size_t i_nchw = ((static_cast<size_t>(b) * c + ch) * h + y) * w + x;
+          if (to_nhwc) dst[i_nhwc] = src[i_nchw];
+          else dst[i_nchw] = src[i_nhwc];
+        }
+}
+bool IsImageTag(DataFormat f) {
+  return f == dlxnet::TensorProto::NHWC4 || f == dlxnet::TensorProto::NHWC;
+}
+}  // namespace
+
+void Context::CopyCPUTensorToDevice(const Tensor* cpu, Tensor* dev) {
+  CHECK(cpu->is_host()) << "source must be a host tensor";
+  CHECK(dev->mem_type() != Tensor::HOST_MEMORY) << "destination must be a device tensor";
+  CHECK_EQ(cpu->num_elements(), dev->num_elements());
+  const size_t bytes = cpu->num_elements() * sizeof(float);
+  if (bytes == 0) return;
+  hipStream_t s = static_cast<hipStream_t>(stream());
+  // The host tensor's element order is the device's: NHWC images, ANY tensors and
+  // filters in the file's OIHW order are all dense row-major over shape().
+  OGLE_HIP_CALL(hipMemcpyAsync(dev->device_ptr(), cpu->host(), bytes, hipMemcpyHostToDevice, s));
+  OGLE_HIP_CALL(hipStreamSynchronize(s));
+  dev->set_initialized(true);
+}
+
+void Context::CopyDeviceTensorToCPU(const Tensor* dev, Tensor* cpu) {
+  CHECK(cpu->is_host()) << "destination must be a host tensor";
+  CHECK(dev->mem_type() != Tensor::HOST_MEMORY) << "source must be a device tensor";
+  CHECK_EQ(cpu->num_elements(), dev->num_elements());
+  const size_t bytes = dev->num_elements() * sizeof(float);
+  hipStream_t s = static_cast<hipStream_t>(stream());
+  if (bytes == 0) {
+    OGLE_HIP_CALL(hipStreamSynchronize(s));
+    return;
+  }
+  if (cpu->dformat() == dlxnet::TensorProto::NCHW && IsImageTag(dev->dformat())) {
+    CHECK_EQ(dev->dims_size(), 4);
+    std::vector<float> tmp(dev->num_elements());
+    OGLE_HIP_CALL(hipMemcpyAsync(tmp.data(), dev->device_ptr(), bytes, hipMemcpyDeviceToHost, s));
+    OGLE_HIP_CALL(hipStreamSynchronize(s));
+    Permute4(tmp.data(), cpu->host<float>(), dev->shape(), false);
+  } else {
+    OGLE_HIP_CALL(hipMemcpyAsync(cpu->host(), dev->device_ptr(), bytes, hipMemcpyDeviceToHost, s));
+    OGLE_HIP_CALL(hipStreamSynchronize(s));
+  }
+  cpu->set_initialized(true);
+}
+
+void Context::Finish() { OGLE_HIP_CALL(hipStreamSynchronize(static_cast<hipStream_t>(stream()))); }
+
+Context* GetContext() {
+  static Context* context = new Context;
+  return context;
+}
+
+// ---- Program ---------------------------------------------------------------
+
+void Program::Check(int32_t status, const char* what) const {
+  if (status != OGLE_OK)
+    LOG(FATAL) << what << " (" << name_ << "): " << ogle_hip_status_string(status) << ": "
+               << ogle_hip_last_error();
+}
+void Program::RunConv2d(const OgleConvArgs& a) const {
+  Check(ogle_hip_conv2d(&a, context_->stream()), "ogle_hip_conv2d");
+}
+void Program::RunDepthwise(const OgleConvArgs& a) const {
+  Check(ogle_hip_dwconv2d(&a, context_->stream()), "ogle_hip_dwconv2d");
+}
+void Program::RunPointwise(const OgleConvArgs& a) const {
+  Check(ogle_hip_pwconv_gemm(&a, context_->stream()), "ogle_hip_pwconv_gemm");
+}
+void Program::RunPool(const OglePoolArgs& a) const {
+  Check(ogle_hip_pool2d(&a, context_->stream()), "ogle_hip_pool2d");
+}
+void Program::RunConcat(const OgleConcatArgs& a) const {
+  Check(ogle_hip_concat(&a, context_->stream()), "ogle_hip_concat");
+}
+void Program::RunDecode(const OgleDecodeArgs& a) const {
+  Check(ogle_hip_ssd_decode(&a, context_->stream()), "ogle_hip_ssd_decode");
+}
+void Program::RunTranspose(const OgleTransposeArgs& a) const {
+  Check(ogle_hip_transpose(&a, context_->stream()), "ogle_hip_transpose");
+}
+
+}  // namespace opengl

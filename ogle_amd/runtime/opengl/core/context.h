@@ -1,0 +1,49 @@
+// Device context: the stream, host<->device tensor copies and the program cache.
+// Counterpart of ogl_runtime/opengl/core/context.h:26-62 with HIP in place of GL.
+#ifndef OPENGL_CORE_CONTEXT_H_
+#define OPENGL_CORE_CONTEXT_H_
+
+#include <map>
+#include <memory>
+#include <string>
+
+#include "opengl/core/program.h"
+#include "opengl/core/tensor.h"
+#include "opengl/core/types.h"
+
+namespace opengl {
+
+class Context {
+ public:
+  Context();
+  ~Context();
+
+  // The HIP stream every kernel of this context is launched on (a hipStream_t),
+  // created on first use so that graph loading and validation need no device.
+  void* stream();
+
+  // Looks `kernel_fname` (a shader stem such as "conv2d_pw") up in the HIP kernel
+  // registry; programs are cached by name + build options and owned by the context
+  // (context.cc:288-313 of the reference).
+  Program* CreateProgram(const std::string& kernel_fname, const std::string& build_options = "");
+
+  // Host -> device.  Both sides are dense row-major over the logical shape (NHWC
+  // images, ANY tensors, OIHW filters), so this is one copy.
+  void CopyCPUTensorToDevice(const Tensor* cpu_tensor, Tensor* device_tensor);
+  // Device -> host, converting to the host tensor's dformat; synchronises.
+  void CopyDeviceTensorToCPU(const Tensor* device_tensor, Tensor* cpu_tensor);
+
+  void Finish();  // glFinish: waits for the stream
+  void Reset() {}
+
+ private:
+  void* stream_ = nullptr;
+  std::map<std::string, std::unique_ptr<Program>> programs_;
+};
+
+// Process-wide context (context.cc:316-319 of the reference).
+Context* GetContext();
+
+}  // namespace opengl
+
+#endif  // OPENGL_CORE_CONTEXT_H_

@@ -1,0 +1,246 @@
+#include "opengl/core/fbo_session.h"
+
+#include <hip/hip_runtime_api.h>
+
+#include <fstream>
+#include <sstream>
+
+#include "opengl/core/kernel.h"
+#include "opengl/core/kernel_registry.h"
+#include "opengl/core/tensor.h"
+#include "opengl/utils/logging.h"
+
+namespace opengl {
+
+#define OGLE_HIP_CALL(expr)                                                       \
+  do {                                                                            \
+    const hipError_t e__ = (expr);                                                \
+    if (e__ != hipSuccess) LOG(FATAL) << #expr << ": " << hipGetErrorString(e__); \
+  } while (0)
+
+FBOSession::FBOSession(Context* context) : context_(context) { context_->Reset(); }
+
+FBOSession::~FBOSession() {
+  if (graph_exec_ != nullptr) (void)hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph_exec_));
+  if (graph_ != nullptr) (void)hipGraphDestroy(static_cast<hipGraph_t>(graph_));
+  // Views must go before the buffers they alias; both are plain frees, so order
+  // only matters for tidiness: release in reverse creation order.
+  for (auto it = total_tensors_.rbegin(); it != total_tensors_.rend(); ++it) it->reset();
+}
+
+void FBOSession::LoadGraph(std::string model_path) {
+  std::ifstream in(model_path, std::ios::binary);
+  CHECK(in.good()) << "Load Graph " << model_path << " Failed: cannot open file";
+  std::stringstream buffer;
+  buffer << in.rdbuf();
+  const std::string bytes = buffer.str();
+  dlxnet::ModelProto model;
+  CHECK(model.ParseFromString(bytes)) << "Load Graph " << model_path << " Failed: not a .dlx model";
+  LoadGraph(model);
+}
+
+void FBOSession::LoadGraph(const ::dlxnet::ModelProto& model_proto) {
+  model_ = model_proto;
+  kernels_.clear();
+  total_tensors_.clear();
+  tensor_name_index_.clear();
+  default_input_sizes_.clear();
+  const dlxnet::GraphProto& graph = model_.graph();
+  total_tensors_.resize(graph.tensor_names_size());
+  for (int i = 0; i < graph.tensor_names_size(); ++i) tensor_name_index_[graph.tensor_names(i)] = i;
+
+  for (const dlxnet::NodeProto& node : graph.node()) {
+    if (node.type() == "Input") {
+      // Remembers the model's own spatial size (fbo_session.cc:102-111); no kernel.
+      const auto& dims = node.attr().input_attr().dims();
+      CHECK_GE(dims.size(), 2u) << "Input node '" << node.name() << "' needs at least 2 dims";
+      for (size_t i = dims.size() - 2; i < dims.size(); ++i) default_input_sizes_.push_back(dims[i]);
+      continue;
+    }
+    Kernel* kernel = nullptr;
+    KernelRegistry::Global()->CreateKernel(node.type(), &kernel, context_);
+    if (kernel == nullptr) LOG(FATAL) << "unsupported kernel name " << node.type();
+    std::unique_ptr<Kernel> owned(kernel);
+    for (auto idx : node.input_index())
+      CHECK(idx >= 0 && idx < graph.tensor_names_size()) << "node '" << node.name()
+                                                         << "' input index out of range";
+    for (auto idx : node.output_index())
+      CHECK(idx >= 0 && idx < graph.tensor_names_size()) << "node '" << node.name()
+                                                         << "' output index out of range";
+    kernel->Setup(node, this);
+    kernels_.push_back(std::move(owned));
+  }
+  finalized_ = false;
+  graph_created_ = true;
+}
+
+void FBOSession::Setup(const NamedTensorList& inputs_cpu) {
+  CHECK(graph_created_) << "No Graph Loaded!";
+  for (const auto& named : inputs_cpu) {
+    const Tensor* input_cpu = named.second;
+    auto it = tensor_name_index_.find(named.first);
+    if (it == tensor_name_index_.end()) LOG(FATAL) << "tensor_name: " << named.first << " Cannot Find";
+    const int index = it->second;
+    if (!finalized_) {
+      total_tensors_[index].reset(new Tensor(Tensor::DT_FLOAT, input_cpu->shape(),
+                                             Tensor::DEVICE_BUFFER,
+                                             FormatToStride4(input_cpu->dformat())));
+    } else {
+      // The input shape is fixed after the first Run (allow_resized_ is never set).
+      CHECK(allow_resized_ || total_tensors_[index]->shape() == input_cpu->shape())
+          << "input '" << named.first << "' changed shape after the session was finalized";
+    }
+    context_->CopyCPUTensorToDevice(input_cpu, total_tensors_[index].get());
+  }
+  if (finalized_) return;
+
+  ready_.assign(total_tensors_.size(), false);
+  for (size_t i = 0; i < kernels_.size(); ++i) {
+    Kernel* kernel = kernels_[i].get();
+    kernel->input_tensors_.clear();
+    kernel->output_tensors_.clear();
+    for (int idx : kernel->input_tensor_indexes_) {
+      Tensor* t = total_tensors_[idx].get();
+      CHECK(t != nullptr) << "input tensor is uninitialized of kernel index: " << i << " ("
+                          << kernel->kernel_type() << " '" << kernel->kernel_name() << "')";
+      kernel->input_tensors_.push_back(t);
+    }
+    kernel->SelectKernel(kernel->input_tensors_);
+    kernel->SetupProgram(context_->CreateProgram(kernel->kernel_fname(), kernel->build_options()));
+
+    TensorShapeList output_shapes;
+    kernel->InferOutputShape(kernel->input_tensors_, output_shapes);
+    CHECK_GT(output_shapes.size(), 0u);
+    CHECK_EQ(output_shapes.size(), kernel->output_tensor_indexes_.size())
+        << kernel->kernel_type() << " '" << kernel->kernel_name() << "'";
+    for (size_t j = 0; j < output_shapes.size(); ++j) {
+      const DataFormat dformat = kernel->GetOutputDFormat(static_cast<int>(j));
+      const int alias = kernel->OutputAliasesInput(static_cast<int>(j));
+      Tensor* out = nullptr;
+      if (alias >= 0) {
+        out = new Tensor(kernel->input_tensors_[alias], output_shapes[j], dformat);
+      } else {
+        out = new Tensor(Tensor::DT_FLOAT, output_shapes[j], Tensor::DEVICE_BUFFER, dformat);
+      }
+      total_tensors_[kernel->output_tensor_indexes_[j]].reset(out);
+      kernel->output_tensors_.push_back(out);
+    }
+    if (CheckKernelReady(kernel)) {
+      // Constants and constant-only subgraphs run once, here (fbo_session.cc:240-244).
+      kernel->Compute();
+      UpdateKernelReady(kernel);
+    }
+  }
+  finalized_ = true;
+}
+
+void FBOSession::Compute() {
+  CHECK(finalized_) << "Please Setup Session First";
+  for (auto& kernel : kernels_) {
+    if (CheckKernelReady(kernel.get())) continue;
+    kernel->Compute();
+  }
+}
+
+void FBOSession::Run(const NamedTensorList& inputs_cpu) {
+  Setup(inputs_cpu);
+  Compute();
+}
+
+void FBOSession::RunProfiled(std::vector<NodeTiming>* timings) {
+  CHECK(finalized_) << "Please Setup Session First";
+  hipStream_t s = static_cast<hipStream_t>(context_->stream());
+  std::vector<Kernel*> live;
+  for (auto& kernel : kernels_)
+    if (!CheckKernelReady(kernel.get())) live.push_back(kernel.get());
+  std::vector<hipEvent_t> ev(live.size() + 1);
+  for (auto& e : ev) OGLE_HIP_CALL(hipEventCreate(&e));
+  OGLE_HIP_CALL(hipEventRecord(ev[0], s));
+  for (size_t i = 0; i < live.size(); ++i) {
+    live[i]->Compute();
+    OGLE_HIP_CALL(hipEventRecord(ev[i + 1], s));
+  }
+  OGLE_HIP_CALL(hipStreamSynchronize(s));
+  timings->clear();
+  for (size_t i = 0; i < live.size(); ++i) {
+    float ms = 0.f;
+    OGLE_HIP_CALL(hipEventElapsedTime(&ms, ev[i], ev[i + 1]));
+    timings->push_back({live[i]->kernel_name() + "#" + live[i]->kernel_type() + "#",
+                        live[i]->kernel_type(), ms});
+  }
+  for (auto& e : ev) (void)hipEventDestroy(e);
+}
+
+void FBOSession::CaptureGraph() {
+  CHECK(finalized_) << "Please Setup Session First";
+  if (graph_exec_ != nullptr) return;
+  hipStream_t s = static_cast<hipStream_t>(context_->stream());
+  OGLE_HIP_CALL(hipStreamSynchronize(s));
+  hipGraph_t graph = nullptr;
+  OGLE_HIP_CALL(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal));
+  try {
+    Compute();
+  } catch (...) {
+    (void)hipStreamEndCapture(s, &graph);
+    if (graph != nullptr) (void)hipGraphDestroy(graph);
+    throw;
+  }
+  OGLE_HIP_CALL(hipStreamEndCapture(s, &graph));
+  hipGraphExec_t exec = nullptr;
+  OGLE_HIP_CALL(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0));
+  graph_ = graph;
+  graph_exec_ = exec;
+}
+
+void FBOSession::LaunchGraph() {
+  CHECK(graph_exec_ != nullptr) << "CaptureGraph first";
+  OGLE_HIP_CALL(hipGraphLaunch(static_cast<hipGraphExec_t>(graph_exec_),
+                               static_cast<hipStream_t>(context_->stream())));
+}
+
+bool FBOSession::CheckKernelReady(const Kernel* kernel) {
+  if (kernel->ForceReady()) return true;
+  for (int id : kernel->input_tensor_indexes_)
+    if (!ready_[id]) return false;
+  return true;
+}
+
+void FBOSession::UpdateKernelReady(const Kernel* kernel) {
+  for (int id : kernel->output_tensor_indexes_) ready_[id] = true;
+}
+
+void FBOSession::GetOutputs(const TensorNameList& output_names, const StringList& output_dformats,
+                            TensorList* outputs) {
+  CHECK_EQ(output_names.size(), output_dformats.size());
+  if (outputs->size() < output_names.size()) outputs->resize(output_names.size(), nullptr);
+  for (size_t i = 0; i < output_names.size(); ++i) {
+    Tensor* gpu_tensor = FindTensorByName(output_names[i]);
+    CHECK(gpu_tensor != nullptr) << "tensor '" << output_names[i] << "' was never produced";
+    const DataFormat dformat = StrToFormat(output_dformats[i]);
+    if (outputs->at(i) == nullptr) {
+      // The caller owns the host tensors GetOutputs creates (fbo_session.cc:294).
+      outputs->at(i) = new Tensor(Tensor::DT_FLOAT, gpu_tensor->shape(), Tensor::HOST_MEMORY, dformat);
+    } else {
+      CHECK(outputs->at(i)->shape() == gpu_tensor->shape()) << "reused output tensor has another shape";
+    }
+    context_->CopyDeviceTensorToCPU(gpu_tensor, outputs->at(i));
+  }
+}
+
+std::string FBOSession::DebugString() const {
+  return "ModelProto: " + model_.DebugString() + "\n";
+}
+
+Tensor* FBOSession::FindTensorByName(const std::string& tensor_name) {
+  auto it = tensor_name_index_.find(tensor_name);
+  if (it == tensor_name_index_.end()) LOG(FATAL) << "tensor_name: " << tensor_name << " Cannot Find";
+  return FindTensorById(it->second);
+}
+
+Tensor* FBOSession::FindTensorById(int id) {
+  CHECK_GE(id, 0);
+  CHECK_LT(id, static_cast<int>(total_tensors_.size()));
+  return total_tensors_[id].get();
+}
+
+}  // namespace opengl

@@ -1,0 +1,85 @@
+// Graph executor: loads a .dlx model, creates one Kernel per node, allocates every
+// tensor once on the first Run and then replays the kernels in file order.
+//
+// Public interface and behaviour follow ogl_runtime/opengl/core/fbo_session.h:11-90
+// and fbo_session.cc:62-325: nodes run in proto order (the converter emits them
+// topologically sorted), "Input" nodes have no kernel, constants and constant-only
+// subgraphs are computed once during Setup (the ready_ flags), only the first Run
+// allocates.  Additions for a launch-bound GPU: Compute() replays the kernels
+// without re-uploading inputs, RunProfiled() brackets every node with HIP events,
+// and CaptureGraph()/LaunchGraph() replay the whole run as one hipGraph.
+#ifndef OPENGL_CORE_FBO_SESSION_H_
+#define OPENGL_CORE_FBO_SESSION_H_
+
+#include <string>
+#include <vector>
+
+#include "opengl/core/context.h"
+#include "opengl/core/dlxnet.h"
+#include "opengl/core/types.h"
+
+namespace opengl {
+
+struct NodeTiming {
+  std::string name;  // "<node>#<type>#", the label the reference's TraceMe uses
+  std::string type;
+  float ms;
+};
+
+class FBOSession {
+ public:
+  explicit FBOSession(Context* context);
+  FBOSession() : FBOSession(GetContext()) {}
+  virtual ~FBOSession();
+
+  void LoadGraph(const ::dlxnet::ModelProto& model_proto);
+  void LoadGraph(std::string model_path);
+
+  // Allocates (first call only) and uploads the named host inputs.
+  void Setup(const NamedTensorList& inputs_cpu);
+  // Setup + one pass over the kernels.  Asynchronous: GetOutputs is the sync point.
+  void Run(const NamedTensorList& inputs_cpu);
+  // One pass over the kernels with the inputs already on the device.
+  void Compute();
+  // Compute() with a HIP event pair around every node; returns after the pass.
+  void RunProfiled(std::vector<NodeTiming>* timings);
+
+  // Records one Compute() pass into a hipGraph (once) and replays it.
+  void CaptureGraph();
+  void LaunchGraph();
+  bool graph_captured() const { return graph_exec_ != nullptr; }
+
+  void GetOutputs(const TensorNameList& output_names, const StringList& output_dformats,
+                  TensorList* outputs);
+
+  std::string DebugString() const;
+  Context* context() const { return context_; }
+  bool IsONNX() const { return model_.producer_name() == "ONNX"; }
+  Tensor* FindTensorByName(const std::string& name);
+  Tensor* FindTensorById(int id);
+  bool allow_resized() const { return allow_resized_; }
+  void set_allow_resized(bool flag) { allow_resized_ = flag; }
+  const IntList& default_input_sizes() const { return default_input_sizes_; }
+  int num_kernels() const { return static_cast<int>(kernels_.size()); }
+
+ private:
+  bool CheckKernelReady(const Kernel* kernel);
+  void UpdateKernelReady(const Kernel* kernel);
+
+  Context* context_;
+  OwnedKernelList kernels_;
+  dlxnet::ModelProto model_;
+  OwnedTensorList total_tensors_;
+  bool finalized_ = false;
+  bool graph_created_ = false;
+  NamedIndex tensor_name_index_;
+  std::vector<bool> ready_;
+  bool allow_resized_ = false;
+  IntList default_input_sizes_;
+  void* graph_ = nullptr;       // hipGraph_t
+  void* graph_exec_ = nullptr;  // hipGraphExec_t
+};
+
+}  // namespace opengl
+
+#endif  // OPENGL_CORE_FBO_SESSION_H_

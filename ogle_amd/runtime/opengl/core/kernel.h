@@ -1,0 +1,87 @@
+// Base class of every graph op: the drop-in boundary of the runtime.
+//
+// The virtuals and their call order are those of the reference
+// (ogl_runtime/opengl/core/kernel.h:15-123; driven by FBOSession::Setup/Run,
+// fbo_session.cc:201-245,140-153): Setup -> SetupAttr, then once per session
+// SelectKernel -> (program lookup) -> InferOutputShape, then Compute per run.
+// SelectKernel now names an entry of the HIP kernel registry instead of a GLSL
+// source; kernel_fname() / build_options() keep their meaning as the lookup key.
+#ifndef OPENGL_CORE_KERNEL_H_
+#define OPENGL_CORE_KERNEL_H_
+
+#include <string>
+#include <vector>
+
+#include "opengl/core/dlxnet.h"
+#include "opengl/core/types.h"
+#include "opengl/utils/logging.h"
+
+namespace opengl {
+class Program;
+class FBOSession;
+
+class Kernel {
+ public:
+  explicit Kernel(Context* context);
+  virtual ~Kernel();
+
+  virtual void SetupProgram(Program* program);
+  // Enqueues the op's device work on the context's stream.
+  virtual void Compute(TensorList& inputs, TensorList& outputs) = 0;
+  virtual void SetupAttr(const dlxnet::Attribute& attr) = 0;
+  virtual void Setup(const dlxnet::NodeProto& node_proto, FBOSession* session);
+  void Compute();
+
+  DataFormat GetOutputDFormat(int i) const;
+  DataFormat GetRequestInputDFormat(int i) const;
+  std::string DebugString() const;
+
+  // Output shapes from input shapes; ops that need input values or formats
+  // (Reshape, Concat, Decoder) override the tensor overload instead.
+  virtual void InferOutputShape(TensorShapeList& inputs, TensorShapeList& outputs) = 0;
+  virtual void InferOutputShape(const TensorList& inputs, TensorShapeList& output_shapes);
+
+  void set_kernel_name(const std::string& name) { kernel_name_ = name; }
+  void set_kernel_type(const std::string& name) { kernel_type_ = name; }
+  std::string kernel_name() const { return kernel_name_; }
+  std::string kernel_type() const { return kernel_type_; }
+  void set_session(FBOSession* session) { session_ = session; }
+  FBOSession* session() const { return session_; }
+
+  // A kernel that must run during Setup even though its inputs are not constant
+  // (ShapeKernel in the reference, shape.h:19).
+  virtual bool ForceReady() const { return false; }
+  const std::string kernel_fname() const { return kernel_fname_; }
+  std::string build_options() const { return build_options_; }
+  void set_build_options(const std::string& opt) { build_options_ = opt; }
+  virtual void SelectKernel(const TensorList& inputs) { (void)inputs; }
+
+  // Index of the input whose device buffer output `i` may share (the op is a pure
+  // re-interpretation of dense memory), or -1.  Not in the reference, where every
+  // layout change is a draw call; with linear NHWC buffers Reshape and an identity
+  // Transpose move no data.  Consulted by the executor after InferOutputShape.
+  virtual int OutputAliasesInput(int i) const {
+    (void)i;
+    return -1;
+  }
+
+ protected:
+  Program* program_ = nullptr;  // not owned (the context owns programs)
+  Context* context_;            // not owned
+  std::string kernel_fname_;
+  std::vector<Tensor*> input_tensors_;   // not owned
+  std::vector<Tensor*> output_tensors_;  // not owned
+  std::vector<int> input_tensor_indexes_;
+  std::vector<int> output_tensor_indexes_;
+  std::vector<DataFormat> request_tensor_dformats_;
+  std::vector<DataFormat> output_tensor_dformats_;
+  friend class FBOSession;
+  std::string kernel_name_;
+  std::string kernel_type_;
+  std::string build_options_;
+  FBOSession* session_ = nullptr;
+};
+
+}  // namespace opengl
+
+#endif  // OPENGL_CORE_KERNEL_H_

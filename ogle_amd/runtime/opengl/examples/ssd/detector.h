@@ -1,0 +1,84 @@
+// SSD detector driver: runs the graph, decodes boxes and filters scores on the
+// device, then top-k and NMS on the host.  Counterpart of
+// ogl_runtime/opengl/examples/ssd/detector.{h,cc} without the OpenCV image I/O:
+// the caller passes preprocessed float images (NHWC) and the size the boxes are
+// scaled to.  Unlike the reference, which post-processes the first image only
+// (detector.cc:184), every image of the batch is handled.
+#ifndef OPENGL_EXAMPLES_SSD_DETECTOR_H_
+#define OPENGL_EXAMPLES_SSD_DETECTOR_H_
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "opengl/core/types.h"
+
+namespace opengl {
+
+// Integer rectangle with cv::Rect's fields.
+struct Rect {
+  int x = 0, y = 0, width = 0, height = 0;
+};
+
+// examples/ssd/common.h:29-45 of the reference.
+struct BoxInfo {
+  Rect box;
+  float score = 0.f;
+  float cx = 0.f, cy = 0.f;
+  float width = 0.f, height = 0.f;
+  int class_name = 0;
+  int index = 0;  // prior index
+};
+
+struct DetectorOptions {
+  string model_name;
+  int input_width = 0;
+  int input_height = 0;
+  float nms_threshold = 0.45f;
+  float score_threshold = 0.3f;
+  int topk = 100;
+  std::vector<float> variances = {0.1f, 0.1f, 0.2f, 0.2f};
+  TensorNameList input_names = {"input"};
+  TensorNameList output_names = {"cls_logits", "box_preds", "anchors"};
+};
+
+class FBOSession;
+
+class Detector {
+ public:
+  static std::unique_ptr<Detector> Create(const DetectorOptions& options);
+  // Wraps a session the caller already loaded (not owned).
+  static std::unique_ptr<Detector> Create(FBOSession* session, const DetectorOptions& options);
+  ~Detector();
+
+  // images: host NHWC float tensor, already mean-subtracted and resized
+  // (Preprocess, detector.cc:99-109, is image I/O and stays with the caller).
+  // Boxes are scaled to raw_width x raw_height.  One vector per image.
+  void Detect(const Tensor* images, int raw_width, int raw_height,
+              std::vector<std::vector<BoxInfo>>* final_boxes);
+
+  // The stages, as in the reference.
+  void Run(const Tensor* images);
+  void LoadToOutputTensors(const TensorNameList& names, int raw_width, int raw_height);
+  void GenerateBoxInfo(int image, std::vector<BoxInfo>* box_infos) const;
+  static void GetTopK(std::vector<BoxInfo>& input, int top_k);
+  static void NMS(std::vector<BoxInfo>& boxes, std::vector<BoxInfo>& boxes_left, float threshold);
+
+  FBOSession* session() const { return session_; }
+
+ private:
+  Detector(FBOSession* session, bool owned, const DetectorOptions& options);
+  DetectorOptions options_;
+  FBOSession* session_;
+  bool owns_session_;
+  int batch_ = 0, priors_ = 0, classes_ = 0;
+  // device results of the fused decode + score filter, and their host copies
+  std::unique_ptr<Tensor> boxes_dev_, count_dev_, prior_dev_, class_dev_, score_dev_, box_dev_,
+      rect_dev_;
+  std::vector<int32_t> count_, prior_, class_, rect_;
+  std::vector<float> score_, box_;
+};
+
+float iou(const Rect& box0, const Rect& box1);
+
+}  // namespace opengl
+#endif  // OPENGL_EXAMPLES_SSD_DETECTOR_H_

@@ -1,0 +1,144 @@
+#include "opengl/nn/kernels/conv2d.h"
+
+#include "opengl/core/context.h"
+#include "opengl/core/kernel_registry.h"
+#include "opengl/core/program.h"
+
+namespace opengl {
+
+Conv2DKernel::Conv2DKernel(Context* context) : Kernel(context) {}
+Conv2DKernel::~Conv2DKernel() {}
+
+// Attribute rules of conv2d.cc:67-111: four equal pads, two equal strides, a square
+// kernel; group 0 means 1; one or two equal dilations, default 1.
+void Conv2DKernel::SetupAttr(const dlxnet::Attribute& attr) {
+  const dlxnet::Conv2dAttribute& p = attr.conv2d_attr();
+  CHECK_EQ(p.pads_size(), 4);
+  for (auto pad : p.pads()) CHECK_EQ(p.pads(0), pad);
+  padding_ = static_cast<int>(p.pads(0));
+  CHECK_EQ(p.strides_size(), 2);
+  CHECK_EQ(p.strides(0), p.strides(1));
+  stride_ = static_cast<int>(p.strides(0));
+  CHECK_EQ(p.kernel_shape_size(), 2);
+  CHECK_EQ(p.kernel_shape(0), p.kernel_shape(1));
+  kernel_size_ = static_cast<int>(p.kernel_shape(0));
+  group_size_ = p.group() == 0 ? 1 : static_cast<int>(p.group());
+  if (p.dilations_size() == 2) {
+    CHECK_EQ(p.dilations(0), p.dilations(1));
+    dilation_ = static_cast<int>(p.dilations(0));
+  } else if (p.dilations_size() == 1) {
+    dilation_ = static_cast<int>(p.dilations(0));
+  } else {
+    dilation_ = 1;
+  }
+  activation_type_ = p.activation_type();
+  min_ = p.min();
+  max_ = p.max();
+}
+
+// Variant choice of conv2d.cc:19-65.  The names are the shader stems the registry
+// is keyed by; the *_any4 stems select the same HIP kernels with the any4 reading
+// of min/max for the fused activation.
+void Conv2DKernel::SelectKernel(const TensorList& inputs) {
+  const bool any4 = inputs[0]->dformat() == dlxnet::TensorProto::ANY4;
+  const bool pointwise = kernel_size_ == 1 && group_size_ == 1 && dilation_ == 1 && stride_ == 1 &&
+                         padding_ == 0;
+  if (pointwise) {
+    variant_ = kPointwise;
+    kernel_fname_ = any4 ? "conv2d_pw_any4" : "conv2d_pw";
+  } else if (group_size_ != 1) {
+    const int in_c = inputs[0]->shape()[3];
+    if (any4) {
+      CHECK_EQ(group_size_, in_c);
+      variant_ = kDepthwise;
+      kernel_fname_ = "conv2d_dw_any4";
+    } else if (group_size_ == in_c && group_size_ == inputs[1]->shape()[0]) {
+      variant_ = kDepthwise;
+      kernel_fname_ = "conv2d_dw";
+    } else {
+      variant_ = kGrouped;
+      kernel_fname_ = "conv2d_grp";
+    }
+  } else {
+    variant_ = kDense;
+    kernel_fname_ = any4 ? "conv2d_any4" : "conv2d";
+  }
+  act_variant_ = any4 ? OGLE_VARIANT_ANY4 : (variant_ == kPointwise ? OGLE_VARIANT_PW : OGLE_VARIANT_NHWC4);
+
+  if (input_tensor_indexes_.size() == 3) build_options_ += "#define USE_BIAS\n";
+  if (activation_type_ == "Clip") {
+    build_options_ += "#define USE_CLIP\n";
+  } else if (activation_type_ == "Relu") {
+    build_options_ += "#define USE_RELU\n";
+  }
+  output_tensor_dformats_.emplace_back(inputs[0]->dformat());
+}
+
+void Conv2DKernel::InferOutputShape(TensorShapeList& input_shapes, TensorShapeList& output_shapes) {
+  CHECK(input_shapes.size() == 3 || input_shapes.size() == 2);
+  output_shapes.clear();
+  output_shapes.resize(1);
+  const IntList& image_shape = input_shapes[0];   // (n, h, w, c)
+  const IntList& filter_shape = input_shapes[1];  // (n_out, n_in / group, k, k)
+  CHECK_EQ(image_shape.size(), 4u);
+  CHECK_EQ(filter_shape.size(), 4u);
+  CHECK_EQ(filter_shape[2], kernel_size_);
+  CHECK_EQ(filter_shape[3], kernel_size_);
+  CHECK_EQ(filter_shape[1] * group_size_, image_shape[3]);
+  if (input_shapes.size() == 3) {
+    size_t bias_elems = 1;
+    for (int d : input_shapes[2]) bias_elems *= static_cast<size_t>(d);
+    CHECK_EQ(bias_elems, static_cast<size_t>(filter_shape[0])) << "bias length";
+  }
+  const int kernel_size = kernel_size_ * dilation_ - dilation_ + 1;
+  const int output_height = (image_shape[1] - kernel_size + 2 * padding_) / stride_ + 1;
+  const int output_width = (image_shape[2] - kernel_size + 2 * padding_) / stride_ + 1;
+  output_shapes[0] = {image_shape[0], output_height, output_width, filter_shape[0]};
+}
+
+void Conv2DKernel::PackFilter(const Tensor* filter) {
+  const IntList& fs = filter->shape();
+  const int layout = variant_ == kDepthwise ? OGLE_FILTER_HWC : OGLE_FILTER_OHWI;
+  if (variant_ == kDepthwise) CHECK_EQ(fs[1], 1) << "depthwise filters have one input channel";
+  packed_filter_.reset(new Tensor(Tensor::DT_FLOAT, fs, Tensor::DEVICE_BUFFER, filter->dformat()));
+  const int32_t st =
+      ogle_hip_pack_filter(static_cast<const float*>(filter->device_ptr()), packed_filter_->device_ptr(),
+                           layout, OGLE_F32, fs[0], fs[1], fs[2], fs[3], context_->stream());
+  if (st != OGLE_OK) LOG(FATAL) << "ogle_hip_pack_filter: " << ogle_hip_last_error();
+  packed_from_ = filter->device_ptr();
+}
+
+void Conv2DKernel::Compute(TensorList& inputs, TensorList& outputs) {
+  program_->Activate();
+  const Tensor* image = inputs[0];
+  const Tensor* filter = inputs[1];
+  if (!packed_filter_ || packed_from_ != filter->device_ptr()) PackFilter(filter);
+
+  const IntList& in = image->shape();
+  const IntList& out = outputs[0]->shape();
+  OgleConvArgs a{};
+  a.input_dev = image->device_ptr();
+  a.filter_dev = packed_filter_->device_ptr();
+  a.bias_dev = inputs.size() > 2 ? static_cast<const float*>(inputs[2]->device_ptr()) : nullptr;
+  a.output_dev = outputs[0]->device_ptr();
+  a.n = in[0]; a.in_h = in[1]; a.in_w = in[2]; a.in_c = in[3];
+  a.out_h = out[1]; a.out_w = out[2]; a.out_c = out[3];
+  a.kernel_size = kernel_size_; a.stride = stride_; a.padding = padding_;
+  a.dilation = dilation_; a.group = group_size_;
+  // "act" uniform: 1 clip, otherwise 2 for any non-empty activation (conv2d.cc:137-147).
+  a.act = activation_type_.empty() ? OGLE_ACT_NONE
+                                   : (activation_type_ == "Clip" ? OGLE_ACT_CLIP : OGLE_ACT_RELU);
+  a.min_value = min_;
+  a.max_value = max_;
+  a.act_variant = act_variant_;
+  a.dtype = OGLE_F32;
+  switch (variant_) {
+    case kPointwise: program_->RunPointwise(a); break;
+    case kDepthwise: program_->RunDepthwise(a); break;
+    default: program_->RunConv2d(a); break;
+  }
+}
+
+REGISTER_KERNEL_WITH_NAME(Conv2DKernel, "Conv");
+
+}  // namespace opengl

@@ -1,0 +1,233 @@
+"""ctypes binding of the graph runtime's C ABI (include/ogle_runtime.h).
+
+`Session` mirrors opengl::FBOSession (ogl_runtime/opengl/core/fbo_session.h:11-90):
+load_graph, run, get_outputs, plus the additions of this runtime (compute with
+resident inputs, hipGraph replay, per-node timing) and the SSD Detector.
+"""
+import ctypes
+import os
+
+import numpy as np
+
+from . import hip as _hip
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libogle_runtime.so")
+
+SYMBOLS = [
+    "ogle_rt_last_error", "ogle_rt_session_create", "ogle_rt_session_destroy",
+    "ogle_rt_load_file", "ogle_rt_load_bytes", "ogle_rt_run", "ogle_rt_compute",
+    "ogle_rt_compute_graph", "ogle_rt_sync", "ogle_rt_time_compute", "ogle_rt_profile",
+    "ogle_rt_profile_entry", "ogle_rt_tensor_shape", "ogle_rt_tensor_device_ptr",
+    "ogle_rt_stream", "ogle_rt_get_output", "ogle_rt_num_kernels",
+    "ogle_rt_registered_kernel_count", "ogle_rt_registered_kernel_name", "ogle_rt_detect",
+    "ogle_rt_reserialize", "ogle_rt_model_debug_string", "ogle_rt_tensor_dformat",
+]
+
+
+class Detection(ctypes.Structure):
+    _fields_ = [("image", ctypes.c_int32), ("prior", ctypes.c_int32), ("class_id", ctypes.c_int32),
+                ("score", ctypes.c_float), ("x", ctypes.c_int32), ("y", ctypes.c_int32),
+                ("width", ctypes.c_int32), ("height", ctypes.c_int32), ("cx", ctypes.c_float),
+                ("cy", ctypes.c_float)]
+
+
+class RuntimeError_(RuntimeError):
+    pass
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        _hip.lib()  # the kernels first: fails loudly if they were not built
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError_("%s is missing: build it with `make -C ogle_amd/runtime`" % LIB_PATH)
+        l = ctypes.CDLL(LIB_PATH)
+        vp, i32, i64, cp = ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64, ctypes.c_char_p
+        l.ogle_rt_last_error.restype = cp
+        l.ogle_rt_session_create.restype = vp
+        l.ogle_rt_session_destroy.argtypes = [vp]
+        l.ogle_rt_load_file.argtypes = [vp, cp]
+        l.ogle_rt_load_bytes.argtypes = [vp, vp, ctypes.c_size_t]
+        l.ogle_rt_run.argtypes = [vp, i32, ctypes.POINTER(cp), ctypes.POINTER(vp),
+                                  ctypes.POINTER(ctypes.POINTER(i32)), ctypes.POINTER(i32),
+                                  ctypes.POINTER(cp)]
+        l.ogle_rt_compute.argtypes = [vp]
+        l.ogle_rt_compute_graph.argtypes = [vp]
+        l.ogle_rt_sync.argtypes = [vp]
+        l.ogle_rt_time_compute.argtypes = [vp, i32, i32, i32, ctypes.POINTER(ctypes.c_float),
+                                           ctypes.POINTER(ctypes.c_float)]
+        l.ogle_rt_profile.argtypes = [vp]
+        l.ogle_rt_profile_entry.argtypes = [vp, i32, ctypes.POINTER(cp), ctypes.POINTER(cp),
+                                            ctypes.POINTER(ctypes.c_float)]
+        l.ogle_rt_tensor_shape.argtypes = [vp, cp, ctypes.POINTER(i32)]
+        l.ogle_rt_tensor_dformat.argtypes = [vp, cp]
+        l.ogle_rt_tensor_device_ptr.argtypes = [vp, cp]
+        l.ogle_rt_tensor_device_ptr.restype = vp
+        l.ogle_rt_stream.argtypes = [vp]
+        l.ogle_rt_stream.restype = vp
+        l.ogle_rt_get_output.argtypes = [vp, cp, cp, vp, i64]
+        l.ogle_rt_get_output.restype = i64
+        l.ogle_rt_num_kernels.argtypes = [vp]
+        l.ogle_rt_registered_kernel_name.argtypes = [i32]
+        l.ogle_rt_registered_kernel_name.restype = cp
+        l.ogle_rt_detect.argtypes = [vp, vp, ctypes.POINTER(i32), cp, cp, cp, cp, ctypes.c_float,
+                                     ctypes.c_float, i32, i32, i32, ctypes.POINTER(Detection), i64]
+        l.ogle_rt_detect.restype = i64
+        l.ogle_rt_reserialize.argtypes = [vp, ctypes.c_size_t, vp, i64]
+        l.ogle_rt_reserialize.restype = i64
+        l.ogle_rt_model_debug_string.argtypes = [vp, ctypes.c_size_t, vp, i64]
+        l.ogle_rt_model_debug_string.restype = i64
+        _lib = l
+    return _lib
+
+
+def _check(rc):
+    if rc < 0:
+        raise RuntimeError_(lib().ogle_rt_last_error().decode())
+    return rc
+
+
+def reserialize(model_bytes):
+    """Round trip through the runtime's C++ .dlx codec (parse, then serialize)."""
+    src = ctypes.create_string_buffer(bytes(model_bytes), len(model_bytes))
+    dst = ctypes.create_string_buffer(len(model_bytes) + 1024)
+    n = _check(lib().ogle_rt_reserialize(ctypes.cast(src, ctypes.c_void_p), len(model_bytes),
+                                         ctypes.cast(dst, ctypes.c_void_p), len(dst)))
+    return dst.raw[:n]
+
+
+def model_debug_string(model_bytes):
+    src = ctypes.create_string_buffer(bytes(model_bytes), len(model_bytes))
+    dst = ctypes.create_string_buffer(1 << 22)
+    _check(lib().ogle_rt_model_debug_string(ctypes.cast(src, ctypes.c_void_p), len(model_bytes),
+                                            ctypes.cast(dst, ctypes.c_void_p), len(dst)))
+    return dst.value.decode()
+
+
+def registered_kernels():
+    l = lib()
+    return [l.ogle_rt_registered_kernel_name(i).decode()
+            for i in range(l.ogle_rt_registered_kernel_count())]
+
+
+class Session:
+    def __init__(self):
+        self._h = lib().ogle_rt_session_create()
+        if not self._h:
+            raise RuntimeError_(lib().ogle_rt_last_error().decode())
+
+    def close(self):
+        if self._h:
+            lib().ogle_rt_session_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def load_graph(self, model):
+        """model: a path, serialized bytes, or a dlx.GraphBuilder."""
+        if hasattr(model, "serialize"):
+            model = model.serialize()
+        if isinstance(model, (bytes, bytearray)):
+            buf = ctypes.create_string_buffer(bytes(model), len(model))
+            _check(lib().ogle_rt_load_bytes(self._h, ctypes.cast(buf, ctypes.c_void_p), len(model)))
+        else:
+            _check(lib().ogle_rt_load_file(self._h, str(model).encode()))
+
+    def run(self, inputs, dformats=None):
+        """inputs: {name: float32 ndarray}; dformats: {name: "NHWC"|"NCHW"|"ANY"} (default NHWC
+        for rank 4, ANY otherwise)."""
+        names = list(inputs)
+        arrs = [np.ascontiguousarray(inputs[n], dtype=np.float32) for n in names]
+        n = len(names)
+        c_names = (ctypes.c_char_p * n)(*[s.encode() for s in names])
+        c_data = (ctypes.c_void_p * n)(*[a.ctypes.data for a in arrs])
+        dims = [(ctypes.c_int32 * a.ndim)(*a.shape) for a in arrs]
+        c_dims = (ctypes.POINTER(ctypes.c_int32) * n)(
+            *[ctypes.cast(d, ctypes.POINTER(ctypes.c_int32)) for d in dims])
+        c_ranks = (ctypes.c_int32 * n)(*[a.ndim for a in arrs])
+        fm = [(dformats or {}).get(nm, "NHWC" if a.ndim == 4 else "ANY") for nm, a in zip(names, arrs)]
+        c_fm = (ctypes.c_char_p * n)(*[f.encode() for f in fm])
+        _check(lib().ogle_rt_run(self._h, n, c_names, c_data, c_dims, c_ranks, c_fm))
+
+    def compute(self, graph=False):
+        _check(lib().ogle_rt_compute_graph(self._h) if graph else lib().ogle_rt_compute(self._h))
+
+    def sync(self):
+        _check(lib().ogle_rt_sync(self._h))
+
+    def time_compute(self, warmup, iters, graph=False):
+        """Returns (per-pass ms array, total ms) measured with HIP events on the session stream."""
+        each = (ctypes.c_float * iters)()
+        total = ctypes.c_float(0)
+        _check(lib().ogle_rt_time_compute(self._h, warmup, iters, 1 if graph else 0, each,
+                                          ctypes.byref(total)))
+        return np.array(each[:], np.float64), float(total.value)
+
+    def profile(self):
+        """One pass with per-node events: list of (label, type, ms)."""
+        n = _check(lib().ogle_rt_profile(self._h))
+        out = []
+        label, typ, ms = ctypes.c_char_p(), ctypes.c_char_p(), ctypes.c_float()
+        for i in range(n):
+            _check(lib().ogle_rt_profile_entry(self._h, i, ctypes.byref(label), ctypes.byref(typ),
+                                               ctypes.byref(ms)))
+            out.append((label.value.decode(), typ.value.decode(), float(ms.value)))
+        return out
+
+    def tensor_shape(self, name):
+        dims = (ctypes.c_int32 * 8)()
+        rank = _check(lib().ogle_rt_tensor_shape(self._h, name.encode(), dims))
+        return tuple(dims[:rank])
+
+    def tensor_dformat(self, name):
+        """Layout tag as a string: "NHWC4", "ANY4", "HWN4C4", ..."""
+        from . import dlx
+        return dlx.DFORMAT_NAMES[_check(lib().ogle_rt_tensor_dformat(self._h, name.encode()))]
+
+    def tensor_device_ptr(self, name):
+        return lib().ogle_rt_tensor_device_ptr(self._h, name.encode())
+
+    @property
+    def stream(self):
+        return lib().ogle_rt_stream(self._h)
+
+    @property
+    def num_kernels(self):
+        return lib().ogle_rt_num_kernels(self._h)
+
+    def get_output(self, name, dformat="ANY"):
+        shape = self.tensor_shape(name)
+        out = np.empty(shape, np.float32)
+        if dformat == "NCHW" and len(shape) == 4 and self.tensor_dformat(name) in ("NHWC", "NHWC4"):
+            out = np.empty((shape[0], shape[3], shape[1], shape[2]), np.float32)
+        n = _check(lib().ogle_rt_get_output(self._h, name.encode(), dformat.encode(),
+                                            out.ctypes.data, out.size))
+        assert n == out.size
+        return out
+
+    def get_outputs(self, names, dformats):
+        return [self.get_output(n, f) for n, f in zip(names, dformats)]
+
+    def detect(self, images, raw_width, raw_height, score_threshold=0.3, nms_threshold=0.45,
+               topk=100, input_name=None, output_names=None, capacity=4096):
+        images = np.ascontiguousarray(images, dtype=np.float32)
+        dims = (ctypes.c_int32 * 4)(*images.shape)
+        names = [None, None, None] if output_names is None else [s.encode() for s in output_names]
+        buf = (Detection * capacity)()
+        n = _check(lib().ogle_rt_detect(self._h, images.ctypes.data, dims,
+                                        input_name.encode() if input_name else None, names[0],
+                                        names[1], names[2], score_threshold, nms_threshold, topk,
+                                        raw_width, raw_height, buf, capacity))
+        per_image = [[] for _ in range(images.shape[0])]
+        for d in buf[:min(n, capacity)]:
+            per_image[d.image].append(dict(prior=d.prior, cls=d.class_id, score=d.score,
+                                           rect=(d.x, d.y, d.width, d.height), cx=d.cx, cy=d.cy))
+        return per_image

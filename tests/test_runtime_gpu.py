@@ -1,0 +1,284 @@
+"""GPU tests of the graph runtime: .dlx graphs are loaded into the C++ FBOSession through
+its C ABI, run on the device, read back with GetOutputs and compared with the CPU oracle.
+
+The single-node tests follow the pattern of the reference's kernel tests
+(ogl_runtime/opengl/nn/kernels/conv2d_test.cc:141-204, concat_test.cc:51-95): build a one-node
+graph, Run, fetch the result AND the constants as the device holds them, compare with the
+in-test CPU function (here the oracle)."""
+import numpy as np
+import pytest
+
+import oracle as O
+from ogle_amd import dlx, models, session
+from util import assert_conv_close, rng
+
+pytestmark = pytest.mark.gpu
+
+
+def conv_graph(x_shape, w, b, k, s, p, d=1, g=1, act="", minv=0.0, maxv=0.0):
+    n, h, wd, c = x_shape
+    gb = dlx.GraphBuilder()
+    x = gb.add_input("input", [n, c, h, wd])
+    wi = gb.add_filter("conv2d1.weight", w)
+    bi = gb.add_const("conv2d1.bias", b) if b is not None else None
+    gb.add_conv("output", x, wi, bi, k, s, p, d, g, act, minv, maxv)
+    gb.add_output_name("output")
+    return gb
+
+
+CONV_GRAPH_CASES = [
+    # n, h, w, c, o, k, s, p, d, g, bias, act
+    (1, 3, 3, 3, 1, 3, 1, 1, 1, 1, True, ""),
+    (2, 16, 16, 8, 12, 3, 1, 1, 1, 1, False, "Relu"),
+    (1, 32, 32, 3, 32, 3, 2, 1, 1, 1, True, "Clip"),     # stem-like
+    (2, 9, 9, 16, 16, 3, 1, 1, 1, 16, True, "Clip"),     # depthwise
+    (1, 8, 8, 8, 12, 3, 1, 1, 1, 4, True, ""),           # grouped
+    (3, 7, 7, 32, 48, 1, 1, 0, 1, 1, True, "Clip"),      # pointwise
+    (1, 8, 8, 4, 4, 3, 1, 2, 2, 1, False, ""),           # dilation 2
+    (1, 6, 6, 8, 8, 1, 2, 0, 1, 1, True, "Relu"),        # 1x1 stride 2 -> dense variant
+]
+
+
+@pytest.mark.parametrize("case", CONV_GRAPH_CASES)
+def test_single_conv_node_graph(case):
+    n, h, w, c, o, k, s, p, d, g, use_bias, act = case
+    r = rng(7000 + CONV_GRAPH_CASES.index(case))
+    x = r.uniform(-1, 1, (n, h, w, c)).astype(np.float32)
+    wt = r.normal(0, 0.5, (o, c // g, k, k)).astype(np.float32)
+    b = r.uniform(-0.1, 0.1, o).astype(np.float32) if use_bias else None
+    sess = session.Session()
+    sess.load_graph(conv_graph(x.shape, wt, b, k, s, p, d, g, act, 0.0, 6.0 if act == "Clip" else 0.0))
+    sess.run({"input": x})
+    got = sess.get_output("output", "NHWC")
+    # constants as the device saw them
+    np.testing.assert_array_equal(sess.get_output("conv2d1.weight", "NCHW"), wt)
+    if use_bias:
+        np.testing.assert_array_equal(sess.get_output("conv2d1.bias", "ANY"), b)
+    oact = {"": O.ACT_NONE, "Relu": O.ACT_RELU, "Clip": O.ACT_CLIP}[act]
+    variant = O.VARIANT_PW if (k == 1 and s == 1 and p == 0 and g == 1) else O.VARIANT_NHWC4
+    ref = O.conv2d(x, wt, b, s, p, d, g, oact, 0.0, 6.0, variant)
+    assert_conv_close(got, ref, O.conv2d_abs(x, wt, b, s, p, d, g), 1e-4, str(case))
+    # NCHW readback is the transpose of the NHWC one
+    np.testing.assert_array_equal(sess.get_output("output", "NCHW"), got.transpose(0, 3, 1, 2))
+    # a second Run with new data reuses the allocation
+    x2 = r.uniform(-1, 1, x.shape).astype(np.float32)
+    sess.run({"input": x2})
+    ref2 = O.conv2d(x2, wt, b, s, p, d, g, oact, 0.0, 6.0, variant)
+    assert_conv_close(sess.get_output("output", "NHWC"), ref2, O.conv2d_abs(x2, wt, b, s, p, d, g),
+                      1e-4, "second run")
+    # the input shape is fixed after the first Run
+    with pytest.raises(RuntimeError, match="changed shape"):
+        sess.run({"input": np.zeros((n, h + 1, w, c), np.float32)})
+
+
+@pytest.mark.parametrize("shapes,axis", [
+    (((2, 3, 5), (2, 3, 5)), 0), (((2, 3, 5), (2, 4, 5)), 1), (((2, 3, 5), (2, 3, 7)), 2),
+    (((1, 2, 3, 4), (1, 2, 3, 6)), -1), (((5,), (3,)), 0), (((2, 6), (2, 1)), 1),
+    (((3, 2, 4, 4), (1, 2, 4, 4)), 0),
+])
+def test_concat_of_constants(shapes, axis):
+    """concat_test.cc:51-95: both inputs are Const nodes, Run({}) computes at Setup."""
+    r = rng(7200)
+    a = [r.normal(0, 1, s).astype(np.float32) for s in shapes]
+    gb = dlx.GraphBuilder()
+    ids = [gb.add_const("const%d" % (i + 1), t) for i, t in enumerate(a)]
+    gb.add_concat("output", ids, axis)
+    sess = session.Session()
+    sess.load_graph(gb)
+    sess.run({})
+    np.testing.assert_array_equal(sess.get_output("const1", "ANY"), a[0])
+    np.testing.assert_array_equal(sess.get_output("output", "ANY"), O.concat(a, axis))
+
+
+def test_concat_shape_mismatch_is_fatal():
+    gb = dlx.GraphBuilder()
+    ids = [gb.add_const("a", np.zeros((2, 3), np.float32)), gb.add_const("b", np.zeros((3, 3), np.float32))]
+    gb.add_concat("output", ids, 1)
+    sess = session.Session()
+    sess.load_graph(gb)
+    with pytest.raises(RuntimeError, match="Check failed"):
+        sess.run({})
+
+
+@pytest.mark.parametrize("kind,k,s,p", [("MaxPool", 3, 2, 1), ("MaxPool", 2, 2, 0), ("AveragePool", 3, 1, 1),
+                                        ("GlobalAveragePool", 0, 0, 0)])
+def test_pool_node_graph(kind, k, s, p):
+    r = rng(7300)
+    x = r.normal(0, 1, (2, 14, 14, 12)).astype(np.float32)
+    gb = dlx.GraphBuilder()
+    xi = gb.add_input("input", [2, 12, 14, 14])
+    gb.add_pool("output", xi, kind, k, s, p)
+    sess = session.Session()
+    sess.load_graph(gb)
+    sess.run({"input": x})
+    ptype = {"MaxPool": O.POOL_MAX, "AveragePool": O.POOL_AVG, "GlobalAveragePool": O.POOL_GLOBAL_AVG}[kind]
+    ref = O.pool2d(x, k, s, p, ptype)
+    got = sess.get_output("output", "NHWC")
+    if kind == "GlobalAveragePool":
+        np.testing.assert_allclose(got, ref, rtol=0, atol=1e-6)
+    else:
+        np.testing.assert_array_equal(got, ref)
+
+
+def test_decoder_node_graph():
+    r = rng(7400)
+    batch, hh, ww = 2, 5, 6
+    pred = r.normal(0, 1, (batch, hh * ww, 4)).astype(np.float32)
+    anchors = np.concatenate([r.uniform(.1, .9, (batch, hh, ww, 2)), r.uniform(.05, .5, (batch, hh, ww, 2))],
+                             -1).astype(np.float32)
+    gb = dlx.GraphBuilder()
+    pi = gb.add_const("pred", pred)
+    ai = gb.add_const("anchors", anchors)
+    gb.add_decoder("boxes", pi, ai)
+    sess = session.Session()
+    sess.load_graph(gb)
+    sess.run({})
+    got = sess.get_output("boxes", "ANY")
+    for b in range(batch):
+        ref = O.ssd_decode(pred[b:b + 1], anchors[b].reshape(-1, 4))
+        np.testing.assert_allclose(got[b:b + 1], ref, rtol=0, atol=1e-4)
+    # anchors must be (N, H, W, 4) with H*W == priors (decoder.cc:82-85)
+    gb = dlx.GraphBuilder()
+    gb.add_decoder("boxes", gb.add_const("pred", pred), gb.add_const("anchors", anchors[:, :, :5]))
+    sess = session.Session()
+    sess.load_graph(gb)
+    with pytest.raises(RuntimeError, match="Check failed"):
+        sess.run({})
+
+
+def test_transpose_and_reshape_nodes():
+    r = rng(7500)
+    x = r.normal(0, 1, (2, 5, 4, 6)).astype(np.float32)   # NHWC
+    gb = dlx.GraphBuilder()
+    xi = gb.add_input("input", [2, 6, 5, 4])
+    # ONNX perm over NCHW axes: [0,2,3,1] is the identity on NHWC storage (a view here)
+    t0 = gb.add_transpose("t_identity", xi, [0, 2, 3, 1])
+    shp = gb.add_const("shape", np.array([0, -1, 3], np.float32))
+    gb.add_reshape("view", t0, shp)
+    # ONNX perm [0,1,3,2] over NCHW axes; the output is laid out in the ONNX output axis order
+    gb.add_transpose("t_swap", xi, [0, 1, 3, 2])
+    sess = session.Session()
+    sess.load_graph(gb)
+    sess.run({"input": x})
+    np.testing.assert_array_equal(sess.get_output("t_identity", "ANY"), x)
+    np.testing.assert_array_equal(sess.get_output("view", "ANY"), x.reshape(2, -1, 3))
+    # renamed perm: p -> {0,3,1,2}[p], so [0,1,3,2] -> [0,3,2,1]; out[d] = in[perm[d]]
+    np.testing.assert_array_equal(sess.get_output("t_swap", "ANY"), x.transpose(0, 3, 2, 1))
+    assert sess.tensor_device_ptr("view") == sess.tensor_device_ptr("input")
+
+
+@pytest.mark.parametrize("batch", [1, 8])
+def test_config2_block_through_session(batch):
+    g, w = models.separable_block(batch)
+    x = rng(20240002).uniform(0, 6, (batch, 38, 38, 256)).astype(np.float32)
+    sess = session.Session()
+    sess.load_graph(g)
+    sess.run({"input": x})
+    dw = sess.get_output("dw", "NHWC")
+    pw = sess.get_output("pw", "NHWC")
+    ref1 = O.conv2d(x, w["wd"], w["bd"], 1, 1, 1, 256, O.ACT_CLIP, 0.0, 6.0)
+    assert_conv_close(dw, ref1, O.conv2d_abs(x, w["wd"], w["bd"], 1, 1, 1, 256), 1e-4, "dw")
+    ref2 = O.conv2d(dw, w["wp"], w["bp"], act=O.ACT_CLIP, maxv=6.0, variant=O.VARIANT_PW)
+    assert_conv_close(pw, ref2, O.conv2d_abs(dw, w["wp"], w["bp"]), 1e-4, "pw")
+
+
+def _run_ssd(batch, seed=20240005):
+    g, info = models.mobilenet_v1_ssd(batch, seed=seed, with_weights=True)
+    x = rng(seed + 1).uniform(-1, 1, (batch, 300, 300, 3)).astype(np.float32)
+    sess = session.Session()
+    sess.load_graph(g)
+    sess.run({"input": x})
+    return sess, info, x
+
+
+def test_mobilenet_ssd_every_layer_matches_oracle():
+    """Full MobileNet-v1 SSD 300x300, batch 1: every conv layer is checked against the oracle
+    applied to the DEVICE's input of that layer, so each of the 47 convolutions is held to the
+    fp32 tolerance on its own (errors do not compound across the check)."""
+    sess, info, x = _run_ssd(1)
+    produced = {"input": x}
+    prev = "input"
+    feature_of = {}
+    worst = 0.0
+    for l in info["layers"]:
+        name = l["name"]
+        if name.startswith("head"):
+            src = feature_of[int(name[4])]
+        else:
+            src = prev
+        xin = produced[src]
+        w, b = info["weights"][name]
+        act = O.ACT_CLIP if l["act"] else O.ACT_NONE
+        variant = O.VARIANT_PW if l["kind"] == "pw" else O.VARIANT_NHWC4
+        ref = O.conv2d(xin, w, b, l["stride"], l["pad"], 1, l["group"], act, 0.0, 6.0, variant)
+        got = sess.get_output(name, "NHWC")
+        worst = max(worst, assert_conv_close(got, ref, O.conv2d_abs(xin, w, b, l["stride"], l["pad"], 1,
+                                                                    l["group"]), 1e-4, name))
+        produced[name] = got
+        if not name.startswith("head"):
+            prev = name
+            if name in ("block11.pw", "block13.pw"):
+                feature_of[0 if name == "block11.pw" else 1] = name
+            if name.startswith("extra") and name.endswith(".conv"):
+                feature_of[int(name[5]) + 1] = name
+    loc = sess.get_output("box_preds", "ANY")
+    conf = sess.get_output("cls_logits", "ANY")
+    assert loc.shape == (1, 1917, 4) and conf.shape == (1, 1917, 21)
+    np.testing.assert_array_equal(
+        loc, np.concatenate([produced["head%d.loc" % i].reshape(1, -1, 4) for i in range(6)], 1))
+    np.testing.assert_array_equal(
+        conf, np.concatenate([produced["head%d.conf" % i].reshape(1, -1, 21) for i in range(6)], 1))
+    np.testing.assert_array_equal(sess.get_output("anchors", "ANY"), info["anchors"])
+
+
+def test_graph_replay_equals_eager_batch2():
+    """The captured hipGraph is replayed several times with eager work and synchronisations in
+    between; every replay must reproduce the eager result bit for bit."""
+    sess, info, x = _run_ssd(2, seed=77)
+    eager_loc = sess.get_output("box_preds", "ANY")
+    eager_conf = sess.get_output("cls_logits", "ANY")
+    for i in range(3):
+        sess.compute(graph=True)
+        np.testing.assert_array_equal(sess.get_output("box_preds", "ANY"), eager_loc)
+        np.testing.assert_array_equal(sess.get_output("cls_logits", "ANY"), eager_conf)
+        sess.compute(graph=False)
+        sess.sync()
+    # new input through the normal path, then replay: the graph reads the same buffers
+    x2 = rng(1234).uniform(-1, 1, x.shape).astype(np.float32)
+    sess.run({"input": x2})
+    loc2 = sess.get_output("box_preds", "ANY")
+    assert not np.array_equal(loc2, eager_loc)
+    sess.compute(graph=True)
+    np.testing.assert_array_equal(sess.get_output("box_preds", "ANY"), loc2)
+    # per-node profile covers every live node once
+    prof = sess.profile()
+    assert len(prof) == 47 + 24 + 2 and all(ms >= 0 for _, _, ms in prof)
+    assert prof[0][0] == "conv0#Conv#"
+
+
+def test_detector_matches_oracle_pipeline():
+    """Detector::Detect: graph -> decode + score filter (device) -> top-k -> NMS, against the
+    oracle's restatement of GenerateBoxInfo / GetTopK / NMS fed with the device's own logits and
+    box predictions.  Head weights ~N(0, 0.05) give logits wide enough that priors pass."""
+    batch = 2
+    g, info = models.mobilenet_v1_ssd(batch, seed=31, head_std=0.05)
+    x = rng(32).uniform(-1, 1, (batch, 300, 300, 3)).astype(np.float32)
+    sess = session.Session()
+    sess.load_graph(g)
+    dets = sess.detect(x, 640, 480, 0.3, 0.45, 100)
+    conf = sess.get_output("cls_logits", "ANY")
+    loc = sess.get_output("box_preds", "ANY")
+    boxes = O.ssd_decode(loc, info["anchors"])
+    ora = O.box_info(conf, boxes, 0.3, 640.0, 480.0)
+    total = 0
+    for b in range(batch):
+        keep = O.topk_nms(ora[b]["score"], ora[b]["rect"], 100, 0.45)
+        exp_prior = ora[b]["prior"][keep]
+        got_prior = np.array([d["prior"] for d in dets[b]], np.int32)
+        np.testing.assert_array_equal(got_prior, exp_prior)
+        np.testing.assert_array_equal(np.array([d["cls"] for d in dets[b]], np.int32), ora[b]["cls"][keep])
+        got_rect = np.array([d["rect"] for d in dets[b]], np.int32).reshape(-1, 4)
+        exp_rect = ora[b]["rect"][keep]
+        assert np.abs(got_rect - exp_rect).max(initial=0) <= 1   # 1e-4 in coordinates can move a truncation
+        total += len(got_prior)
+    assert total > 0
