@@ -1,0 +1,193 @@
+#!/usr/bin/env python3
+"""Benchmark of the hot path on one MI355X.
+
+Workload (BASELINE configs[4]): MobileNet-v1 SSD 300x300, fp32, random init, BN folded,
+21 classes, 1917 priors, followed by the SSD decode + score filter.  A step is one pass of
+the whole network over one batch of 16 synthetic images that are already resident in HBM.
+The graph is a .dlx model loaded into the C++ FBOSession; the pass is replayed as a hipGraph.
+
+Printed JSON (one line): images/s at batch 16 (`value`), p50 latency at batch 1, the roofline
+of the dominant kernel family measured with HIP events on the session's stream inside this
+process, a per-family table, and the CPU restatement timed on the host cores.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+import numpy as np  # noqa: E402
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+MFMA_F32_PEAK_TFLOPS = 157.3   # dense fp32 MFMA
+
+METRIC = "MobileNet-SSD 300² images/s (b16) + p50 ms (b1); per-kernel % of roofline"
+
+
+def family_of(layer):
+    return {"pw": "pointwise 1x1 (MFMA implicit GEMM)", "dw": "depthwise 3x3",
+            "dense": "dense 3x3 (MFMA implicit GEMM)"}[layer["kind"]] \
+        if not (layer["kind"] == "dense" and layer["cin"] == 3) else "dense 3x3 stem (direct)"
+
+
+def build_session(batch, seed=20240005):
+    from ogle_amd import models, session
+    g, info = models.mobilenet_v1_ssd(batch, seed=seed)
+    x = np.random.Generator(np.random.PCG64(seed + 1)).uniform(-1, 1, (batch, 300, 300, 3)) \
+        .astype(np.float32)
+    s = session.Session()
+    s.load_graph(g)
+    s.run({"input": x})   # allocates, uploads weights and the input; inputs stay resident
+    s.sync()
+    return s, info
+
+
+def per_family_roofline(sess, info, batch, passes):
+    """Per-node HIP-event durations (averaged over `passes` profiled passes), grouped by kernel
+    family, against the algorithmic FLOPs / bytes of each layer."""
+    acc = {}
+    for _ in range(passes):
+        for label, typ, ms in sess.profile():
+            acc[label] = acc.get(label, 0.0) + ms / passes
+    fams = {}
+    for l in info["layers"]:
+        ms = acc[l["name"] + "#Conv#"]
+        f = fams.setdefault(family_of(l), dict(ms=0.0, flops=0.0, bytes=0.0, launches=0))
+        f["ms"] += ms
+        f["flops"] += l["flops_per_image"] * batch
+        f["bytes"] += l["act_bytes_per_image"] * batch + l["weight_bytes"]
+        f["launches"] += 1
+    out = []
+    for name, f in fams.items():
+        sec = f["ms"] * 1e-3
+        tflops = f["flops"] / sec / 1e12
+        gbs = f["bytes"] / sec / 1e9
+        bound = "hbm" if "depthwise" in name or "stem" in name else "mfma"
+        out.append(dict(kernel=name, launches=f["launches"], ms_per_step=round(f["ms"], 4),
+                        avg_launch_us=round(f["ms"] * 1e3 / f["launches"], 2), bound=bound,
+                        tflops=round(tflops, 2), gbs=round(gbs, 1),
+                        frac=round(gbs / HBM_PEAK_GBS if bound == "hbm" else tflops / MFMA_F32_PEAK_TFLOPS, 4),
+                        flops_per_step=f["flops"], bytes_per_step=f["bytes"]))
+    other = sum(ms for label, ms in acc.items() if not label.endswith("#Conv#"))
+    out.sort(key=lambda d: -d["ms_per_step"])
+    return out, other, sum(acc.values())
+
+
+def cpu_baseline(seed=20240005, images=2, repeats=1):
+    """The oracle (CPU restatement of the reference's arithmetic) on the host cores: every conv
+    layer of the network, concat and the decode + score filter, for `images` images."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import oracle as O
+    from ogle_amd import models
+    _, info = models.mobilenet_v1_ssd(images, seed=seed, with_weights=True)
+    x = np.random.Generator(np.random.PCG64(seed + 1)).uniform(-1, 1, (images, 300, 300, 3)) \
+        .astype(np.float32)
+
+    def one_pass():
+        cur, feats, locs, confs = x, [], [], []
+        for l in info["layers"]:
+            w, b = info["weights"][l["name"]]
+            if l["name"].startswith("head"):
+                y = O.conv2d(feats[int(l["name"][4])], w, b, 1, 1)
+                if l["name"].endswith("loc"):
+                    locs.append(y.reshape(images, -1, 4))
+                else:
+                    confs.append(y.reshape(images, -1, info["num_classes"]))
+                continue
+            cur = O.conv2d(cur, w, b, l["stride"], l["pad"], 1, l["group"], O.ACT_CLIP, 0.0, 6.0,
+                           O.VARIANT_PW if l["kind"] == "pw" else O.VARIANT_NHWC4)
+            if l["name"] in ("block11.pw", "block13.pw") or l["name"].endswith(".conv"):
+                feats.append(cur)
+        loc, conf = O.concat(locs, 1), O.concat(confs, 1)
+        boxes = O.ssd_decode(loc, info["anchors"])
+        return O.box_info(conf, boxes, 0.3, 300.0, 300.0)
+
+    t0 = time.perf_counter()
+    one_pass()  # warm-up (page in, thread pool); also sizes the sample
+    first = time.perf_counter() - t0
+    repeats = max(repeats, int(12.0 / max(first, 1e-3)))  # about 12 s of CPU work
+    t0 = time.perf_counter()
+    for _ in range(repeats):
+        one_pass()
+    dt = time.perf_counter() - t0
+    return dict(value=round(images * repeats / dt, 3), unit="images/s", cores=O.num_threads(),
+                kind="port",
+                sample="%d pass(es) of the full network + decoder over %d image(s), %.1f s of CPU work; "
+                       "C restatement of the shaders' arithmetic, OpenMP over output rows "
+                       "(not the reference under Mesa llvmpipe, which cannot be built here)"
+                       % (repeats, images, dt))
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--batch", type=int, default=16)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--eager", action="store_true", help="launch kernel by kernel instead of a hipGraph")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU; --gpus %d is not supported (every image is "
+              "independent, so more GPUs would each take a slice of the batch)" % args.gpus,
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(2)
+
+    use_graph = not args.eager
+    sess, info = build_session(args.batch)
+    # timed region: K passes (network + decode/score filter), inputs resident, bracketed by syncs
+    sess.time_compute(args.warmup, 0, graph=use_graph, with_detect=True)
+    sess.sync()
+    t0 = time.perf_counter()
+    each, total_ms = sess.time_compute(0, args.steps, graph=use_graph, with_detect=True)
+    sess.sync()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    ms_per_step = wall_ms / args.steps
+    images_per_s = args.batch * args.steps / (wall_ms * 1e-3)
+
+    fams, other_ms, node_sum_ms = per_family_roofline(sess, info, args.batch, passes=10)
+    dom = fams[0]
+    roofline = dict(bound=dom["bound"], kernel=dom["kernel"],
+                    achieved=dom["gbs"] if dom["bound"] == "hbm" else dom["tflops"],
+                    peak=HBM_PEAK_GBS if dom["bound"] == "hbm" else MFMA_F32_PEAK_TFLOPS,
+                    unit="GB/s" if dom["bound"] == "hbm" else "TFLOP/s", frac=dom["frac"],
+                    traffic=None, launches_per_step=dom["launches"],
+                    avg_launch_us=dom["avg_launch_us"],
+                    algorithmic_per_step=dom["flops_per_step"] if dom["bound"] == "mfma" else dom["bytes_per_step"])
+
+    # batch-1 latency: each pass waits for the previous one
+    s1, _ = build_session(1)
+    lat, _ = s1.time_compute(20, 300, graph=use_graph, with_detect=True, sync_each=True)
+    lat_eager, _ = s1.time_compute(5, 100, graph=False, with_detect=True, sync_each=True)
+
+    result = {
+        "metric": METRIC, "value": round(images_per_s, 1), "unit": "images/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "MobileNet-v1-SSD 300x300 fp32, random init, BN folded, 21 classes, "
+                               "1917 priors + SSD decode/score filter (BASELINE configs[4])",
+                   "batch": args.batch, "launch": "hipGraph" if use_graph else "eager",
+                   "inputs": "resident in HBM", "flops_per_image": 2803531136},
+        "p50_ms_b1": round(float(np.percentile(lat, 50)), 4),
+        "p50_ms_b1_eager": round(float(np.percentile(lat_eager, 50)), 4),
+        "event_ms_per_step": round(total_ms / args.steps, 4),
+        "network_tflops": round(2803531136 * args.batch / (ms_per_step * 1e-3) / 1e12, 2),
+        "roofline": roofline,
+        "kernels": fams,
+        "non_conv_ms_per_step": round(other_ms, 4),
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -143,7 +143,15 @@ typedef struct OgleConvArgs {
   float max_value;     /* "max_value" uniform                                 */
   int32_t act_variant; /* OgleActVariant                                      */
   int32_t dtype;       /* OgleDType of input/filter/output; accumulation fp32 */
+  /* Optional scratch for kernels that split the contraction over workgroups (few
+   * output tiles, long K).  NULL / 0 is always valid: the launch then uses a plan
+   * that needs none.  Launches on one stream may share one workspace. */
+  void* workspace_dev;
+  size_t workspace_bytes;
 } OgleConvArgs;
+
+/* Bytes of workspace the fastest plan for `args` would use (0 if it needs none). */
+size_t ogle_hip_conv_workspace_bytes(const OgleConvArgs* args);
 
 /* Dense (group 1) or grouped KxK convolution: conv2d.glsl:29-92,
  * conv2d_grp.glsl:30-123, conv2d_any4.glsl:29-96.  Filter layout OHWI. */

@@ -52,11 +52,15 @@ int32_t ogle_rt_sync(OgleSession* s);
 /*
  * Times `iters` passes (after `warmup` untimed ones) with HIP events recorded on
  * the session's stream; inputs stay resident.  use_graph selects ogle_rt_compute
- * or ogle_rt_compute_graph.  ms_each (may be NULL) receives one duration per pass,
- * each pass bracketed by its own event pair; *total_ms the span of all passes.
+ * or ogle_rt_compute_graph; with_detect appends the SSD decode + score-filter launch
+ * (Detector's device stage, default tensor names and thresholds) to every pass;
+ * sync_each waits for each pass before enqueuing the next (latency mode).
+ * ms_each (may be NULL) receives one duration per pass, each pass bracketed by its
+ * own event pair; *total_ms the span of all passes.
  */
 int32_t ogle_rt_time_compute(OgleSession* s, int32_t warmup, int32_t iters, int32_t use_graph,
-                             float* ms_each, float* total_ms);
+                             int32_t with_detect, int32_t sync_each, float* ms_each,
+                             float* total_ms);
 
 /*
  * One pass with an event pair around every node (the reference's per-node TraceMe

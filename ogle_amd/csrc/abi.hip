@@ -78,6 +78,10 @@ int32_t validate_conv(const OgleConvArgs* a, const char* who) {
     set_error("%s: unknown dtype %d", who, a->dtype);
     return OGLE_ERR_INVALID_ARG;
   }
+  if (a->workspace_dev == nullptr && a->workspace_bytes != 0) {
+    set_error("%s: workspace_bytes without workspace_dev", who);
+    return OGLE_ERR_INVALID_ARG;
+  }
   if (a->act < OGLE_ACT_NONE || a->act > OGLE_ACT_RELU) {
     set_error("%s: unknown activation %d", who, a->act);
     return OGLE_ERR_INVALID_ARG;
@@ -182,6 +186,19 @@ int32_t ogle_hip_convert(const void* src_dev, int32_t src_dtype, void* dst_dev,
       (dst_dtype != OGLE_F32 && dst_dtype != OGLE_F16))
     return fail(OGLE_ERR_INVALID_ARG, "convert: unknown dtype");
   return launch_convert(src_dev, src_dtype, dst_dev, dst_dtype, count, as_stream(stream));
+}
+
+size_t ogle_hip_conv_workspace_bytes(const OgleConvArgs* a) {
+  if (a == nullptr) return 0;
+  OgleConvArgs q = *a;  // a size query needs no buffers: only shapes are validated
+  static char dummy;
+  q.input_dev = q.filter_dev = &dummy;
+  q.output_dev = &dummy;
+  q.workspace_dev = nullptr;
+  q.workspace_bytes = 0;
+  if (validate_conv(&q, "conv_workspace_bytes") != OGLE_OK) return 0;
+  if (q.group == q.in_c && q.group == q.out_c && q.group != 1) return 0;  // depthwise
+  return conv_igemm_workspace_bytes(q);
 }
 
 int32_t ogle_hip_conv2d(const OgleConvArgs* a, ogle_stream_t stream) {

@@ -68,7 +68,8 @@ struct Mma<__half> {
 template <typename T, int BM, int BN, int WM, int WN, int ROWB, bool PW>
 __global__ __launch_bounds__(256) void conv_igemm_kernel(
     ConvGeom g, const T* __restrict__ x, const T* __restrict__ w,
-    const float* __restrict__ bias, T* __restrict__ y, Epilogue ep, int tiles_n) {
+    const float* __restrict__ bias, T* __restrict__ y, Epilogue ep, int tiles_n,
+    float* __restrict__ partial, int slabs_per_split) {
   static_assert(WM * WN == 4, "four waves per workgroup");
   constexpr int WTM = BM / WM, WTN = BN / WN;
   constexpr int TM = WTM / 32, TN = WTN / 32;
@@ -189,12 +190,17 @@ __global__ __launch_bounds__(256) void conv_igemm_kernel(
   const int l32 = lane & 31;
   const int lh = lane >> 5;
 
-  load_slab(0);
+  // Split-K: workgroup z of the grid contracts K slabs [kt_begin, kt_end) only and
+  // leaves its partial sums in `partial`; a second kernel adds the splits in order.
+  const int kt_begin = blockIdx.z * slabs_per_split;
+  const int kt_end = min(g.ktiles, kt_begin + slabs_per_split);
+
+  load_slab(kt_begin);
   store_slab(0);
   __syncthreads();
-  for (int kt = 0; kt < g.ktiles; ++kt) {
-    const int buf = kt & 1;
-    const bool more = kt + 1 < g.ktiles;
+  for (int kt = kt_begin; kt < kt_end; ++kt) {
+    const int buf = (kt - kt_begin) & 1;
+    const bool more = kt + 1 < kt_end;
     if (more) load_slab(kt + 1);
     const unsigned char* pa = lds + buf * STAGE + (wave_m * WTM + l32) * LROW + lh * 16;
     const unsigned char* pb = lds + buf * STAGE + (BM + wave_n * WTN + l32) * LROW + lh * 16;
@@ -216,6 +222,25 @@ __global__ __launch_bounds__(256) void conv_igemm_kernel(
     __syncthreads();
   }
 
+  if (partial != nullptr) {
+    float* dst = partial + (long)blockIdx.z * g.m_total * g.o;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int col = n0 + wave_n * WTN + j * 32 + l32;
+      if (col >= g.o) continue;
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const int rbase = m0 + wave_m * WTM + i * 32 + lh * 4;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int row = rbase + (r >> 2) * 8 + (r & 3);
+          if (row < g.m_total) dst[(long)row * g.o + col] = acc[i][j][r];
+        }
+      }
+    }
+    return;
+  }
+
   // Epilogue: bias, activation, store.
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
@@ -235,46 +260,135 @@ __global__ __launch_bounds__(256) void conv_igemm_kernel(
   }
 }
 
+// Sums the split-K partials in split order, then bias and activation.
+template <typename T>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial,
+                                                            const float* __restrict__ bias,
+                                                            T* __restrict__ y, long mn, int o,
+                                                            int splits, Epilogue ep) {
+  for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < mn;
+       idx += (long)gridDim.x * blockDim.x) {
+    float acc = partial[idx];
+    for (int z = 1; z < splits; ++z) acc += partial[(long)z * mn + idx];
+    if (bias != nullptr) acc += bias[idx % o];
+    y[idx] = from_f32<T>(apply_epilogue(acc, ep));
+  }
+}
+
+// Tile configurations (BM, BN, waves along M, waves along N).
+enum TileCfg { CFG_128x128 = 0, CFG_128x64 = 1, CFG_64x64 = 2, CFG_128x32 = 3 };
+constexpr int kCfgBM[] = {128, 128, 64, 128};
+constexpr int kCfgBN[] = {128, 64, 64, 32};
+
+struct IgemmPlan {
+  int cfg;
+  int splits;
+  int slabs_per_split;
+  int ktiles;
+  int cchunks;
+  size_t workspace_bytes;  // splits * M * N floats when splits > 1
+};
+
+constexpr long kComputeUnits = 256;
+
+// Picks the output tile and the K split.  Large problems get the largest tile that
+// still yields about two workgroups per compute unit; problems with few output
+// tiles but a long contraction (the SSD heads, the small feature maps) are split
+// along K until the grid fills the chip, provided a workspace was supplied.
+IgemmPlan plan_igemm(const OgleConvArgs& a, long m, bool allow_split) {
+  IgemmPlan p{};
+  const int esz = a.dtype == OGLE_F16 ? 2 : 4;
+  const int rowb = a.dtype == OGLE_F16 ? 128 : 64;
+  const int epr = rowb / esz;
+  p.cchunks = (a.in_c + epr - 1) / epr;
+  p.ktiles = a.kernel_size * a.kernel_size * p.cchunks;
+  auto tiles = [&](int cfg) {
+    return ((m + kCfgBM[cfg] - 1) / kCfgBM[cfg]) * ((a.out_c + kCfgBN[cfg] - 1) / kCfgBN[cfg]);
+  };
+  if (a.out_c <= 32) {
+    p.cfg = CFG_128x32;
+  } else if (a.out_c <= 64) {
+    p.cfg = tiles(CFG_128x64) >= 2 * kComputeUnits ? CFG_128x64 : CFG_64x64;
+  } else if (tiles(CFG_128x128) >= 2 * kComputeUnits) {
+    p.cfg = CFG_128x128;
+  } else if (tiles(CFG_128x64) >= kComputeUnits) {
+    p.cfg = CFG_128x64;
+  } else {
+    p.cfg = CFG_64x64;
+  }
+  p.splits = 1;
+  const long t = tiles(p.cfg);
+  if (allow_split && 2 * t <= kComputeUnits && p.ktiles >= 8) {
+    long want = (3 * kComputeUnits + t - 1) / t;   // about three workgroups per unit
+    long most = p.ktiles / 4;                      // at least four slabs per split
+    long sp = want < most ? want : most;
+    if (sp > 64) sp = 64;
+    if (sp >= 2) p.splits = (int)sp;
+  }
+  p.slabs_per_split = (p.ktiles + p.splits - 1) / p.splits;
+  p.splits = (p.ktiles + p.slabs_per_split - 1) / p.slabs_per_split;  // no empty split
+  p.workspace_bytes = p.splits > 1 ? (size_t)p.splits * (size_t)m * a.out_c * sizeof(float) : 0;
+  return p;
+}
+
 template <typename T, int BM, int BN, int WM, int WN, int ROWB, bool PW>
-int32_t launch_cfg(const ConvGeom& g0, const OgleConvArgs& a, hipStream_t s) {
+int32_t launch_cfg(const ConvGeom& g0, const OgleConvArgs& a, const IgemmPlan& p, hipStream_t s) {
   ConvGeom g = g0;
-  constexpr int EPR = ROWB / (int)sizeof(T);
-  g.cchunks = (g.c + EPR - 1) / EPR;
-  g.ktiles = g.k * g.k * g.cchunks;
+  g.cchunks = p.cchunks;
+  g.ktiles = p.ktiles;
   const int tiles_m = (g.m_total + BM - 1) / BM;
   const int tiles_n = (g.o + BN - 1) / BN;
   const Epilogue ep = make_epilogue(a.act, a.min_value, a.max_value, a.act_variant);
+  float* partial = p.splits > 1 ? static_cast<float*>(a.workspace_dev) : nullptr;
   hipLaunchKernelGGL((conv_igemm_kernel<T, BM, BN, WM, WN, ROWB, PW>),
-                     dim3((unsigned)(tiles_m * tiles_n)), dim3(256), 0, s, g,
+                     dim3((unsigned)(tiles_m * tiles_n), 1, (unsigned)p.splits), dim3(256), 0, s, g,
                      static_cast<const T*>(a.input_dev), static_cast<const T*>(a.filter_dev),
-                     a.bias_dev, static_cast<T*>(a.output_dev), ep, tiles_n);
-  return check_launch("conv_igemm");
+                     a.bias_dev, static_cast<T*>(a.output_dev), ep, tiles_n, partial,
+                     p.slabs_per_split);
+  int32_t st = check_launch("conv_igemm");
+  if (st != OGLE_OK || p.splits == 1) return st;
+  const long mn = (long)g.m_total * g.o;
+  long blocks = (mn + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  hipLaunchKernelGGL((splitk_reduce_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, s, partial,
+                     a.bias_dev, static_cast<T*>(a.output_dev), mn, g.o, p.splits, ep);
+  return check_launch("splitk_reduce");
 }
 
 template <typename T, int ROWB, bool PW>
-int32_t pick_tile(const ConvGeom& g, const OgleConvArgs& a, hipStream_t s) {
-  const long m = g.m_total;
-  auto tiles = [&](int bm, int bn) { return ((m + bm - 1) / bm) * ((g.o + bn - 1) / bn); };
-  constexpr long kFill = 256;  // compute units
-  if (g.o <= 32) return launch_cfg<T, 128, 32, 4, 1, ROWB, PW>(g, a, s);
-  if (g.o <= 64) {
-    if (tiles(128, 64) >= 2 * kFill) return launch_cfg<T, 128, 64, 2, 2, ROWB, PW>(g, a, s);
-    return launch_cfg<T, 64, 64, 2, 2, ROWB, PW>(g, a, s);
+int32_t launch_plan(const ConvGeom& g, const OgleConvArgs& a, const IgemmPlan& p, hipStream_t s) {
+  switch (p.cfg) {
+    case CFG_128x128: return launch_cfg<T, 128, 128, 2, 2, ROWB, PW>(g, a, p, s);
+    case CFG_128x64: return launch_cfg<T, 128, 64, 2, 2, ROWB, PW>(g, a, p, s);
+    case CFG_64x64: return launch_cfg<T, 64, 64, 2, 2, ROWB, PW>(g, a, p, s);
+    default: return launch_cfg<T, 128, 32, 4, 1, ROWB, PW>(g, a, p, s);
   }
-  if (tiles(128, 128) >= 2 * kFill) return launch_cfg<T, 128, 128, 2, 2, ROWB, PW>(g, a, s);
-  if (tiles(128, 64) >= kFill) return launch_cfg<T, 128, 64, 2, 2, ROWB, PW>(g, a, s);
-  return launch_cfg<T, 64, 64, 2, 2, ROWB, PW>(g, a, s);
+}
+
+bool igemm_eligible(const OgleConvArgs& a, long* m_out) {
+  if (a.group != 1) return false;
+  const int ve = a.dtype == OGLE_F16 ? 8 : 4;
+  if (a.in_c % ve != 0) return false;
+  if ((long)a.kernel_size * a.kernel_size * a.in_c < 32) return false;
+  const long m = (long)a.n * a.out_h * a.out_w;
+  if (m <= 0 || m > 0x7fffffffL) return false;
+  *m_out = m;
+  return true;
 }
 
 }  // namespace
 
+size_t conv_igemm_workspace_bytes(const OgleConvArgs& a) {
+  long m = 0;
+  if (!igemm_eligible(a, &m)) return 0;
+  return plan_igemm(a, m, true).workspace_bytes;
+}
+
 int32_t launch_conv_igemm(const OgleConvArgs& a, hipStream_t s) {
-  if (a.group != 1) return OGLE_ERR_UNSUPPORTED;
-  const int ve = a.dtype == OGLE_F16 ? 8 : 4;
-  if (a.in_c % ve != 0) return OGLE_ERR_UNSUPPORTED;
-  if ((long)a.kernel_size * a.kernel_size * a.in_c < 32) return OGLE_ERR_UNSUPPORTED;
-  const long m = (long)a.n * a.out_h * a.out_w;
-  if (m <= 0 || m > 0x7fffffffL) return OGLE_ERR_UNSUPPORTED;
+  long m = 0;
+  if (!igemm_eligible(a, &m)) return OGLE_ERR_UNSUPPORTED;
+  IgemmPlan p = plan_igemm(a, m, a.workspace_dev != nullptr);
+  if (p.workspace_bytes > a.workspace_bytes) p = plan_igemm(a, m, false);  // workspace too small
   ConvGeom g{};
   g.n = a.n; g.h = a.in_h; g.w = a.in_w; g.c = a.in_c;
   g.oh = a.out_h; g.ow = a.out_w; g.o = a.out_c;
@@ -282,9 +396,9 @@ int32_t launch_conv_igemm(const OgleConvArgs& a, hipStream_t s) {
   g.m_total = (int)m;
   const bool pw = a.kernel_size == 1 && a.stride == 1 && a.padding == 0;
   if (a.dtype == OGLE_F16) {
-    return pw ? pick_tile<__half, 128, true>(g, a, s) : pick_tile<__half, 128, false>(g, a, s);
+    return pw ? launch_plan<__half, 128, true>(g, a, p, s) : launch_plan<__half, 128, false>(g, a, p, s);
   }
-  return pw ? pick_tile<float, 64, true>(g, a, s) : pick_tile<float, 64, false>(g, a, s);
+  return pw ? launch_plan<float, 64, true>(g, a, p, s) : launch_plan<float, 64, false>(g, a, p, s);
 }
 
 }  // namespace ogle

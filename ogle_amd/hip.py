@@ -25,7 +25,7 @@ SYMBOLS = [
     "ogle_hip_sync", "ogle_hip_packed_filter_elems", "ogle_hip_pack_filter",
     "ogle_hip_convert", "ogle_hip_conv2d", "ogle_hip_dwconv2d", "ogle_hip_pwconv_gemm",
     "ogle_hip_pool2d", "ogle_hip_concat", "ogle_hip_ssd_decode", "ogle_hip_ssd_detect",
-    "ogle_hip_expf", "ogle_hip_transpose",
+    "ogle_hip_expf", "ogle_hip_transpose", "ogle_hip_conv_workspace_bytes",
 ]
 
 
@@ -46,6 +46,7 @@ class ConvArgs(ctypes.Structure):
         ("padding", ctypes.c_int32), ("dilation", ctypes.c_int32), ("group", ctypes.c_int32),
         ("act", ctypes.c_int32), ("min_value", ctypes.c_float), ("max_value", ctypes.c_float),
         ("act_variant", ctypes.c_int32), ("dtype", ctypes.c_int32),
+        ("workspace_dev", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
     ]
 
 
@@ -128,6 +129,8 @@ def lib():
                           ("ogle_hip_ssd_detect", DetectArgs),
                           ("ogle_hip_transpose", TransposeArgs)):
             getattr(l, name).argtypes = [ctypes.POINTER(typ), ctypes.c_void_p]
+        l.ogle_hip_conv_workspace_bytes.argtypes = [ctypes.POINTER(ConvArgs)]
+        l.ogle_hip_conv_workspace_bytes.restype = ctypes.c_size_t
         l.ogle_hip_expf.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64,
                                     ctypes.c_void_p]
         _lib = l
@@ -166,4 +169,4 @@ def conv_args(x_ptr, w_ptr, b_ptr, y_ptr, n, h, w, c, o, k, stride=1, pad=0, dil
               act=ACT_NONE, minv=0.0, maxv=0.0, variant=VARIANT_NHWC4, dtype=F32):
     return ConvArgs(x_ptr, w_ptr, b_ptr, y_ptr, n, h, w, c,
                     out_size(h, k, stride, pad, dilation), out_size(w, k, stride, pad, dilation), o,
-                    k, stride, pad, dilation, group, act, minv, maxv, variant, dtype)
+                    k, stride, pad, dilation, group, act, minv, maxv, variant, dtype, None, 0)

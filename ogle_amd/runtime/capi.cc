@@ -126,9 +126,12 @@ int32_t ogle_rt_sync(OgleSession* s) {
 }
 
 int32_t ogle_rt_time_compute(OgleSession* s, int32_t warmup, int32_t iters, int32_t use_graph,
-                             float* ms_each, float* total_ms) {
+                             int32_t with_detect, int32_t sync_each, float* ms_each,
+                             float* total_ms) {
   return (int32_t)Guard([&]() -> int64_t {
     hipStream_t st = static_cast<hipStream_t>(s->context->stream());
+    opengl::DetectorOptions opt;
+    if (with_detect && !s->detector) s->detector = opengl::Detector::Create(s->session.get(), opt);
     auto pass = [&]() {
       if (use_graph) {
         if (!s->session->graph_captured()) s->session->CaptureGraph();
@@ -136,6 +139,8 @@ int32_t ogle_rt_time_compute(OgleSession* s, int32_t warmup, int32_t iters, int3
       } else {
         s->session->Compute();
       }
+      if (with_detect) s->detector->EnqueuePostprocess(opt.output_names, 300, 300);
+      if (sync_each) s->context->Finish();
     };
     for (int i = 0; i < warmup; ++i) pass();
     s->context->Finish();

@@ -23,7 +23,22 @@ void* Context::stream() {
   return stream_;
 }
 
+void* Context::Workspace(size_t bytes) {
+  if (bytes <= workspace_bytes_) return workspace_;
+  if (workspace_ != nullptr) {
+    Finish();  // earlier launches may still be using the old buffer
+    (void)hipFree(workspace_);
+    workspace_ = nullptr;
+    workspace_bytes_ = 0;
+  }
+  const size_t rounded = (bytes + (1u << 20) - 1) & ~((size_t(1) << 20) - 1);
+  OGLE_HIP_CALL(hipMalloc(&workspace_, rounded));
+  workspace_bytes_ = rounded;
+  return workspace_;
+}
+
 Context::~Context() {
+  if (workspace_ != nullptr) (void)hipFree(workspace_);
   if (stream_ != nullptr) (void)hipStreamDestroy(static_cast<hipStream_t>(stream_));
 }
 

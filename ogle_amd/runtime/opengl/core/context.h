@@ -33,11 +33,19 @@ class Context {
   // Device -> host, converting to the host tensor's dformat; synchronises.
   void CopyDeviceTensorToCPU(const Tensor* device_tensor, Tensor* cpu_tensor);
 
+  // Scratch memory shared by every kernel launched on this context's stream (they
+  // run one after the other).  Grows on demand; the pointer is stable once every
+  // kernel of a session has run once.
+  void* Workspace(size_t bytes);
+  size_t workspace_bytes() const { return workspace_bytes_; }
+
   void Finish();  // glFinish: waits for the stream
   void Reset() {}
 
  private:
   void* stream_ = nullptr;
+  void* workspace_ = nullptr;
+  size_t workspace_bytes_ = 0;
   std::map<std::string, std::unique_ptr<Program>> programs_;
 };
 

@@ -40,6 +40,11 @@ void Detector::Run(const Tensor* images) {
 // filter of GenerateBoxInfo (detector.cc:184-225) in one device launch, then one
 // readback of the compacted results.
 void Detector::LoadToOutputTensors(const TensorNameList& names, int raw_width, int raw_height) {
+  EnqueuePostprocess(names, raw_width, raw_height);
+  Readback();
+}
+
+void Detector::EnqueuePostprocess(const TensorNameList& names, int raw_width, int raw_height) {
   CHECK_EQ(names.size(), 3u);
   Tensor* cls_logits = session_->FindTensorByName(names[0]);
   Tensor* box_preds = session_->FindTensorByName(names[1]);
@@ -96,6 +101,11 @@ void Detector::LoadToOutputTensors(const TensorNameList& names, int raw_width, i
   hipStream_t s = static_cast<hipStream_t>(session_->context()->stream());
   const int32_t st = ogle_hip_ssd_detect(&a, s);
   if (st != OGLE_OK) LOG(FATAL) << "ogle_hip_ssd_detect: " << ogle_hip_last_error();
+}
+
+void Detector::Readback() {
+  CHECK(batch_ > 0) << "EnqueuePostprocess first";
+  hipStream_t s = static_cast<hipStream_t>(session_->context()->stream());
   auto back = [&](void* dst, const Tensor* src, size_t bytes) {
     const hipError_t e = hipMemcpyAsync(dst, src->device_ptr(), bytes, hipMemcpyDeviceToHost, s);
     if (e != hipSuccess) LOG(FATAL) << "readback: " << hipGetErrorString(e);

@@ -59,6 +59,10 @@ class Detector {
   // The stages, as in the reference.
   void Run(const Tensor* images);
   void LoadToOutputTensors(const TensorNameList& names, int raw_width, int raw_height);
+  // The two halves of LoadToOutputTensors: the device launch (asynchronous, buffers
+  // allocated on first use) and the readback of its compacted results (synchronises).
+  void EnqueuePostprocess(const TensorNameList& names, int raw_width, int raw_height);
+  void Readback();
   void GenerateBoxInfo(int image, std::vector<BoxInfo>* box_infos) const;
   static void GetTopK(std::vector<BoxInfo>& input, int top_k);
   static void NMS(std::vector<BoxInfo>& boxes, std::vector<BoxInfo>& boxes_left, float threshold);

@@ -132,6 +132,11 @@ void Conv2DKernel::Compute(TensorList& inputs, TensorList& outputs) {
   a.max_value = max_;
   a.act_variant = act_variant_;
   a.dtype = OGLE_F32;
+  if (workspace_need_ < 0) workspace_need_ = static_cast<long>(ogle_hip_conv_workspace_bytes(&a));
+  if (workspace_need_ > 0) {
+    a.workspace_dev = context_->Workspace(static_cast<size_t>(workspace_need_));
+    a.workspace_bytes = static_cast<size_t>(workspace_need_);
+  }
   switch (variant_) {
     case kPointwise: program_->RunPointwise(a); break;
     case kDepthwise: program_->RunDepthwise(a); break;

@@ -38,6 +38,7 @@ class Conv2DKernel : public Kernel {
   // constant the first time the node computes.
   std::unique_ptr<Tensor> packed_filter_;
   const void* packed_from_ = nullptr;
+  long workspace_need_ = -1;  // bytes of scratch the launch plan wants; -1 until asked
 };
 
 }  // namespace opengl

@@ -18,8 +18,13 @@ class DecoderKernel : public Kernel {
   void SelectKernel(const TensorList& inputs) override;
 
  private:
-  float score_threshold_;
-  float nms_threshold_;
+  float score_threshold_;  // kept for parity with the reference's fields; the score
+  float nms_threshold_;    // filter and NMS run in the Detector, not in this op
+ public:
+  float score_threshold() const { return score_threshold_; }
+  float nms_threshold() const { return nms_threshold_; }
+
+ private:
   std::vector<float> variances_;
 };
 

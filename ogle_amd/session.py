@@ -58,7 +58,8 @@ def lib():
         l.ogle_rt_compute.argtypes = [vp]
         l.ogle_rt_compute_graph.argtypes = [vp]
         l.ogle_rt_sync.argtypes = [vp]
-        l.ogle_rt_time_compute.argtypes = [vp, i32, i32, i32, ctypes.POINTER(ctypes.c_float),
+        l.ogle_rt_time_compute.argtypes = [vp, i32, i32, i32, i32, i32,
+                                           ctypes.POINTER(ctypes.c_float),
                                            ctypes.POINTER(ctypes.c_float)]
         l.ogle_rt_profile.argtypes = [vp]
         l.ogle_rt_profile_entry.argtypes = [vp, i32, ctypes.POINTER(cp), ctypes.POINTER(cp),
@@ -163,11 +164,14 @@ class Session:
     def sync(self):
         _check(lib().ogle_rt_sync(self._h))
 
-    def time_compute(self, warmup, iters, graph=False):
-        """Returns (per-pass ms array, total ms) measured with HIP events on the session stream."""
+    def time_compute(self, warmup, iters, graph=False, with_detect=False, sync_each=False):
+        """Returns (per-pass ms array, total ms) measured with HIP events on the session stream.
+        with_detect appends the SSD decode + score-filter launch to every pass; sync_each waits
+        for each pass before the next is enqueued (per-pass latency instead of throughput)."""
         each = (ctypes.c_float * iters)()
         total = ctypes.c_float(0)
-        _check(lib().ogle_rt_time_compute(self._h, warmup, iters, 1 if graph else 0, each,
+        _check(lib().ogle_rt_time_compute(self._h, warmup, iters, 1 if graph else 0,
+                                          1 if with_detect else 0, 1 if sync_each else 0, each,
                                           ctypes.byref(total)))
         return np.array(each[:], np.float64), float(total.value)
 

@@ -42,8 +42,9 @@ def pack_filter(w_oihw, layout, dtype=H.F32):
 
 
 def gpu_conv(x, w, b=None, stride=1, pad=0, dilation=1, groups=1, act=H.ACT_NONE, minv=0.0,
-             maxv=0.0, variant=H.VARIANT_NHWC4, dtype=H.F32, entry=None):
-    """x NHWC numpy, w OIHW numpy.  Returns NHWC numpy fp32."""
+             maxv=0.0, variant=H.VARIANT_NHWC4, dtype=H.F32, entry=None, workspace=True):
+    """x NHWC numpy, w OIHW numpy.  Returns NHWC numpy fp32.  With workspace=True the launch gets
+    the scratch buffer ogle_hip_conv_workspace_bytes asks for (enables the split-K plans)."""
     torch = _torch()
     tdt = torch.float16 if dtype == H.F16 else torch.float32
     n, h, wd, c = x.shape
@@ -65,6 +66,12 @@ def gpu_conv(x, w, b=None, stride=1, pad=0, dilation=1, groups=1, act=H.ACT_NONE
     args = H.conv_args(xd.data_ptr(), wdv.data_ptr(), bd.data_ptr() if bd is not None else None,
                        y.data_ptr(), n, h, wd, c, o, k, stride, pad, dilation, groups, act, minv,
                        maxv, variant, dtype)
+    ws = None
+    if workspace:
+        need = H.lib().ogle_hip_conv_workspace_bytes(ctypes.byref(args))
+        if need:
+            ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+            args.workspace_dev, args.workspace_bytes = ws.data_ptr(), need
     H.check(getattr(H.lib(), entry)(ctypes.byref(args), stream_ptr()))
     torch.cuda.synchronize()
     return y.float().cpu().numpy()
