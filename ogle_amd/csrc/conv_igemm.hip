@@ -42,6 +42,8 @@ struct ConvGeom {
   int m_total;   // n*oh*ow
   int cchunks;   // K slabs per tap
   int ktiles;    // taps * cchunks
+  unsigned x_bytes;  // size of the input tensor (buffer-load range)
+  unsigned w_bytes;  // size of the packed filter
 };
 
 template <typename T>
@@ -65,6 +67,17 @@ struct Mma<__half> {
   }
 };
 
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+// Offset that is out of range for every operand (operands are kept below 2 GiB), so
+// a buffer load at it returns zeros: this is how padding taps, rows past the end of
+// the problem and the K tail are zero filled without a branch.
+constexpr unsigned kOutOfRange = 0x80000000u;
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, unsigned bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+
 template <typename T, int BM, int BN, int WM, int WN, int ROWB, bool PW>
 __global__ __launch_bounds__(256) void conv_igemm_kernel(
     ConvGeom g, const T* __restrict__ x, const T* __restrict__ w,
@@ -79,12 +92,11 @@ __global__ __launch_bounds__(256) void conv_igemm_kernel(
   constexpr int AP = (BM + RPP - 1) / RPP, BP = (BN + RPP - 1) / RPP;
   constexpr bool A_PART = BM % RPP != 0, B_PART = BN % RPP != 0;  // last pass partly idle
   constexpr int LROW = ROWB + 16;      // padded LDS row, bytes
-  constexpr int VE = 16 / (int)sizeof(T);    // elements per vector
-  constexpr int EPR = ROWB / (int)sizeof(T); // elements per row per slab
+  constexpr int ESZ = (int)sizeof(T);
   constexpr int CHUNKS = ROWB / 32;
-
-  __shared__ __attribute__((aligned(16))) unsigned char lds[2 * (BM + BN) * LROW];
   constexpr int STAGE = (BM + BN) * LROW;  // one buffer: A rows then B rows
+
+  __shared__ __attribute__((aligned(16))) unsigned char lds[2 * STAGE];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -100,16 +112,18 @@ __global__ __launch_bounds__(256) void conv_igemm_kernel(
   const int vcol = tid % VPR;   // which 16-byte vector of the slab row
   const int vrow = tid / VPR;   // row within a pass
 
-  // Per-pass source rows of this thread.
-  long a_base[AP];   // PW: element offset of the row; KxK: image base offset
+  const __amdgpu_buffer_rsrc_t rx = make_rsrc(x, g.x_bytes);
+  const __amdgpu_buffer_rsrc_t rw = make_rsrc(w, g.w_bytes);
+
+  // Per-pass source rows of this thread, as byte offsets into the operands.
+  unsigned a_base[AP];  // PW: row offset; KxK: offset of the image the row lies in
   int a_iy[AP], a_ix[AP];
-  bool a_ok[AP];
 #pragma unroll
   for (int p = 0; p < AP; ++p) {
     const int m = m0 + p * RPP + vrow;
-    a_ok[p] = m < g.m_total && (!A_PART || p * RPP + vrow < BM);
+    const bool ok = m < g.m_total && (!A_PART || p * RPP + vrow < BM);
     if (PW) {
-      a_base[p] = (long)m * g.c;
+      a_base[p] = ok ? (unsigned)m * (unsigned)(g.c * ESZ) : kOutOfRange;
       a_iy[p] = 0;
       a_ix[p] = 0;
     } else {
@@ -117,67 +131,69 @@ __global__ __launch_bounds__(256) void conv_igemm_kernel(
       const int t = m / g.ow;
       const int oy = t % g.oh;
       const int b = t / g.oh;
-      a_base[p] = (long)b * g.h * g.w * g.c;
-      a_iy[p] = oy * g.stride - g.pad;
+      a_base[p] = (unsigned)b * (unsigned)(g.h * g.w * g.c * ESZ);
+      // a row that does not exist fails every in-image test below
+      a_iy[p] = ok ? oy * g.stride - g.pad : -0x40000000;
       a_ix[p] = ox * g.stride - g.pad;
     }
   }
-  const long ktot = (long)g.k * g.k * g.c;
-  long b_base[BP];
-  bool b_ok[BP];
+  const unsigned krow_bytes = (unsigned)(g.k * g.k * g.c * ESZ);
+  unsigned b_base[BP];
 #pragma unroll
   for (int p = 0; p < BP; ++p) {
     const int o = n0 + p * RPP + vrow;
-    b_ok[p] = o < g.o && (!B_PART || p * RPP + vrow < BN);
-    b_base[p] = (long)o * ktot;
+    const bool ok = o < g.o && (!B_PART || p * RPP + vrow < BN);
+    b_base[p] = ok ? (unsigned)o * krow_bytes : kOutOfRange;
   }
 
-  uint4 ra[AP], rb[BP];
-  const uint4 zero = make_uint4(0, 0, 0, 0);
+  u32x4 ra[AP], rb[BP];
 
-  auto load_slab = [&](int kt) {
-    int tap = 0, cc = kt;
-    if (!PW) {
-      tap = kt / g.cchunks;
-      cc = kt - tap * g.cchunks;
-    }
-    const int c0 = cc * EPR + vcol * VE;
-    const bool c_ok = c0 < g.c;
-    int dy = 0, dx = 0;
-    if (!PW) {
-      const int ky = tap / g.k;
-      dy = ky * g.dil;
-      dx = (tap - ky * g.k) * g.dil;
-    }
-#pragma unroll
-    for (int p = 0; p < AP; ++p) {
-      bool ok = a_ok[p] && c_ok;
-      long off;
-      if (PW) {
-        off = a_base[p] + c0;
-      } else {
-        const int iy = a_iy[p] + dy, ix = a_ix[p] + dx;
-        ok = ok && iy >= 0 && iy < g.h && ix >= 0 && ix < g.w;
-        off = a_base[p] + ((long)iy * g.w + ix) * g.c + c0;
-      }
-      ra[p] = ok ? *reinterpret_cast<const uint4*>(x + off) : zero;
-    }
-#pragma unroll
-    for (int p = 0; p < BP; ++p) {
-      const bool ok = b_ok[p] && c_ok;
-      rb[p] = ok ? *reinterpret_cast<const uint4*>(w + b_base[p] + (long)tap * g.c + c0) : zero;
-    }
-  };
-  auto store_slab = [&](int buf) {
-#pragma unroll
-    for (int p = 0; p < AP; ++p)
-      if (!A_PART || p * RPP + vrow < BM)
-        *reinterpret_cast<uint4*>(lds + buf * STAGE + (p * RPP + vrow) * LROW + vcol * 16) = ra[p];
-#pragma unroll
-    for (int p = 0; p < BP; ++p)
-      if (!B_PART || p * RPP + vrow < BN)
-        *reinterpret_cast<uint4*>(lds + buf * STAGE + (BM + p * RPP + vrow) * LROW + vcol * 16) = rb[p];
-  };
+  // Issues the global loads of K slab `kt` into ra / rb (no waiting).
+#define OGLE_LOAD_SLAB(kt)                                                                   \
+  {                                                                                          \
+    int tap_ = 0, cc_ = (kt);                                                                \
+    if (!PW) {                                                                               \
+      tap_ = (kt) / g.cchunks;                                                               \
+      cc_ = (kt) - tap_ * g.cchunks;                                                         \
+    }                                                                                        \
+    const int cbyte_ = cc_ * ROWB + vcol * 16;                                               \
+    const bool c_ok_ = cbyte_ < g.c * ESZ;                                                   \
+    int dy_ = 0, dx_ = 0;                                                                    \
+    if (!PW) {                                                                               \
+      const int ky_ = tap_ / g.k;                                                            \
+      dy_ = ky_ * g.dil;                                                                     \
+      dx_ = (tap_ - ky_ * g.k) * g.dil;                                                      \
+    }                                                                                        \
+    _Pragma("unroll") for (int p = 0; p < AP; ++p) {                                         \
+      unsigned off_;                                                                         \
+      if (PW) {                                                                              \
+        off_ = c_ok_ ? a_base[p] + (unsigned)cbyte_ : kOutOfRange;                           \
+      } else {                                                                               \
+        const int iy_ = a_iy[p] + dy_, ix_ = a_ix[p] + dx_;                                  \
+        const bool in_ = c_ok_ && iy_ >= 0 && iy_ < g.h && ix_ >= 0 && ix_ < g.w;            \
+        off_ = in_ ? a_base[p] + (unsigned)((iy_ * g.w + ix_) * g.c * ESZ + cbyte_)          \
+                   : kOutOfRange;                                                            \
+      }                                                                                      \
+      ra[p] = __builtin_amdgcn_raw_buffer_load_b128(rx, (int)off_, 0, 0);                    \
+    }                                                                                        \
+    _Pragma("unroll") for (int p = 0; p < BP; ++p) {                                         \
+      const unsigned off_ =                                                                  \
+          c_ok_ ? b_base[p] + (unsigned)(tap_ * g.c * ESZ + cbyte_) : kOutOfRange;           \
+      rb[p] = __builtin_amdgcn_raw_buffer_load_b128(rw, (int)off_, 0, 0);                    \
+    }                                                                                        \
+  }
+
+  // Writes ra / rb into LDS buffer `buf`.
+#define OGLE_STORE_SLAB(buf)                                                                 \
+  {                                                                                          \
+    unsigned char* base_ = lds + (buf) * STAGE + vrow * LROW + vcol * 16;                    \
+    _Pragma("unroll") for (int p = 0; p < AP; ++p)                                           \
+      if (!A_PART || p * RPP + vrow < BM)                                                    \
+        *reinterpret_cast<u32x4*>(base_ + p * RPP * LROW) = ra[p];                           \
+    _Pragma("unroll") for (int p = 0; p < BP; ++p)                                           \
+      if (!B_PART || p * RPP + vrow < BN)                                                    \
+        *reinterpret_cast<u32x4*>(base_ + (BM + p * RPP) * LROW) = rb[p];                    \
+  }
 
   floatx16 acc[TM][TN];
 #pragma unroll
@@ -195,13 +211,13 @@ __global__ __launch_bounds__(256) void conv_igemm_kernel(
   const int kt_begin = blockIdx.z * slabs_per_split;
   const int kt_end = min(g.ktiles, kt_begin + slabs_per_split);
 
-  load_slab(kt_begin);
-  store_slab(0);
+  OGLE_LOAD_SLAB(kt_begin);
+  OGLE_STORE_SLAB(0);
   __syncthreads();
   for (int kt = kt_begin; kt < kt_end; ++kt) {
     const int buf = (kt - kt_begin) & 1;
     const bool more = kt + 1 < kt_end;
-    if (more) load_slab(kt + 1);
+    if (more) OGLE_LOAD_SLAB(kt + 1);
     const unsigned char* pa = lds + buf * STAGE + (wave_m * WTM + l32) * LROW + lh * 16;
     const unsigned char* pb = lds + buf * STAGE + (BM + wave_n * WTN + l32) * LROW + lh * 16;
 #pragma unroll
@@ -218,9 +234,11 @@ __global__ __launch_bounds__(256) void conv_igemm_kernel(
 #pragma unroll
         for (int j = 0; j < TN; ++j) Mma<T>::run(av[i], bv[j], acc[i][j]);
     }
-    if (more) store_slab(buf ^ 1);
+    if (more) OGLE_STORE_SLAB(buf ^ 1);
     __syncthreads();
   }
+#undef OGLE_LOAD_SLAB
+#undef OGLE_STORE_SLAB
 
   if (partial != nullptr) {
     float* dst = partial + (long)blockIdx.z * g.m_total * g.o;
@@ -372,6 +390,11 @@ bool igemm_eligible(const OgleConvArgs& a, long* m_out) {
   if ((long)a.kernel_size * a.kernel_size * a.in_c < 32) return false;
   const long m = (long)a.n * a.out_h * a.out_w;
   if (m <= 0 || m > 0x7fffffffL) return false;
+  // operands are addressed with 32-bit byte offsets through buffer loads
+  const long esz = a.dtype == OGLE_F16 ? 2 : 4;
+  const long lim = 0x7fffffffL;
+  if ((long)a.n * a.in_h * a.in_w * a.in_c * esz > lim) return false;
+  if ((long)a.out_c * a.kernel_size * a.kernel_size * a.in_c * esz > lim) return false;
   *m_out = m;
   return true;
 }
@@ -394,6 +417,9 @@ int32_t launch_conv_igemm(const OgleConvArgs& a, hipStream_t s) {
   g.oh = a.out_h; g.ow = a.out_w; g.o = a.out_c;
   g.k = a.kernel_size; g.stride = a.stride; g.pad = a.padding; g.dil = a.dilation;
   g.m_total = (int)m;
+  const long esz = a.dtype == OGLE_F16 ? 2 : 4;
+  g.x_bytes = (unsigned)((long)a.n * a.in_h * a.in_w * a.in_c * esz);
+  g.w_bytes = (unsigned)((long)a.out_c * a.kernel_size * a.kernel_size * a.in_c * esz);
   const bool pw = a.kernel_size == 1 && a.stride == 1 && a.padding == 0;
   if (a.dtype == OGLE_F16) {
     return pw ? launch_plan<__half, 128, true>(g, a, p, s) : launch_plan<__half, 128, false>(g, a, p, s);
