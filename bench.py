@@ -129,6 +129,8 @@ def main():
     ap.add_argument("--batch", type=int, default=16)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--eager", action="store_true", help="launch kernel by kernel instead of a hipGraph")
+    ap.add_argument("--skip-b1", action="store_true",
+                    help="leave out the batch-1 latency leg (keeps a profiler trace to the batch-16 pass)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus %d is not supported (every image is "
@@ -163,9 +165,12 @@ def main():
                     algorithmic_per_step=dom["flops_per_step"] if dom["bound"] == "mfma" else dom["bytes_per_step"])
 
     # batch-1 latency: each pass waits for the previous one
-    s1, _ = build_session(1)
-    lat, _ = s1.time_compute(20, 300, graph=use_graph, with_detect=True, sync_each=True)
-    lat_eager, _ = s1.time_compute(5, 100, graph=False, with_detect=True, sync_each=True)
+    if args.skip_b1:
+        lat = lat_eager = np.array([float("nan")])
+    else:
+        s1, _ = build_session(1)
+        lat, _ = s1.time_compute(20, 300, graph=use_graph, with_detect=True, sync_each=True)
+        lat_eager, _ = s1.time_compute(5, 100, graph=False, with_detect=True, sync_each=True)
 
     result = {
         "metric": METRIC, "value": round(images_per_s, 1), "unit": "images/s", "n_gpus": 1,

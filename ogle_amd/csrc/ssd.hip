@@ -149,6 +149,102 @@ __global__ __launch_bounds__(256) void ssd_detect_kernel(DetectParams p) {
   if (tid == 0) p.kept_count[b] = base;
 }
 
+// Two-kernel form of the same computation, used when every kept_* output is given:
+// ssd_score_kernel spreads the per-prior work over (chunks x images) workgroups and
+// leaves its results UNCOMPACTED in the kept_* arrays at the prior's own slot (prior
+// index, or -1 when the prior is dropped); ssd_compact_kernel then packs each
+// image's survivors to the front in place, in prior order.  A slot is only ever
+// overwritten by an entry that came from the same or a later slot, after the chunk
+// holding it has been read, so the in-place pass needs one barrier per chunk.
+__global__ __launch_bounds__(256) void ssd_score_kernel(DetectParams p) {
+  extern __shared__ float slab[];  // 256 * classes
+  const int b = blockIdx.y;
+  const int start = blockIdx.x * 256;
+  const int tid = threadIdx.x;
+  const int rows = min(256, p.priors - start);
+  const int count = rows * p.classes;
+  const float* src = p.logits + ((long)b * p.priors + start) * p.classes;
+  for (int i = tid; i < count; i += 256) slab[i] = src[i];
+  __syncthreads();
+  if (tid >= rows) return;
+  const int prior = start + tid;
+  const float* l = slab + tid * p.classes;
+  float total_sum = exp_cr(l[0]);
+  int max_id = 0;
+  float max_prob = 0.f;
+  for (int j = 1; j < p.classes; ++j) {
+    const float e = exp_cr(l[j]);
+    total_sum += e;
+    if (max_prob < e) {
+      max_prob = e;
+      max_id = j;
+    }
+  }
+  const long at = (long)b * p.priors + prior;
+  float4 box;
+  if (p.pred != nullptr) {
+    box = decode_one(p.pred[at], p.anchors[b * p.anchor_stride_vec + prior], p.v0, p.v1, p.v2, p.v3);
+    if (p.boxes != nullptr) p.boxes[at] = box;
+  } else {
+    box = p.boxes[at];
+  }
+  max_prob = max_prob / total_sum;
+  const bool keep = max_prob > p.threshold;
+  const float xmin = box.x * p.image_w;
+  const float ymin = box.y * p.image_h;
+  const float xmax = box.z * p.image_w;
+  const float ymax = box.w * p.image_h;
+  p.kept_prior[at] = keep ? prior : -1;
+  p.kept_class[at] = max_id;
+  p.kept_score[at] = max_prob;
+  p.kept_box[at] = make_float4(xmin, ymin, xmax, ymax);
+  p.kept_rect[at] = make_int4((int)xmin, (int)ymin, (int)(xmax - xmin), (int)(ymax - ymin));
+}
+
+__global__ __launch_bounds__(256) void ssd_compact_kernel(DetectParams p) {
+  __shared__ int wave_count[4];
+  const int b = blockIdx.x;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const long row0 = (long)b * p.priors;
+  int base = 0;
+  for (int start = 0; start < p.priors; start += 256) {
+    const int prior = start + tid;
+    int kept = -1, cls = 0;
+    float score = 0.f;
+    float4 box = make_float4(0.f, 0.f, 0.f, 0.f);
+    int4 rect = make_int4(0, 0, 0, 0);
+    if (prior < p.priors) {
+      kept = p.kept_prior[row0 + prior];
+      if (kept >= 0) {
+        cls = p.kept_class[row0 + prior];
+        score = p.kept_score[row0 + prior];
+        box = p.kept_box[row0 + prior];
+        rect = p.kept_rect[row0 + prior];
+      }
+    }
+    const bool keep = kept >= 0;
+    const unsigned long long ballot = __ballot(keep);
+    const int before = __popcll(ballot & ((1ull << lane) - 1ull));
+    if (lane == 0) wave_count[wave] = __popcll(ballot);
+    __syncthreads();  // every read of this chunk is done; wave counts are visible
+    int wave_base = 0;
+    for (int wv = 0; wv < wave; ++wv) wave_base += wave_count[wv];
+    const int chunk_total = wave_count[0] + wave_count[1] + wave_count[2] + wave_count[3];
+    if (keep) {
+      const long slot = row0 + base + wave_base + before;
+      p.kept_prior[slot] = kept;
+      p.kept_class[slot] = cls;
+      p.kept_score[slot] = score;
+      p.kept_box[slot] = box;
+      p.kept_rect[slot] = rect;
+    }
+    base += chunk_total;
+    __syncthreads();  // wave_count is rewritten by the next chunk
+  }
+  if (tid == 0) p.kept_count[b] = base;
+}
+
 }  // namespace
 
 int32_t launch_decode(const OgleDecodeArgs& a, hipStream_t s) {
@@ -181,6 +277,15 @@ int32_t launch_detect(const OgleDetectArgs& a, hipStream_t s) {
   p.kept_box = reinterpret_cast<float4*>(a.kept_box_dev);
   p.kept_rect = reinterpret_cast<int4*>(a.kept_rect_dev);
   const size_t lds = sizeof(float) * 256 * (size_t)a.classes;
+  const bool all_outputs = p.kept_prior && p.kept_class && p.kept_score && p.kept_box && p.kept_rect;
+  if (all_outputs && a.priors > 256 && a.batch <= 65535) {
+    hipLaunchKernelGGL(ssd_score_kernel, dim3((unsigned)((a.priors + 255) / 256), (unsigned)a.batch),
+                       dim3(256), lds, s, p);
+    const int32_t st = check_launch("ssd_score_kernel");
+    if (st != OGLE_OK) return st;
+    hipLaunchKernelGGL(ssd_compact_kernel, dim3((unsigned)a.batch), dim3(256), 0, s, p);
+    return check_launch("ssd_compact_kernel");
+  }
   hipLaunchKernelGGL(ssd_detect_kernel, dim3((unsigned)a.batch), dim3(256), lds, s, p);
   return check_launch("ssd_detect_kernel");
 }

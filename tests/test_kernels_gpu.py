@@ -279,6 +279,37 @@ def test_detect_kept_sets_bit_exact(batch):
         np.testing.assert_array_equal(res2[b]["box"], ora[b]["box"])
 
 
+def test_detect_single_kernel_path_and_optional_outputs():
+    """Fewer than 257 priors, or a missing optional output, takes the one-kernel form."""
+    import ctypes
+    import torch
+    r = rng(3300)
+    for priors, drop_rect in ((200, False), (700, True)):
+        logits = r.normal(0, 0.9, (3, priors, 21)).astype(np.float32)
+        pred = r.normal(0, 1.0, (3, priors, 4)).astype(np.float32)
+        anchors = np.concatenate([r.uniform(.1, .9, (priors, 2)), r.uniform(.05, .5, (priors, 2))],
+                                 1).astype(np.float32)
+        if not drop_rect:
+            res, boxes = gpu_detect(logits, pred, anchors, 0.3, 100.0, 50.0)
+            ora = O.box_info(logits, boxes, 0.3, 100.0, 50.0)
+            for b in range(3):
+                np.testing.assert_array_equal(res[b]["prior"], ora[b]["prior"])
+                np.testing.assert_array_equal(res[b]["rect"], ora[b]["rect"])
+            continue
+        ld, pd, ad = (torch.from_numpy(a).cuda() for a in (logits, pred, anchors))
+        cnt = torch.full((3,), -1, dtype=torch.int32, device="cuda")
+        prior = torch.full((3, priors), -1, dtype=torch.int32, device="cuda")
+        args = H.DetectArgs(ld.data_ptr(), pd.data_ptr(), ad.data_ptr(), None, 3, priors, 21, 0,
+                            (ctypes.c_float * 4)(.1, .1, .2, .2), 0.3, 100.0, 50.0, cnt.data_ptr(),
+                            prior.data_ptr(), None, None, None, None)
+        H.check(H.lib().ogle_hip_ssd_detect(ctypes.byref(args), torch.cuda.current_stream().cuda_stream))
+        torch.cuda.synchronize()
+        ora = O.box_info(logits, O.ssd_decode(pred, anchors), 0.3, 100.0, 50.0)
+        for b in range(3):
+            k = int(cnt[b])
+            np.testing.assert_array_equal(prior[b, :k].cpu().numpy(), ora[b]["prior"])
+
+
 def test_device_exp_matches_host_libm():
     """The device exponential is the correctly rounded expf (binary64 exp, rounded once).  The
     host's libm expf is within 0.502 ulp of the true value, so the two agree except on the few
