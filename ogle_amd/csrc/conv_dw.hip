@@ -3,12 +3,14 @@
 // reading every input element from HBM once and writing every output once.
 //
 // Thread mapping: consecutive threads take consecutive 16-byte channel vectors
-// of consecutive pixels of one image row, so a wave's loads and stores are
-// contiguous runs of NHWC memory.  Each thread owns a vertical strip of R
-// output rows and walks the input rows the strip needs once, so vertically
-// adjacent outputs share their input rows in registers; the horizontal
-// neighbours (x-1, x+1) are the same bytes other lanes of the same and the
-// adjacent wave load at the same time and are served by the vector L1.
+// of consecutive pixel columns of one image row, so a wave's loads and stores
+// are contiguous runs of NHWC memory.  Each thread owns a small patch of output
+// pixels (R rows x Q columns) and requests every input vector the patch needs
+// with branch-free buffer loads before it starts to accumulate, so all of a
+// wave's loads are in flight at once; neighbouring patches' halo vectors are the
+// same bytes other lanes and the adjacent wave load at the same time and are
+// served by the vector L1 / the XCD's L2 (the block order keeps neighbours on one
+// XCD).
 //
 // Semantics follow conv2d_dw.glsl:38-96: accumulator starts at the bias, taps
 // outside the image are skipped, order ky then kx, then the fused activation.
@@ -18,6 +20,8 @@
 namespace ogle {
 namespace {
 
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
 template <typename T>
 struct Vec;
 template <>
@@ -26,6 +30,10 @@ struct Vec<float> {
   __device__ static void load(const float* p, float (&v)[4]) {
     const float4 t = *reinterpret_cast<const float4*>(p);
     v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+  }
+  __device__ static void unpack(const u32x4& t, float (&v)[4]) {
+    v[0] = __uint_as_float(t.x); v[1] = __uint_as_float(t.y);
+    v[2] = __uint_as_float(t.z); v[3] = __uint_as_float(t.w);
   }
   __device__ static void store(float* p, const float (&v)[4]) {
     *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
@@ -44,6 +52,15 @@ struct Vec<__half> {
       v[2 * i + 1] = f.y;
     }
   }
+  __device__ static void unpack(const u32x4& t, float (&v)[8]) {
+    const __half2* h = reinterpret_cast<const __half2*>(&t);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float2 f = __half22float2(h[i]);
+      v[2 * i] = f.x;
+      v[2 * i + 1] = f.y;
+    }
+  }
   __device__ static void store(__half* p, const float (&v)[8]) {
     uint4 t;
     __half2* h = reinterpret_cast<__half2*>(&t);
@@ -54,60 +71,83 @@ struct Vec<__half> {
 };
 
 // 3x3, dilation 1, stride S, channel count a multiple of the vector width.
-template <typename T, int S, int R>
+// A thread owns a patch of R output rows x Q output columns of one channel vector.
+template <typename T, int S, int R, int Q>
 __global__ __launch_bounds__(256) void dwconv3x3_strip(
     const T* __restrict__ x, const T* __restrict__ w, const float* __restrict__ bias,
-    T* __restrict__ y, int n, int h, int wd, int c, int oh, int ow, int pad, Epilogue ep) {
+    T* __restrict__ y, int n, int h, int wd, int c, int oh, int ow, int pad, Epilogue ep,
+    unsigned x_bytes) {
   constexpr int V = Vec<T>::N;
   constexpr int IN_ROWS = (R - 1) * S + 3;
+  constexpr int IN_COLS = (Q - 1) * S + 3;
   const int cv = c / V;
   const int strips = (oh + R - 1) / R;
-  const long total = (long)n * strips * ow * cv;
-  const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  const int colgroups = (ow + Q - 1) / Q;
+  const long total = (long)n * strips * colgroups * cv;
+  // Consecutive logical blocks (neighbouring pixels and strips, which share halo
+  // rows) are kept on one XCD so that the re-read rows hit that XCD's L2.
+  const long idx = (long)xcd_swizzle(blockIdx.x, gridDim.x) * blockDim.x + threadIdx.x;
   if (idx >= total) return;
   const int cg = (int)(idx % cv);
   long t = idx / cv;
-  const int ox = (int)(t % ow);
-  t /= ow;
+  const int oxg = (int)(t % colgroups);
+  t /= colgroups;
   const int strip = (int)(t % strips);
   const int b = (int)(t / strips);
   const int ch = cg * V;
   const int oy0 = strip * R;
+  const int ox0 = oxg * Q;
 
   float wt[9][V];
 #pragma unroll
   for (int tap = 0; tap < 9; ++tap) Vec<T>::load(w + (long)tap * c + ch, wt[tap]);
 
-  float acc[R][V];
+  float acc[R][Q][V];
 #pragma unroll
   for (int r = 0; r < R; ++r)
 #pragma unroll
-    for (int v = 0; v < V; ++v) acc[r][v] = bias != nullptr ? bias[ch + v] : 0.f;
+    for (int q = 0; q < Q; ++q)
+#pragma unroll
+      for (int v = 0; v < V; ++v) acc[r][q][v] = bias != nullptr ? bias[ch + v] : 0.f;
 
+  // Every input vector the patch needs is requested up front with buffer loads;
+  // taps outside the image get an out-of-range offset and come back as zeros, so
+  // there is no branch between the loads and they are all in flight together.
   const int iy0 = oy0 * S - pad;
-  const int ix0 = ox * S - pad;
-  const T* xb = x + (long)b * h * wd * c + ch;
+  const int ix0 = ox0 * S - pad;
+  const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<T*>(x), 0, (int)x_bytes, 0x00020000);
+  const unsigned img = (unsigned)b * (unsigned)(h * wd * c) + (unsigned)ch;
+  u32x4 raw[IN_ROWS][IN_COLS];
 #pragma unroll
   for (int j = 0; j < IN_ROWS; ++j) {
     const int iy = iy0 + j;
-    if (iy < 0 || iy >= h) continue;
-    float in[3][V];
-    bool ok[3];
+    const bool row_ok = iy >= 0 && iy < h;
 #pragma unroll
-    for (int s = 0; s < 3; ++s) {
+    for (int s = 0; s < IN_COLS; ++s) {
       const int ix = ix0 + s;
-      ok[s] = ix >= 0 && ix < wd;
-      if (ok[s]) Vec<T>::load(xb + ((long)iy * wd + ix) * c, in[s]);
+      const bool ok = row_ok && ix >= 0 && ix < wd;
+      const unsigned off =
+          ok ? (img + (unsigned)((iy * wd + ix) * c)) * (unsigned)sizeof(T) : 0x80000000u;
+      raw[j][s] = __builtin_amdgcn_raw_buffer_load_b128(rx, (int)off, 0, 0);
     }
+  }
+#pragma unroll
+  for (int j = 0; j < IN_ROWS; ++j) {
+    float in[IN_COLS][V];
+#pragma unroll
+    for (int s = 0; s < IN_COLS; ++s) Vec<T>::unpack(raw[j][s], in[s]);
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       const int ky = j - r * S;  // compile-time after unrolling
       if (ky < 0 || ky > 2) continue;
 #pragma unroll
-      for (int s = 0; s < 3; ++s) {
-        if (!ok[s]) continue;
+      for (int q = 0; q < Q; ++q) {
 #pragma unroll
-        for (int v = 0; v < V; ++v) acc[r][v] += wt[ky * 3 + s][v] * in[s][v];
+        for (int kx = 0; kx < 3; ++kx) {
+#pragma unroll
+          for (int v = 0; v < V; ++v) acc[r][q][v] += wt[ky * 3 + kx][v] * in[q * S + kx][v];
+        }
       }
     }
   }
@@ -115,10 +155,15 @@ __global__ __launch_bounds__(256) void dwconv3x3_strip(
   for (int r = 0; r < R; ++r) {
     const int oy = oy0 + r;
     if (oy >= oh) break;
-    float out[V];
 #pragma unroll
-    for (int v = 0; v < V; ++v) out[v] = apply_epilogue(acc[r][v], ep);
-    Vec<T>::store(y + (((long)b * oh + oy) * ow + ox) * c + ch, out);
+    for (int q = 0; q < Q; ++q) {
+      const int ox = ox0 + q;
+      if (ox >= ow) break;
+      float out[V];
+#pragma unroll
+      for (int v = 0; v < V; ++v) out[v] = apply_epilogue(acc[r][q][v], ep);
+      Vec<T>::store(y + (((long)b * oh + oy) * ow + ox) * c + ch, out);
+    }
   }
 }
 
@@ -152,27 +197,32 @@ __global__ __launch_bounds__(256) void dwconv_general(
   }
 }
 
-template <typename T, int S, int R>
+template <typename T, int S, int R, int Q = 1>
 int32_t launch_strip(const OgleConvArgs& a, hipStream_t s, const Epilogue& ep) {
   constexpr int V = Vec<T>::N;
-  const long total = (long)a.n * ((a.out_h + R - 1) / R) * a.out_w * (a.in_c / V);
-  const int blocks = ceil_div(total, 256);
-  hipLaunchKernelGGL((dwconv3x3_strip<T, S, R>), dim3(blocks), dim3(256), 0, s,
+  const long total =
+      (long)a.n * ((a.out_h + R - 1) / R) * ((a.out_w + Q - 1) / Q) * (a.in_c / V);
+  const int blocks = (ceil_div(total, 256) + 7) / 8 * 8;  // whole XCD rounds
+  hipLaunchKernelGGL((dwconv3x3_strip<T, S, R, Q>), dim3(blocks), dim3(256), 0, s,
                      static_cast<const T*>(a.input_dev), static_cast<const T*>(a.filter_dev),
                      a.bias_dev, static_cast<T*>(a.output_dev), a.n, a.in_h, a.in_w, a.in_c,
-                     a.out_h, a.out_w, a.padding, ep);
+                     a.out_h, a.out_w, a.padding, ep,
+                     (unsigned)((long)a.n * a.in_h * a.in_w * a.in_c * sizeof(T)));
   return check_launch("dwconv3x3_strip");
 }
 
 template <typename T, int S>
 int32_t pick_strip(const OgleConvArgs& a, hipStream_t s, const Epilogue& ep) {
   constexpr int V = Vec<T>::N;
-  // Taller strips reuse more input rows in registers but cut the thread count;
-  // keep at least ~4 waves per SIMD's worth of threads on the 256 CUs.
+  // A 2x2 (stride 1) or 2x1 patch per thread shares input rows and columns in
+  // registers; smaller problems fall back to one output per thread so that the
+  // grid still covers the 256 CUs (measured on MI355X: patches beyond 2 rows gain
+  // nothing once all loads of a patch are in flight together).
   const long per_row_threads = (long)a.n * a.out_w * (a.in_c / V);
   const long want = 256L * 256 * 4;
-  if (per_row_threads * ((a.out_h + 3) / 4) >= want) return launch_strip<T, S, 4>(a, s, ep);
-  if (per_row_threads * ((a.out_h + 1) / 2) >= want) return launch_strip<T, S, 2>(a, s, ep);
+  if (S == 1 && per_row_threads / 2 * ((a.out_h + 1) / 2) >= want / 2)
+    return launch_strip<T, S, 2, 2>(a, s, ep);
+  if (per_row_threads * ((a.out_h + 1) / 2) >= want / 2) return launch_strip<T, S, 2, 1>(a, s, ep);
   return launch_strip<T, S, 1>(a, s, ep);
 }
 
@@ -180,7 +230,9 @@ template <typename T>
 int32_t run_dw(const OgleConvArgs& a, hipStream_t s) {
   const Epilogue ep = make_epilogue(a.act, a.min_value, a.max_value, a.act_variant);
   constexpr int V = Vec<T>::N;
-  if (a.kernel_size == 3 && a.dilation == 1 && a.in_c % V == 0 &&
+  // the strip kernel addresses the input with 32-bit byte offsets (buffer loads)
+  const bool fits = (long)a.n * a.in_h * a.in_w * a.in_c * (long)sizeof(T) < 0x7fffffffL;
+  if (a.kernel_size == 3 && a.dilation == 1 && a.in_c % V == 0 && fits &&
       (a.stride == 1 || a.stride == 2)) {
     if (a.stride == 1) return pick_strip<T, 1>(a, s, ep);
     return pick_strip<T, 2>(a, s, ep);

@@ -146,10 +146,12 @@ __global__ __launch_bounds__(256) void conv_igemm_kernel(
     b_base[p] = ok ? (unsigned)o * krow_bytes : kOutOfRange;
   }
 
-  u32x4 ra[AP], rb[BP];
+  // Two register sets: slab kt+1 is already in flight in one while slab kt+2 is
+  // being requested into the other, so a load has two slabs of MFMA work to land.
+  u32x4 ra[2][AP], rb[2][BP];
 
   // Issues the global loads of K slab `kt` into ra / rb (no waiting).
-#define OGLE_LOAD_SLAB(kt)                                                                   \
+#define OGLE_LOAD_SLAB(kt, SET)                                                                 \
   {                                                                                          \
     int tap_ = 0, cc_ = (kt);                                                                \
     if (!PW) {                                                                               \
@@ -157,7 +159,7 @@ __global__ __launch_bounds__(256) void conv_igemm_kernel(
       cc_ = (kt) - tap_ * g.cchunks;                                                         \
     }                                                                                        \
     const int cbyte_ = cc_ * ROWB + vcol * 16;                                               \
-    const bool c_ok_ = cbyte_ < g.c * ESZ;                                                   \
+    const bool c_ok_ = cbyte_ < g.c * ESZ && (kt) < kt_end; /* past the end: zeros */       \
     int dy_ = 0, dx_ = 0;                                                                    \
     if (!PW) {                                                                               \
       const int ky_ = tap_ / g.k;                                                            \
@@ -174,25 +176,25 @@ __global__ __launch_bounds__(256) void conv_igemm_kernel(
         off_ = in_ ? a_base[p] + (unsigned)((iy_ * g.w + ix_) * g.c * ESZ + cbyte_)          \
                    : kOutOfRange;                                                            \
       }                                                                                      \
-      ra[p] = __builtin_amdgcn_raw_buffer_load_b128(rx, (int)off_, 0, 0);                    \
+      ra[SET][p] = __builtin_amdgcn_raw_buffer_load_b128(rx, (int)off_, 0, 0);               \
     }                                                                                        \
     _Pragma("unroll") for (int p = 0; p < BP; ++p) {                                         \
       const unsigned off_ =                                                                  \
           c_ok_ ? b_base[p] + (unsigned)(tap_ * g.c * ESZ + cbyte_) : kOutOfRange;           \
-      rb[p] = __builtin_amdgcn_raw_buffer_load_b128(rw, (int)off_, 0, 0);                    \
+      rb[SET][p] = __builtin_amdgcn_raw_buffer_load_b128(rw, (int)off_, 0, 0);               \
     }                                                                                        \
   }
 
   // Writes ra / rb into LDS buffer `buf`.
-#define OGLE_STORE_SLAB(buf)                                                                 \
+#define OGLE_STORE_SLAB(buf, SET)                                                            \
   {                                                                                          \
     unsigned char* base_ = lds + (buf) * STAGE + vrow * LROW + vcol * 16;                    \
     _Pragma("unroll") for (int p = 0; p < AP; ++p)                                           \
       if (!A_PART || p * RPP + vrow < BM)                                                    \
-        *reinterpret_cast<u32x4*>(base_ + p * RPP * LROW) = ra[p];                           \
+        *reinterpret_cast<u32x4*>(base_ + p * RPP * LROW) = ra[SET][p];                      \
     _Pragma("unroll") for (int p = 0; p < BP; ++p)                                           \
       if (!B_PART || p * RPP + vrow < BN)                                                    \
-        *reinterpret_cast<u32x4*>(base_ + (BM + p * RPP) * LROW) = rb[p];                    \
+        *reinterpret_cast<u32x4*>(base_ + (BM + p * RPP) * LROW) = rb[SET][p];               \
   }
 
   floatx16 acc[TM][TN];
@@ -211,68 +213,108 @@ __global__ __launch_bounds__(256) void conv_igemm_kernel(
   const int kt_begin = blockIdx.z * slabs_per_split;
   const int kt_end = min(g.ktiles, kt_begin + slabs_per_split);
 
-  OGLE_LOAD_SLAB(kt_begin);
-  OGLE_STORE_SLAB(0);
+  // One K slab from LDS buffer `buf` into the accumulators.
+#define OGLE_COMPUTE_SLAB(buf)                                                               \
+  {                                                                                          \
+    const unsigned char* pa = lds + (buf) * STAGE + (wave_m * WTM + l32) * LROW + lh * 16;   \
+    const unsigned char* pb = lds + (buf) * STAGE + (BM + wave_n * WTN + l32) * LROW + lh * 16; \
+    _Pragma("unroll") for (int ch = 0; ch < CHUNKS; ++ch) {                                  \
+      uint4 av[TM], bv[TN];                                                                  \
+      _Pragma("unroll") for (int i = 0; i < TM; ++i)                                         \
+        av[i] = *reinterpret_cast<const uint4*>(pa + i * 32 * LROW + ch * 32);               \
+      _Pragma("unroll") for (int j = 0; j < TN; ++j)                                         \
+        bv[j] = *reinterpret_cast<const uint4*>(pb + j * 32 * LROW + ch * 32);               \
+      _Pragma("unroll") for (int i = 0; i < TM; ++i)                                         \
+        _Pragma("unroll") for (int j = 0; j < TN; ++j) Mma<T>::run(av[i], bv[j], acc[i][j]); \
+    }                                                                                        \
+  }
+
+  // Software pipeline, unrolled by two so that the register sets and LDS buffers
+  // are compile-time: while slab kt is multiplied out of one LDS buffer, slab kt+1
+  // (requested one step earlier) is moved from its registers into the other buffer
+  // and slab kt+2 is requested.  Requests past kt_end return zeros and are dropped.
+  OGLE_LOAD_SLAB(kt_begin, 0);
+  OGLE_LOAD_SLAB(kt_begin + 1, 1);
+  OGLE_STORE_SLAB(0, 0);
   __syncthreads();
-  for (int kt = kt_begin; kt < kt_end; ++kt) {
-    const int buf = (kt - kt_begin) & 1;
-    const bool more = kt + 1 < kt_end;
-    if (more) OGLE_LOAD_SLAB(kt + 1);
-    const unsigned char* pa = lds + buf * STAGE + (wave_m * WTM + l32) * LROW + lh * 16;
-    const unsigned char* pb = lds + buf * STAGE + (BM + wave_n * WTN + l32) * LROW + lh * 16;
-#pragma unroll
-    for (int ch = 0; ch < CHUNKS; ++ch) {
-      uint4 av[TM], bv[TN];
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-        av[i] = *reinterpret_cast<const uint4*>(pa + i * 32 * LROW + ch * 32);
-#pragma unroll
-      for (int j = 0; j < TN; ++j)
-        bv[j] = *reinterpret_cast<const uint4*>(pb + j * 32 * LROW + ch * 32);
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j) Mma<T>::run(av[i], bv[j], acc[i][j]);
-    }
-    if (more) OGLE_STORE_SLAB(buf ^ 1);
+  for (int kt = kt_begin; kt < kt_end; kt += 2) {
+    // An odd slab count runs one extra all-zero slab through the second half: a
+    // loop without early exits keeps the accumulators in one set of registers.
+    OGLE_LOAD_SLAB(kt + 2, 0);
+    OGLE_COMPUTE_SLAB(0);
+    OGLE_STORE_SLAB(1, 1);
+    __syncthreads();
+    OGLE_LOAD_SLAB(kt + 3, 1);
+    OGLE_COMPUTE_SLAB(1);
+    OGLE_STORE_SLAB(0, 0);
     __syncthreads();
   }
+#undef OGLE_COMPUTE_SLAB
 #undef OGLE_LOAD_SLAB
 #undef OGLE_STORE_SLAB
 
-  if (partial != nullptr) {
-    float* dst = partial + (long)blockIdx.z * g.m_total * g.o;
+  // Epilogue.  When the row pitch allows 16-byte stores (out_c % 4 == 0) the
+  // accumulators go through a wave-private LDS region to be transposed from the MFMA
+  // layout (a lane holds one column) into rows, so that a wave writes whole
+  // contiguous row segments with 16-byte stores; bias and activation are applied
+  // on the way out.  Otherwise each lane stores its elements one by one.
+  float* const pdst = partial != nullptr ? partial + (long)blockIdx.z * g.m_total * g.o : nullptr;
+  if ((g.o & 3) == 0 && (sizeof(T) == 4 || pdst != nullptr)) {
+    constexpr int SROW = WTN + 4;            // floats per staged row (padded)
+    constexpr int LPR = WTN / 4;             // lanes covering one staged row
+    constexpr int RPI = 64 / LPR;            // rows one store instruction covers
+    static_assert(4 * 32 * SROW * 4 <= 2 * STAGE, "epilogue staging exceeds the K-loop LDS");
+    float* smw = reinterpret_cast<float*>(lds) + wave * 32 * SROW;
+    const int cv = lane % LPR;
+    const int rsub = lane / LPR;
+    const int col = n0 + wave_n * WTN + cv * 4;
+    float4 bias4 = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (pdst == nullptr && bias != nullptr && col < g.o)
+      bias4 = *reinterpret_cast<const float4*>(bias + col);
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int col = n0 + wave_n * WTN + j * 32 + l32;
-      if (col >= g.o) continue;
+    for (int i = 0; i < TM; ++i) {
 #pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        const int rbase = m0 + wave_m * WTM + i * 32 + lh * 4;
+      for (int j = 0; j < TN; ++j)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int row = rbase + (r >> 2) * 8 + (r & 3);
-          if (row < g.m_total) dst[(long)row * g.o + col] = acc[i][j][r];
+        for (int r = 0; r < 16; ++r)
+          smw[((r >> 2) * 8 + lh * 4 + (r & 3)) * SROW + j * 32 + l32] = acc[i][j][r];
+#pragma unroll
+      for (int it = 0; it < 32 / RPI; ++it) {
+        const int row = it * RPI + rsub;
+        float4 v = *reinterpret_cast<const float4*>(smw + row * SROW + cv * 4);
+        const int grow = m0 + wave_m * WTM + i * 32 + row;
+        if (grow < g.m_total && col < g.o) {
+          if (pdst != nullptr) {
+            *reinterpret_cast<float4*>(pdst + (long)grow * g.o + col) = v;
+          } else {
+            v.x = apply_epilogue(v.x + bias4.x, ep);
+            v.y = apply_epilogue(v.y + bias4.y, ep);
+            v.z = apply_epilogue(v.z + bias4.z, ep);
+            v.w = apply_epilogue(v.w + bias4.w, ep);
+            *reinterpret_cast<float4*>(reinterpret_cast<float*>(y) + (long)grow * g.o + col) = v;
+          }
         }
       }
     }
     return;
   }
-
-  // Epilogue: bias, activation, store.
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
     const int col = n0 + wave_n * WTN + j * 32 + l32;
     if (col >= g.o) continue;
-    const float bv = bias != nullptr ? bias[col] : 0.f;
+    const float bv = (pdst == nullptr && bias != nullptr) ? bias[col] : 0.f;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
       const int rbase = m0 + wave_m * WTM + i * 32 + lh * 4;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int row = rbase + (r >> 2) * 8 + (r & 3);
-        if (row < g.m_total)
+        if (row >= g.m_total) continue;
+        if (pdst != nullptr) {
+          pdst[(long)row * g.o + col] = acc[i][j][r];
+        } else {
           y[(long)row * g.o + col] = from_f32<T>(apply_epilogue(acc[i][j][r] + bv, ep));
+        }
       }
     }
   }
@@ -344,6 +386,7 @@ IgemmPlan plan_igemm(const OgleConvArgs& a, long m, bool allow_split) {
     if (sp >= 2) p.splits = (int)sp;
   }
   p.slabs_per_split = (p.ktiles + p.splits - 1) / p.splits;
+  if (p.splits > 1) p.slabs_per_split += p.slabs_per_split & 1;  // the K loop runs slab pairs
   p.splits = (p.ktiles + p.slabs_per_split - 1) / p.slabs_per_split;  // no empty split
   p.workspace_bytes = p.splits > 1 ? (size_t)p.splits * (size_t)m * a.out_c * sizeof(float) : 0;
   return p;
