@@ -351,8 +351,7 @@ struct IgemmPlan {
 
 constexpr long kComputeUnits = 256;
 
-// Picks the output tile and the K split.  Large problems get the largest tile that
-// still yields about two workgroups per compute unit; problems with few output
+// Picks the output tile and the K split.  Problems with few output
 // tiles but a long contraction (the SSD heads, the small feature maps) are split
 // along K until the grid fills the chip, provided a workspace was supplied.
 IgemmPlan plan_igemm(const OgleConvArgs& a, long m, bool allow_split) {
@@ -365,14 +364,14 @@ IgemmPlan plan_igemm(const OgleConvArgs& a, long m, bool allow_split) {
   auto tiles = [&](int cfg) {
     return ((m + kCfgBM[cfg] - 1) / kCfgBM[cfg]) * ((a.out_c + kCfgBN[cfg] - 1) / kCfgBN[cfg]);
   };
+  // Measured on MI355X: 64x64 tiles (eight waves per SIMD resident) match or beat
+  // the larger tiles on every layer of the network because they quantise better
+  // over 256 CUs and hide latency with occupancy; 128x128 only pays off once there
+  // are enough tiles for several rounds.
   if (a.out_c <= 32) {
     p.cfg = CFG_128x32;
-  } else if (a.out_c <= 64) {
-    p.cfg = tiles(CFG_128x64) >= 2 * kComputeUnits ? CFG_128x64 : CFG_64x64;
-  } else if (tiles(CFG_128x128) >= 2 * kComputeUnits) {
+  } else if (tiles(CFG_128x128) >= 4 * kComputeUnits) {
     p.cfg = CFG_128x128;
-  } else if (tiles(CFG_128x64) >= kComputeUnits) {
-    p.cfg = CFG_128x64;
   } else {
     p.cfg = CFG_64x64;
   }
