@@ -81,8 +81,8 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, un
 template <typename T, int BM, int BN, int WM, int WN, int ROWB, bool PW>
 __global__ __launch_bounds__(256) void conv_igemm_kernel(
     ConvGeom g, const T* __restrict__ x, const T* __restrict__ w,
-    const float* __restrict__ bias, T* __restrict__ y, Epilogue ep, int tiles_n,
-    float* __restrict__ partial, int slabs_per_split) {
+    const float* __restrict__ bias, T* __restrict__ y, Epilogue ep, int tiles_n, int tiles,
+    float* __restrict__ partial, int slabs_per_split, int splits) {
   static_assert(WM * WN == 4, "four waves per workgroup");
   constexpr int WTM = BM / WM, WTN = BN / WN;
   constexpr int TM = WTM / 32, TN = WTN / 32;
@@ -103,7 +103,31 @@ __global__ __launch_bounds__(256) void conv_igemm_kernel(
   const int wave = tid >> 6;
   const int wave_m = wave / WN, wave_n = wave % WN;
 
-  const int pid = xcd_swizzle(blockIdx.x, gridDim.x);
+  // Work assignment.  Workgroups are dealt to the 8 XCDs by linear id modulo 8 and
+  // every XCD has a private L2, so the (tile, split) pairs are laid out such that
+  // tiles sharing a band of A rows run on one XCD and, when K is split, an XCD owns
+  // a fixed subset of the K ranges: the filter and input slabs of one K range are
+  // then fetched into one L2 only instead of all eight.
+  int pid, split;
+  {
+    const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
+    if (splits == 1) {
+      // tile row r (the tiles_n tiles that share one band of A rows) goes to XCD
+      // r % 8, so all XCDs advance through memory together
+      const int r = (j / tiles_n) * 8 + xcd;
+      pid = r * tiles_n + j % tiles_n;
+      split = 0;
+    } else if (splits >= 8) {
+      const int zs = splits >> 3;  // splits is a multiple of 8
+      pid = j / zs;
+      split = xcd + 8 * (j - pid * zs);
+    } else {                       // splits is 2 or 4
+      const int xpz = 8 / splits;
+      split = xcd % splits;
+      pid = j * xpz + xcd / splits;
+    }
+    if (pid >= tiles) return;
+  }
   const int tile_n = pid % tiles_n;
   const int tile_m = pid / tiles_n;
   const int m0 = tile_m * BM;
@@ -210,7 +234,7 @@ __global__ __launch_bounds__(256) void conv_igemm_kernel(
 
   // Split-K: workgroup z of the grid contracts K slabs [kt_begin, kt_end) only and
   // leaves its partial sums in `partial`; a second kernel adds the splits in order.
-  const int kt_begin = blockIdx.z * slabs_per_split;
+  const int kt_begin = split * slabs_per_split;
   const int kt_end = min(g.ktiles, kt_begin + slabs_per_split);
 
   // One K slab from LDS buffer `buf` into the accumulators.
@@ -258,7 +282,7 @@ __global__ __launch_bounds__(256) void conv_igemm_kernel(
   // layout (a lane holds one column) into rows, so that a wave writes whole
   // contiguous row segments with 16-byte stores; bias and activation are applied
   // on the way out.  Otherwise each lane stores its elements one by one.
-  float* const pdst = partial != nullptr ? partial + (long)blockIdx.z * g.m_total * g.o : nullptr;
+  float* const pdst = partial != nullptr ? partial + (long)split * g.m_total * g.o : nullptr;
   if ((g.o & 3) == 0 && (sizeof(T) == 4 || pdst != nullptr)) {
     constexpr int SROW = WTN + 4;            // floats per staged row (padded)
     constexpr int LPR = WTN / 4;             // lanes covering one staged row
@@ -350,6 +374,7 @@ struct IgemmPlan {
 };
 
 constexpr long kComputeUnits = 256;
+constexpr int kRowBytesF32 = 64;   // bytes of K per tile row per slab, fp32
 
 // Picks the output tile and the K split.  Problems with few output
 // tiles but a long contraction (the SSD heads, the small feature maps) are split
@@ -357,7 +382,7 @@ constexpr long kComputeUnits = 256;
 IgemmPlan plan_igemm(const OgleConvArgs& a, long m, bool allow_split) {
   IgemmPlan p{};
   const int esz = a.dtype == OGLE_F16 ? 2 : 4;
-  const int rowb = a.dtype == OGLE_F16 ? 128 : 64;
+  const int rowb = a.dtype == OGLE_F16 ? 128 : kRowBytesF32;
   const int epr = rowb / esz;
   p.cchunks = (a.in_c + epr - 1) / epr;
   p.ktiles = a.kernel_size * a.kernel_size * p.cchunks;
@@ -370,7 +395,7 @@ IgemmPlan plan_igemm(const OgleConvArgs& a, long m, bool allow_split) {
   // are enough tiles for several rounds.
   if (a.out_c <= 32) {
     p.cfg = CFG_128x32;
-  } else if (tiles(CFG_128x128) >= 4 * kComputeUnits) {
+  } else if (a.out_c > 64 && tiles(CFG_128x128) >= 4 * kComputeUnits) {
     p.cfg = CFG_128x128;
   } else {
     p.cfg = CFG_64x64;
@@ -382,11 +407,16 @@ IgemmPlan plan_igemm(const OgleConvArgs& a, long m, bool allow_split) {
     long most = p.ktiles / 4;                      // at least four slabs per split
     long sp = want < most ? want : most;
     if (sp > 64) sp = 64;
+    // the kernel's XCD-aware work layout wants a divisor or a multiple of 8
+    if (sp >= 8) sp -= sp % 8;
+    else if (sp >= 4) sp = 4;
+    else if (sp >= 2) sp = 2;
     if (sp >= 2) p.splits = (int)sp;
   }
   p.slabs_per_split = (p.ktiles + p.splits - 1) / p.splits;
   if (p.splits > 1) p.slabs_per_split += p.slabs_per_split & 1;  // the K loop runs slab pairs
-  p.splits = (p.ktiles + p.slabs_per_split - 1) / p.slabs_per_split;  // no empty split
+  // (a split past the end of K would only add zeros; rounding splits down keeps the
+  // divisor-or-multiple-of-8 shape, so empty splits are simply avoided by the cap above)
   p.workspace_bytes = p.splits > 1 ? (size_t)p.splits * (size_t)m * a.out_c * sizeof(float) : 0;
   return p;
 }
@@ -400,11 +430,20 @@ int32_t launch_cfg(const ConvGeom& g0, const OgleConvArgs& a, const IgemmPlan& p
   const int tiles_n = (g.o + BN - 1) / BN;
   const Epilogue ep = make_epilogue(a.act, a.min_value, a.max_value, a.act_variant);
   float* partial = p.splits > 1 ? static_cast<float*>(a.workspace_dev) : nullptr;
-  hipLaunchKernelGGL((conv_igemm_kernel<T, BM, BN, WM, WN, ROWB, PW>),
-                     dim3((unsigned)(tiles_m * tiles_n), 1, (unsigned)p.splits), dim3(256), 0, s, g,
-                     static_cast<const T*>(a.input_dev), static_cast<const T*>(a.filter_dev),
-                     a.bias_dev, static_cast<T*>(a.output_dev), ep, tiles_n, partial,
-                     p.slabs_per_split);
+  const int tiles = tiles_m * tiles_n;
+  unsigned grid;
+  if (p.splits == 1) {
+    grid = 8u * (unsigned)((tiles_m + 7) / 8) * (unsigned)tiles_n;
+  } else if (p.splits >= 8) {
+    grid = (unsigned)tiles * (unsigned)p.splits;
+  } else {
+    const int xpz = 8 / p.splits;
+    grid = 8u * (unsigned)((tiles + xpz - 1) / xpz);
+  }
+  hipLaunchKernelGGL((conv_igemm_kernel<T, BM, BN, WM, WN, ROWB, PW>), dim3(grid), dim3(256), 0, s,
+                     g, static_cast<const T*>(a.input_dev), static_cast<const T*>(a.filter_dev),
+                     a.bias_dev, static_cast<T*>(a.output_dev), ep, tiles_n, tiles, partial,
+                     p.slabs_per_split, p.splits);
   int32_t st = check_launch("conv_igemm");
   if (st != OGLE_OK || p.splits == 1) return st;
   const long mn = (long)g.m_total * g.o;
@@ -466,7 +505,8 @@ int32_t launch_conv_igemm(const OgleConvArgs& a, hipStream_t s) {
   if (a.dtype == OGLE_F16) {
     return pw ? launch_plan<__half, 128, true>(g, a, p, s) : launch_plan<__half, 128, false>(g, a, p, s);
   }
-  return pw ? launch_plan<float, 64, true>(g, a, p, s) : launch_plan<float, 64, false>(g, a, p, s);
+  return pw ? launch_plan<float, kRowBytesF32, true>(g, a, p, s)
+            : launch_plan<float, kRowBytesF32, false>(g, a, p, s);
 }
 
 }  // namespace ogle
