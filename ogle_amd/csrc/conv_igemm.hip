@@ -344,16 +344,27 @@ __global__ __launch_bounds__(256) void conv_igemm_kernel(
   }
 }
 
-// Sums the split-K partials in split order, then bias and activation.
-template <typename T>
+// Sums the split-K partials, then bias and activation.  LANES consecutive lanes
+// share one output element: lane q adds splits q, q+LANES, ... in ascending order and
+// the LANES partial sums are then combined in a fixed butterfly order, so the result
+// depends on neither timing nor grid shape.  Spreading the splits over lanes keeps
+// many loads in flight when there are few outputs but many splits.
+template <typename T, int LANES>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial,
                                                             const float* __restrict__ bias,
                                                             T* __restrict__ y, long mn, int o,
                                                             int splits, Epilogue ep) {
-  for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < mn;
-       idx += (long)gridDim.x * blockDim.x) {
-    float acc = partial[idx];
-    for (int z = 1; z < splits; ++z) acc += partial[(long)z * mn + idx];
+  const int q = threadIdx.x % LANES;
+  const long idx = (long)blockIdx.x * (blockDim.x / LANES) + threadIdx.x / LANES;
+  const bool live = idx < mn;  // dead lanes still take part in the shuffles
+  float acc = 0.f;
+  if (live) {
+#pragma unroll 4
+    for (int z = q; z < splits; z += LANES) acc += partial[(long)z * mn + idx];
+  }
+#pragma unroll
+  for (int d = 1; d < LANES; d <<= 1) acc += __shfl_xor(acc, d, 64);
+  if (live && q == 0) {
     if (bias != nullptr) acc += bias[idx % o];
     y[idx] = from_f32<T>(apply_epilogue(acc, ep));
   }
@@ -447,10 +458,17 @@ int32_t launch_cfg(const ConvGeom& g0, const OgleConvArgs& a, const IgemmPlan& p
   int32_t st = check_launch("conv_igemm");
   if (st != OGLE_OK || p.splits == 1) return st;
   const long mn = (long)g.m_total * g.o;
-  long blocks = (mn + 255) / 256;
-  if (blocks > 4096) blocks = 4096;
-  hipLaunchKernelGGL((splitk_reduce_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, s, partial,
-                     a.bias_dev, static_cast<T*>(a.output_dev), mn, g.o, p.splits, ep);
+  // enough lanes per output that the grid still has about a thousand waves
+  int lanes = 1;
+  while (lanes < 8 && lanes * 2 <= p.splits && mn * lanes < 64L * 1024) lanes *= 2;
+  const dim3 rgrid((unsigned)((mn * lanes + 255) / 256)), block(256);
+  T* out = static_cast<T*>(a.output_dev);
+  switch (lanes) {
+    case 8: hipLaunchKernelGGL((splitk_reduce_kernel<T, 8>), rgrid, block, 0, s, partial, a.bias_dev, out, mn, g.o, p.splits, ep); break;
+    case 4: hipLaunchKernelGGL((splitk_reduce_kernel<T, 4>), rgrid, block, 0, s, partial, a.bias_dev, out, mn, g.o, p.splits, ep); break;
+    case 2: hipLaunchKernelGGL((splitk_reduce_kernel<T, 2>), rgrid, block, 0, s, partial, a.bias_dev, out, mn, g.o, p.splits, ep); break;
+    default: hipLaunchKernelGGL((splitk_reduce_kernel<T, 1>), rgrid, block, 0, s, partial, a.bias_dev, out, mn, g.o, p.splits, ep); break;
+  }
   return check_launch("splitk_reduce");
 }
 
