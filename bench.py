@@ -76,6 +76,35 @@ def per_family_roofline(sess, info, batch, passes):
     return out, other, sum(acc.values())
 
 
+def calibration_copy(megabytes=256, launches=3):
+    """A plain copy of known size through the library's own copy kernel (ogle_hip_convert
+    f32 -> f32), so that a counter run of this script also holds the reference reading that the
+    FETCH_SIZE / WRITE_SIZE counters are scaled by."""
+    import torch
+    from ogle_amd import hip as H
+    n = megabytes * 1024 * 1024 // 4
+    src = torch.ones(n, dtype=torch.float32, device="cuda")
+    dst = torch.empty_like(src)
+    for _ in range(launches):
+        H.check(H.lib().ogle_hip_convert(src.data_ptr(), H.F32, dst.data_ptr(), H.F32, n,
+                                         torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    return n * 4
+
+
+def read_traffic_summary(kernel_family):
+    """HBM bytes per launch of the dominant kernel from the committed counter summary
+    (profiles/bench_b16_pmc_traffic.txt, made from two rocprofv3 --pmc runs of this script)."""
+    path = os.path.join(ROOT, "profiles", "bench_b16_pmc_traffic.txt")
+    try:
+        for line in open(path):
+            if line.startswith("traffic_bytes_per_launch[%s]=" % kernel_family):
+                return float(line.split("=", 1)[1])
+    except OSError:
+        pass
+    return None
+
+
 def cpu_baseline(seed=20240005, images=2, repeats=1):
     """The oracle (CPU restatement of the reference's arithmetic) on the host cores: every conv
     layer of the network, concat and the decode + score filter, for `images` images."""
@@ -160,7 +189,7 @@ def main():
                     achieved=dom["gbs"] if dom["bound"] == "hbm" else dom["tflops"],
                     peak=HBM_PEAK_GBS if dom["bound"] == "hbm" else MFMA_F32_PEAK_TFLOPS,
                     unit="GB/s" if dom["bound"] == "hbm" else "TFLOP/s", frac=dom["frac"],
-                    traffic=None, launches_per_step=dom["launches"],
+                    traffic=read_traffic_summary(dom["kernel"]), launches_per_step=dom["launches"],
                     avg_launch_us=dom["avg_launch_us"],
                     algorithmic_per_step=dom["flops_per_step"] if dom["bound"] == "mfma" else dom["bytes_per_step"])
 
@@ -189,6 +218,7 @@ def main():
         "kernels": fams,
         "non_conv_ms_per_step": round(other_ms, 4),
     }
+    result["calibration_copy_bytes"] = calibration_copy()
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline()
     print(json.dumps(result))
