@@ -157,6 +157,18 @@ size_t ogle_hip_conv_workspace_bytes(const OgleConvArgs* args);
  * conv2d_grp.glsl:30-123, conv2d_any4.glsl:29-96.  Filter layout OHWI. */
 int32_t ogle_hip_conv2d(const OgleConvArgs* args, ogle_stream_t stream);
 
+/*
+ * `count` mutually independent dense / pointwise convolutions (group 1) in as few
+ * launches as possible: the result of each equals ogle_hip_conv2d on it alone, but
+ * problems that use the same MFMA kernel share one grid, so several small
+ * convolutions (the SSD heads) fill the chip side by side instead of one after the
+ * other.  No convolution may read or write another's output, and workspaces must
+ * not be shared between them.  The reference has no counterpart (it draws one node
+ * at a time, fbo_session.cc:140-153); the runtime batches consecutive independent
+ * Conv nodes into this call.
+ */
+int32_t ogle_hip_conv2d_batch(const OgleConvArgs* args, int32_t count, ogle_stream_t stream);
+
 /* Depthwise KxK (group == in_c == out_c): conv2d_dw.glsl:38-96,
  * conv2d_dw_any4.glsl:38-98.  Filter layout HWC. */
 int32_t ogle_hip_dwconv2d(const OgleConvArgs* args, ogle_stream_t stream);

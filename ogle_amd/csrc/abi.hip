@@ -211,6 +211,23 @@ int32_t ogle_hip_conv2d(const OgleConvArgs* a, ogle_stream_t stream) {
   return launch_conv_direct(*a, as_stream(stream));
 }
 
+int32_t ogle_hip_conv2d_batch(const OgleConvArgs* args, int32_t count, ogle_stream_t stream) {
+  if (count < 0 || (count > 0 && args == nullptr))
+    return fail(OGLE_ERR_INVALID_ARG, "conv2d_batch: null args or negative count");
+  for (int i = 0; i < count; ++i) {
+    const int32_t st = validate_conv(&args[i], "conv2d_batch");
+    if (st != OGLE_OK) return st;
+    for (int j = 0; j < i; ++j) {
+      if (args[i].input_dev == args[j].output_dev || args[j].input_dev == args[i].output_dev ||
+          args[i].output_dev == args[j].output_dev)
+        return fail(OGLE_ERR_INVALID_ARG, "conv2d_batch: the convolutions depend on each other");
+      if (args[i].workspace_dev != nullptr && args[i].workspace_dev == args[j].workspace_dev)
+        return fail(OGLE_ERR_INVALID_ARG, "conv2d_batch: two convolutions share one workspace");
+    }
+  }
+  return launch_conv_batch(args, count, as_stream(stream), launch_conv_direct);
+}
+
 int32_t ogle_hip_dwconv2d(const OgleConvArgs* a, ogle_stream_t stream) {
   int32_t st = validate_conv(a, "dwconv2d");
   if (st != OGLE_OK) return st;

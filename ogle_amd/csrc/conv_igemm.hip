@@ -26,6 +26,8 @@
 // Result layout of a 32x32 block: register r of lane l holds
 // row 8*(r/4) + 4*(l/32) + r%4, column l%32, so a store instruction writes two
 // 128-byte runs of one output pixel's channels.
+#include <vector>
+
 #include "common.h"
 
 namespace ogle {
@@ -78,11 +80,13 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, un
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
 }
 
+// One workgroup's share of one convolution: output tile / K range number `bid` of
+// the problem.  Shared by the single-problem kernel and the grouped kernel.
 template <typename T, int BM, int BN, int WM, int WN, int ROWB, bool PW>
-__global__ __launch_bounds__(256) void conv_igemm_kernel(
-    ConvGeom g, const T* __restrict__ x, const T* __restrict__ w,
-    const float* __restrict__ bias, T* __restrict__ y, Epilogue ep, int tiles_n, int tiles,
-    float* __restrict__ partial, int slabs_per_split, int splits) {
+__device__ __forceinline__ void igemm_tile(
+    const ConvGeom& g, const T* __restrict__ x, const T* __restrict__ w,
+    const float* __restrict__ bias, T* __restrict__ y, const Epilogue& ep, int tiles_n,
+    int tiles, float* __restrict__ partial, int slabs_per_split, int splits, int bid) {
   static_assert(WM * WN == 4, "four waves per workgroup");
   constexpr int WTM = BM / WM, WTN = BN / WN;
   constexpr int TM = WTM / 32, TN = WTN / 32;
@@ -110,7 +114,7 @@ __global__ __launch_bounds__(256) void conv_igemm_kernel(
   // then fetched into one L2 only instead of all eight.
   int pid, split;
   {
-    const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
+    const int xcd = bid & 7, j = bid >> 3;
     if (splits == 1) {
       // tile row r (the tiles_n tiles that share one band of A rows) goes to XCD
       // r % 8, so all XCDs advance through memory together
@@ -344,30 +348,96 @@ __global__ __launch_bounds__(256) void conv_igemm_kernel(
   }
 }
 
+// Everything one convolution's workgroups need, as plain data (a kernel argument).
+struct IgemmProblem {
+  ConvGeom g;
+  const void* x;
+  const void* w;
+  const float* bias;
+  void* y;
+  Epilogue ep;
+  int tiles_n, tiles;
+  float* partial;
+  int slabs_per_split, splits;
+};
+
+template <typename T, int BM, int BN, int WM, int WN, int ROWB, bool PW>
+__global__ __launch_bounds__(256) void conv_igemm_kernel(IgemmProblem p) {
+  igemm_tile<T, BM, BN, WM, WN, ROWB, PW>(p.g, static_cast<const T*>(p.x),
+                                          static_cast<const T*>(p.w), p.bias,
+                                          static_cast<T*>(p.y), p.ep, p.tiles_n, p.tiles, p.partial,
+                                          p.slabs_per_split, p.splits, (int)blockIdx.x);
+}
+
+// Several independent convolutions in one grid: blocks [first[i], first[i+1]) work
+// on problem i.  Small problems (the SSD heads) then run side by side instead of
+// one launch after another, each too small to fill the chip.
+constexpr int kMaxGroup = 16;
+struct IgemmGroup {
+  int count;
+  int first[kMaxGroup + 1];
+  IgemmProblem p[kMaxGroup];
+};
+
+template <typename T, int BM, int BN, int WM, int WN, int ROWB, bool PW>
+__global__ __launch_bounds__(256) void conv_igemm_group_kernel(IgemmGroup grp) {
+  int i = 0;
+  while (i + 1 < grp.count && (int)blockIdx.x >= grp.first[i + 1]) ++i;
+  const IgemmProblem& p = grp.p[i];
+  igemm_tile<T, BM, BN, WM, WN, ROWB, PW>(p.g, static_cast<const T*>(p.x),
+                                          static_cast<const T*>(p.w), p.bias,
+                                          static_cast<T*>(p.y), p.ep, p.tiles_n, p.tiles, p.partial,
+                                          p.slabs_per_split, p.splits,
+                                          (int)blockIdx.x - grp.first[i]);
+}
+
+struct ReduceProblem {
+  const float* partial;
+  const float* bias;
+  void* y;
+  long mn;
+  int o, splits;
+  Epilogue ep;
+};
+struct ReduceGroup {
+  int count;
+  int first[kMaxGroup + 1];
+  ReduceProblem p[kMaxGroup];
+};
+
 // Sums the split-K partials, then bias and activation.  LANES consecutive lanes
 // share one output element: lane q adds splits q, q+LANES, ... in ascending order and
 // the LANES partial sums are then combined in a fixed butterfly order, so the result
 // depends on neither timing nor grid shape.  Spreading the splits over lanes keeps
 // many loads in flight when there are few outputs but many splits.
 template <typename T, int LANES>
-__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial,
-                                                            const float* __restrict__ bias,
-                                                            T* __restrict__ y, long mn, int o,
-                                                            int splits, Epilogue ep) {
+__device__ __forceinline__ void splitk_reduce_block(const ReduceProblem& r, int bid) {
   const int q = threadIdx.x % LANES;
-  const long idx = (long)blockIdx.x * (blockDim.x / LANES) + threadIdx.x / LANES;
-  const bool live = idx < mn;  // dead lanes still take part in the shuffles
+  const long idx = (long)bid * (blockDim.x / LANES) + threadIdx.x / LANES;
+  const bool live = idx < r.mn;  // dead lanes still take part in the shuffles
   float acc = 0.f;
   if (live) {
 #pragma unroll 4
-    for (int z = q; z < splits; z += LANES) acc += partial[(long)z * mn + idx];
+    for (int z = q; z < r.splits; z += LANES) acc += r.partial[(long)z * r.mn + idx];
   }
 #pragma unroll
   for (int d = 1; d < LANES; d <<= 1) acc += __shfl_xor(acc, d, 64);
   if (live && q == 0) {
-    if (bias != nullptr) acc += bias[idx % o];
-    y[idx] = from_f32<T>(apply_epilogue(acc, ep));
+    if (r.bias != nullptr) acc += r.bias[idx % r.o];
+    static_cast<T*>(r.y)[idx] = from_f32<T>(apply_epilogue(acc, r.ep));
   }
+}
+
+template <typename T, int LANES>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(ReduceProblem r) {
+  splitk_reduce_block<T, LANES>(r, (int)blockIdx.x);
+}
+
+template <typename T, int LANES>
+__global__ __launch_bounds__(256) void splitk_reduce_group_kernel(ReduceGroup grp) {
+  int i = 0;
+  while (i + 1 < grp.count && (int)blockIdx.x >= grp.first[i + 1]) ++i;
+  splitk_reduce_block<T, LANES>(grp.p[i], (int)blockIdx.x - grp.first[i]);
 }
 
 // Tile configurations (BM, BN, waves along M, waves along N).
@@ -432,54 +502,16 @@ IgemmPlan plan_igemm(const OgleConvArgs& a, long m, bool allow_split) {
   return p;
 }
 
-template <typename T, int BM, int BN, int WM, int WN, int ROWB, bool PW>
-int32_t launch_cfg(const ConvGeom& g0, const OgleConvArgs& a, const IgemmPlan& p, hipStream_t s) {
-  ConvGeom g = g0;
-  g.cchunks = p.cchunks;
-  g.ktiles = p.ktiles;
-  const int tiles_m = (g.m_total + BM - 1) / BM;
-  const int tiles_n = (g.o + BN - 1) / BN;
-  const Epilogue ep = make_epilogue(a.act, a.min_value, a.max_value, a.act_variant);
-  float* partial = p.splits > 1 ? static_cast<float*>(a.workspace_dev) : nullptr;
-  const int tiles = tiles_m * tiles_n;
-  unsigned grid;
-  if (p.splits == 1) {
-    grid = 8u * (unsigned)((tiles_m + 7) / 8) * (unsigned)tiles_n;
-  } else if (p.splits >= 8) {
-    grid = (unsigned)tiles * (unsigned)p.splits;
-  } else {
-    const int xpz = 8 / p.splits;
-    grid = 8u * (unsigned)((tiles + xpz - 1) / xpz);
-  }
-  hipLaunchKernelGGL((conv_igemm_kernel<T, BM, BN, WM, WN, ROWB, PW>), dim3(grid), dim3(256), 0, s,
-                     g, static_cast<const T*>(a.input_dev), static_cast<const T*>(a.filter_dev),
-                     a.bias_dev, static_cast<T*>(a.output_dev), ep, tiles_n, tiles, partial,
-                     p.slabs_per_split, p.splits);
-  int32_t st = check_launch("conv_igemm");
-  if (st != OGLE_OK || p.splits == 1) return st;
-  const long mn = (long)g.m_total * g.o;
-  // enough lanes per output that the grid still has about a thousand waves
-  int lanes = 1;
-  while (lanes < 8 && lanes * 2 <= p.splits && mn * lanes < 64L * 1024) lanes *= 2;
-  const dim3 rgrid((unsigned)((mn * lanes + 255) / 256)), block(256);
-  T* out = static_cast<T*>(a.output_dev);
-  switch (lanes) {
-    case 8: hipLaunchKernelGGL((splitk_reduce_kernel<T, 8>), rgrid, block, 0, s, partial, a.bias_dev, out, mn, g.o, p.splits, ep); break;
-    case 4: hipLaunchKernelGGL((splitk_reduce_kernel<T, 4>), rgrid, block, 0, s, partial, a.bias_dev, out, mn, g.o, p.splits, ep); break;
-    case 2: hipLaunchKernelGGL((splitk_reduce_kernel<T, 2>), rgrid, block, 0, s, partial, a.bias_dev, out, mn, g.o, p.splits, ep); break;
-    default: hipLaunchKernelGGL((splitk_reduce_kernel<T, 1>), rgrid, block, 0, s, partial, a.bias_dev, out, mn, g.o, p.splits, ep); break;
-  }
-  return check_launch("splitk_reduce");
-}
+int tile_bm(int cfg) { return kCfgBM[cfg]; }
+int tile_bn(int cfg) { return kCfgBN[cfg]; }
 
-template <typename T, int ROWB, bool PW>
-int32_t launch_plan(const ConvGeom& g, const OgleConvArgs& a, const IgemmPlan& p, hipStream_t s) {
-  switch (p.cfg) {
-    case CFG_128x128: return launch_cfg<T, 128, 128, 2, 2, ROWB, PW>(g, a, p, s);
-    case CFG_128x64: return launch_cfg<T, 128, 64, 2, 2, ROWB, PW>(g, a, p, s);
-    case CFG_64x64: return launch_cfg<T, 64, 64, 2, 2, ROWB, PW>(g, a, p, s);
-    default: return launch_cfg<T, 128, 32, 4, 1, ROWB, PW>(g, a, p, s);
-  }
+// Grid size of one problem under the kernel's XCD-aware work layout.
+unsigned grid_blocks(const IgemmPlan& p, int tiles_m, int tiles_n) {
+  const int tiles = tiles_m * tiles_n;
+  if (p.splits == 1) return 8u * (unsigned)((tiles_m + 7) / 8) * (unsigned)tiles_n;
+  if (p.splits >= 8) return (unsigned)tiles * (unsigned)p.splits;
+  const int xpz = 8 / p.splits;
+  return 8u * (unsigned)((tiles + xpz - 1) / xpz);
 }
 
 bool igemm_eligible(const OgleConvArgs& a, long* m_out) {
@@ -498,6 +530,106 @@ bool igemm_eligible(const OgleConvArgs& a, long* m_out) {
   return true;
 }
 
+bool is_pointwise(const OgleConvArgs& a) {
+  return a.kernel_size == 1 && a.stride == 1 && a.padding == 0;
+}
+
+// The plan the launch will use: split-K only with a workspace that is large enough.
+IgemmPlan final_plan(const OgleConvArgs& a, long m) {
+  IgemmPlan p = plan_igemm(a, m, a.workspace_dev != nullptr);
+  if (p.workspace_bytes > a.workspace_bytes) p = plan_igemm(a, m, false);
+  return p;
+}
+
+struct Prepared {
+  IgemmProblem prob;
+  ReduceProblem red;
+  unsigned grid;
+  unsigned reduce_grid;
+  int reduce_lanes;
+};
+
+Prepared prepare(const OgleConvArgs& a, long m, const IgemmPlan& p) {
+  Prepared out{};
+  ConvGeom& g = out.prob.g;
+  g.n = a.n; g.h = a.in_h; g.w = a.in_w; g.c = a.in_c;
+  g.oh = a.out_h; g.ow = a.out_w; g.o = a.out_c;
+  g.k = a.kernel_size; g.stride = a.stride; g.pad = a.padding; g.dil = a.dilation;
+  g.m_total = (int)m;
+  g.cchunks = p.cchunks;
+  g.ktiles = p.ktiles;
+  const long esz = a.dtype == OGLE_F16 ? 2 : 4;
+  g.x_bytes = (unsigned)((long)a.n * a.in_h * a.in_w * a.in_c * esz);
+  g.w_bytes = (unsigned)((long)a.out_c * a.kernel_size * a.kernel_size * a.in_c * esz);
+  const int tiles_m = (g.m_total + tile_bm(p.cfg) - 1) / tile_bm(p.cfg);
+  const int tiles_n = (g.o + tile_bn(p.cfg) - 1) / tile_bn(p.cfg);
+  out.prob.x = a.input_dev;
+  out.prob.w = a.filter_dev;
+  out.prob.bias = a.bias_dev;
+  out.prob.y = a.output_dev;
+  out.prob.ep = make_epilogue(a.act, a.min_value, a.max_value, a.act_variant);
+  out.prob.tiles_n = tiles_n;
+  out.prob.tiles = tiles_m * tiles_n;
+  out.prob.partial = p.splits > 1 ? static_cast<float*>(a.workspace_dev) : nullptr;
+  out.prob.slabs_per_split = p.slabs_per_split;
+  out.prob.splits = p.splits;
+  out.grid = grid_blocks(p, tiles_m, tiles_n);
+  if (p.splits > 1) {
+    const long mn = (long)g.m_total * g.o;
+    out.red = ReduceProblem{out.prob.partial, a.bias_dev, a.output_dev, mn, g.o, p.splits, out.prob.ep};
+    // enough lanes per output that the grid still has about a thousand waves
+    int lanes = 1;
+    while (lanes < 8 && lanes * 2 <= p.splits && mn * lanes < 64L * 1024) lanes *= 2;
+    out.reduce_lanes = lanes;
+    out.reduce_grid = (unsigned)((mn * lanes + 255) / 256);
+  }
+  return out;
+}
+
+// Instantiates kernel `K<T, BM, BN, WM, WN, ROWB, PW>` for a runtime (dtype, cfg, pw).
+#define OGLE_IGEMM_DISPATCH(K, dtype, cfg, pw, ...)                                          \
+  do {                                                                                       \
+    if ((dtype) == OGLE_F16) {                                                               \
+      OGLE_IGEMM_DISPATCH_T(K, __half, 128, cfg, pw, __VA_ARGS__);                           \
+    } else {                                                                                 \
+      OGLE_IGEMM_DISPATCH_T(K, float, kRowBytesF32, cfg, pw, __VA_ARGS__);                   \
+    }                                                                                        \
+  } while (0)
+#define OGLE_IGEMM_DISPATCH_T(K, T, ROWB, cfg, pw, ...)                                      \
+  do {                                                                                       \
+    if (pw) {                                                                                \
+      OGLE_IGEMM_DISPATCH_C(K, T, ROWB, true, cfg, __VA_ARGS__);                             \
+    } else {                                                                                 \
+      OGLE_IGEMM_DISPATCH_C(K, T, ROWB, false, cfg, __VA_ARGS__);                            \
+    }                                                                                        \
+  } while (0)
+#define OGLE_IGEMM_DISPATCH_C(K, T, ROWB, PW, cfg, grid, s, arg)                             \
+  switch (cfg) {                                                                             \
+    case CFG_128x128:                                                                        \
+      hipLaunchKernelGGL((K<T, 128, 128, 2, 2, ROWB, PW>), dim3(grid), dim3(256), 0, s, arg); \
+      break;                                                                                 \
+    case CFG_128x64:                                                                         \
+      hipLaunchKernelGGL((K<T, 128, 64, 2, 2, ROWB, PW>), dim3(grid), dim3(256), 0, s, arg);  \
+      break;                                                                                 \
+    case CFG_64x64:                                                                          \
+      hipLaunchKernelGGL((K<T, 64, 64, 2, 2, ROWB, PW>), dim3(grid), dim3(256), 0, s, arg);   \
+      break;                                                                                 \
+    default:                                                                                 \
+      hipLaunchKernelGGL((K<T, 128, 32, 4, 1, ROWB, PW>), dim3(grid), dim3(256), 0, s, arg);  \
+      break;                                                                                 \
+  }
+
+template <typename T>
+void launch_reduce_single(const Prepared& pr, hipStream_t s) {
+  const dim3 grid(pr.reduce_grid), block(256);
+  switch (pr.reduce_lanes) {
+    case 8: hipLaunchKernelGGL((splitk_reduce_kernel<T, 8>), grid, block, 0, s, pr.red); break;
+    case 4: hipLaunchKernelGGL((splitk_reduce_kernel<T, 4>), grid, block, 0, s, pr.red); break;
+    case 2: hipLaunchKernelGGL((splitk_reduce_kernel<T, 2>), grid, block, 0, s, pr.red); break;
+    default: hipLaunchKernelGGL((splitk_reduce_kernel<T, 1>), grid, block, 0, s, pr.red); break;
+  }
+}
+
 }  // namespace
 
 size_t conv_igemm_workspace_bytes(const OgleConvArgs& a) {
@@ -509,22 +641,94 @@ size_t conv_igemm_workspace_bytes(const OgleConvArgs& a) {
 int32_t launch_conv_igemm(const OgleConvArgs& a, hipStream_t s) {
   long m = 0;
   if (!igemm_eligible(a, &m)) return OGLE_ERR_UNSUPPORTED;
-  IgemmPlan p = plan_igemm(a, m, a.workspace_dev != nullptr);
-  if (p.workspace_bytes > a.workspace_bytes) p = plan_igemm(a, m, false);  // workspace too small
-  ConvGeom g{};
-  g.n = a.n; g.h = a.in_h; g.w = a.in_w; g.c = a.in_c;
-  g.oh = a.out_h; g.ow = a.out_w; g.o = a.out_c;
-  g.k = a.kernel_size; g.stride = a.stride; g.pad = a.padding; g.dil = a.dilation;
-  g.m_total = (int)m;
-  const long esz = a.dtype == OGLE_F16 ? 2 : 4;
-  g.x_bytes = (unsigned)((long)a.n * a.in_h * a.in_w * a.in_c * esz);
-  g.w_bytes = (unsigned)((long)a.out_c * a.kernel_size * a.kernel_size * a.in_c * esz);
-  const bool pw = a.kernel_size == 1 && a.stride == 1 && a.padding == 0;
-  if (a.dtype == OGLE_F16) {
-    return pw ? launch_plan<__half, 128, true>(g, a, p, s) : launch_plan<__half, 128, false>(g, a, p, s);
+  const IgemmPlan p = final_plan(a, m);
+  const Prepared pr = prepare(a, m, p);
+  const bool pw = is_pointwise(a);
+  OGLE_IGEMM_DISPATCH(conv_igemm_kernel, a.dtype, p.cfg, pw, pr.grid, s, pr.prob);
+  int32_t st = check_launch("conv_igemm");
+  if (st != OGLE_OK || p.splits == 1) return st;
+  if (a.dtype == OGLE_F16) launch_reduce_single<__half>(pr, s);
+  else launch_reduce_single<float>(pr, s);
+  return check_launch("splitk_reduce");
+}
+
+// Launches `count` mutually independent convolutions.  Those the implicit-GEMM
+// kernel takes are bucketed by kernel instantiation (dtype, tile, pointwise or not)
+// and every bucket goes out as ONE grid (plus one grid for all of its split-K
+// reductions); the others are launched one by one through `fallback`.
+int32_t launch_conv_batch(const OgleConvArgs* args, int count, hipStream_t s,
+                          int32_t (*fallback)(const OgleConvArgs&, hipStream_t)) {
+  struct Item {
+    int index;
+    int key;
+    Prepared pr;
+  };
+  std::vector<Item> items;
+  for (int i = 0; i < count; ++i) {
+    long m = 0;
+    if (!igemm_eligible(args[i], &m)) {
+      const int32_t st = fallback(args[i], s);
+      if (st != OGLE_OK) return st;
+      continue;
+    }
+    const IgemmPlan p = final_plan(args[i], m);
+    Item it;
+    it.index = i;
+    it.key = (args[i].dtype << 8) | (p.cfg << 1) | (is_pointwise(args[i]) ? 1 : 0);
+    it.pr = prepare(args[i], m, p);
+    items.push_back(it);
   }
-  return pw ? launch_plan<float, kRowBytesF32, true>(g, a, p, s)
-            : launch_plan<float, kRowBytesF32, false>(g, a, p, s);
+  std::vector<bool> done(items.size(), false);
+  for (size_t a0 = 0; a0 < items.size(); ++a0) {
+    if (done[a0]) continue;
+    IgemmGroup grp{};
+    ReduceGroup red[4] = {};  // by log2(lanes)
+    const int key = items[a0].key;
+    for (size_t b0 = a0; b0 < items.size() && grp.count < kMaxGroup; ++b0) {
+      if (done[b0] || items[b0].key != key) continue;
+      done[b0] = true;
+      const Prepared& pr = items[b0].pr;
+      grp.first[grp.count + 1] = grp.first[grp.count] + (int)pr.grid;
+      grp.p[grp.count++] = pr.prob;
+      if (pr.prob.splits > 1) {
+        int lg = 0;
+        while ((1 << lg) < pr.reduce_lanes) ++lg;
+        ReduceGroup& r = red[lg];
+        r.first[r.count + 1] = r.first[r.count] + (int)pr.reduce_grid;
+        r.p[r.count++] = pr.red;
+      }
+    }
+    const int dtype = key >> 8, cfg = (key >> 1) & 0x7f;
+    const bool pw = key & 1;
+    if (grp.count == 1) {
+      OGLE_IGEMM_DISPATCH(conv_igemm_kernel, dtype, cfg, pw, (unsigned)grp.first[1], s, grp.p[0]);
+    } else {
+      OGLE_IGEMM_DISPATCH(conv_igemm_group_kernel, dtype, cfg, pw, (unsigned)grp.first[grp.count], s, grp);
+    }
+    int32_t st = check_launch("conv_igemm_group");
+    if (st != OGLE_OK) return st;
+    for (int lg = 0; lg < 4; ++lg) {
+      const ReduceGroup& r = red[lg];
+      if (r.count == 0) continue;
+      const dim3 grid((unsigned)r.first[r.count]), block(256);
+#define OGLE_REDUCE_GROUP(T)                                                                         \
+  switch (lg) {                                                                                      \
+    case 3: hipLaunchKernelGGL((splitk_reduce_group_kernel<T, 8>), grid, block, 0, s, r); break;     \
+    case 2: hipLaunchKernelGGL((splitk_reduce_group_kernel<T, 4>), grid, block, 0, s, r); break;     \
+    case 1: hipLaunchKernelGGL((splitk_reduce_group_kernel<T, 2>), grid, block, 0, s, r); break;     \
+    default: hipLaunchKernelGGL((splitk_reduce_group_kernel<T, 1>), grid, block, 0, s, r); break;    \
+  }
+      if (dtype == OGLE_F16) {
+        OGLE_REDUCE_GROUP(__half)
+      } else {
+        OGLE_REDUCE_GROUP(float)
+      }
+#undef OGLE_REDUCE_GROUP
+      st = check_launch("splitk_reduce_group");
+      if (st != OGLE_OK) return st;
+    }
+  }
+  return OGLE_OK;
 }
 
 }  // namespace ogle

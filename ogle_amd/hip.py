@@ -26,6 +26,7 @@ SYMBOLS = [
     "ogle_hip_convert", "ogle_hip_conv2d", "ogle_hip_dwconv2d", "ogle_hip_pwconv_gemm",
     "ogle_hip_pool2d", "ogle_hip_concat", "ogle_hip_ssd_decode", "ogle_hip_ssd_detect",
     "ogle_hip_expf", "ogle_hip_transpose", "ogle_hip_conv_workspace_bytes",
+    "ogle_hip_conv2d_batch",
 ]
 
 
@@ -129,6 +130,7 @@ def lib():
                           ("ogle_hip_ssd_detect", DetectArgs),
                           ("ogle_hip_transpose", TransposeArgs)):
             getattr(l, name).argtypes = [ctypes.POINTER(typ), ctypes.c_void_p]
+        l.ogle_hip_conv2d_batch.argtypes = [ctypes.POINTER(ConvArgs), ctypes.c_int32, ctypes.c_void_p]
         l.ogle_hip_conv_workspace_bytes.argtypes = [ctypes.POINTER(ConvArgs)]
         l.ogle_hip_conv_workspace_bytes.restype = ctypes.c_size_t
         l.ogle_hip_expf.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64,

@@ -24,17 +24,56 @@ void* Context::stream() {
 }
 
 void* Context::Workspace(size_t bytes) {
-  if (bytes <= workspace_bytes_) return workspace_;
-  if (workspace_ != nullptr) {
-    Finish();  // earlier launches may still be using the old buffer
-    (void)hipFree(workspace_);
-    workspace_ = nullptr;
-    workspace_bytes_ = 0;
+  const size_t need = (bytes + 255) & ~size_t(255);
+  if (workspace_used_ + need > workspace_bytes_) {
+    // Out of room: launch what is deferred (its slices become free), then grow if the
+    // request does not fit even an empty buffer.
+    Flush();
+    if (need > workspace_bytes_) {
+      if (workspace_ != nullptr) {
+        Finish();  // earlier launches may still be using the old buffer
+        (void)hipFree(workspace_);
+        workspace_ = nullptr;
+        workspace_bytes_ = 0;
+      }
+      const size_t rounded = (2 * need + (1u << 20) - 1) & ~((size_t(1) << 20) - 1);
+      OGLE_HIP_CALL(hipMalloc(&workspace_, rounded));
+      workspace_bytes_ = rounded;
+    }
   }
-  const size_t rounded = (bytes + (1u << 20) - 1) & ~((size_t(1) << 20) - 1);
-  OGLE_HIP_CALL(hipMalloc(&workspace_, rounded));
-  workspace_bytes_ = rounded;
-  return workspace_;
+  void* p = static_cast<char*>(workspace_) + workspace_used_;
+  workspace_used_ += need;
+  return p;
+}
+
+void Context::BeforeConv(const void* input, const void* filter, const void* bias,
+                         const void* output) {
+  bool flush = pending_.size() >= 16;
+  for (const OgleConvArgs& p : pending_) {
+    if (p.output_dev == input || p.output_dev == filter || p.output_dev == bias ||
+        p.output_dev == output || p.input_dev == output)
+      flush = true;
+  }
+  if (flush) Flush();
+}
+
+void Context::EnqueueConv(const OgleConvArgs& args) {
+  pending_.push_back(args);
+  if (!batching_) Flush();
+}
+
+void Context::Flush() {
+  if (pending_.empty()) {
+    workspace_used_ = 0;
+    return;
+  }
+  std::vector<OgleConvArgs> batch;
+  batch.swap(pending_);
+  workspace_used_ = 0;
+  const int32_t st = ogle_hip_conv2d_batch(batch.data(), static_cast<int32_t>(batch.size()), stream());
+  if (st != OGLE_OK)
+    LOG(FATAL) << "ogle_hip_conv2d_batch: " << ogle_hip_status_string(st) << ": "
+               << ogle_hip_last_error();
 }
 
 Context::~Context() {
@@ -80,6 +119,7 @@ void Context::CopyCPUTensorToDevice(const Tensor* cpu, Tensor* dev) {
   CHECK_EQ(cpu->num_elements(), dev->num_elements());
   const size_t bytes = cpu->num_elements() * sizeof(float);
   if (bytes == 0) return;
+  Flush();
   hipStream_t s = static_cast<hipStream_t>(stream());
   // The host tensor's element order is the device's: NHWC images, ANY tensors and
   // filters in the file's OIHW order are all dense row-major over shape().
@@ -93,6 +133,7 @@ void Context::CopyDeviceTensorToCPU(const Tensor* dev, Tensor* cpu) {
   CHECK(dev->mem_type() != Tensor::HOST_MEMORY) << "source must be a device tensor";
   CHECK_EQ(cpu->num_elements(), dev->num_elements());
   const size_t bytes = dev->num_elements() * sizeof(float);
+  Flush();
   hipStream_t s = static_cast<hipStream_t>(stream());
   if (bytes == 0) {
     OGLE_HIP_CALL(hipStreamSynchronize(s));
@@ -111,7 +152,10 @@ void Context::CopyDeviceTensorToCPU(const Tensor* dev, Tensor* cpu) {
   cpu->set_initialized(true);
 }
 
-void Context::Finish() { OGLE_HIP_CALL(hipStreamSynchronize(static_cast<hipStream_t>(stream()))); }
+void Context::Finish() {
+  Flush();
+  OGLE_HIP_CALL(hipStreamSynchronize(static_cast<hipStream_t>(stream())));
+}
 
 Context* GetContext() {
   static Context* context = new Context;
@@ -125,25 +169,29 @@ void Program::Check(int32_t status, const char* what) const {
     LOG(FATAL) << what << " (" << name_ << "): " << ogle_hip_status_string(status) << ": "
                << ogle_hip_last_error();
 }
-void Program::RunConv2d(const OgleConvArgs& a) const {
-  Check(ogle_hip_conv2d(&a, context_->stream()), "ogle_hip_conv2d");
-}
+void Program::RunConv2d(const OgleConvArgs& a) const { context_->EnqueueConv(a); }
 void Program::RunDepthwise(const OgleConvArgs& a) const {
+  context_->Flush();
   Check(ogle_hip_dwconv2d(&a, context_->stream()), "ogle_hip_dwconv2d");
 }
 void Program::RunPointwise(const OgleConvArgs& a) const {
-  Check(ogle_hip_pwconv_gemm(&a, context_->stream()), "ogle_hip_pwconv_gemm");
+  // the pointwise attribute rules (conv2d.cc:37) were checked by SelectKernel
+  context_->EnqueueConv(a);
 }
 void Program::RunPool(const OglePoolArgs& a) const {
+  context_->Flush();
   Check(ogle_hip_pool2d(&a, context_->stream()), "ogle_hip_pool2d");
 }
 void Program::RunConcat(const OgleConcatArgs& a) const {
+  context_->Flush();
   Check(ogle_hip_concat(&a, context_->stream()), "ogle_hip_concat");
 }
 void Program::RunDecode(const OgleDecodeArgs& a) const {
+  context_->Flush();
   Check(ogle_hip_ssd_decode(&a, context_->stream()), "ogle_hip_ssd_decode");
 }
 void Program::RunTranspose(const OgleTransposeArgs& a) const {
+  context_->Flush();
   Check(ogle_hip_transpose(&a, context_->stream()), "ogle_hip_transpose");
 }
 

@@ -6,6 +6,7 @@
 #include <map>
 #include <memory>
 #include <string>
+#include <vector>
 
 #include "opengl/core/program.h"
 #include "opengl/core/tensor.h"
@@ -33,11 +34,25 @@ class Context {
   // Device -> host, converting to the host tensor's dformat; synchronises.
   void CopyDeviceTensorToCPU(const Tensor* device_tensor, Tensor* cpu_tensor);
 
-  // Scratch memory shared by every kernel launched on this context's stream (they
-  // run one after the other).  Grows on demand; the pointer is stable once every
-  // kernel of a session has run once.
+  // Scratch memory for the kernels launched on this context's stream.  Each call
+  // returns a slice that no other deferred convolution is using; slices are recycled
+  // when the deferred batch is launched.  Grows on demand (first pass only).
   void* Workspace(size_t bytes);
   size_t workspace_bytes() const { return workspace_bytes_; }
+
+  // Deferred convolutions.  Dense and pointwise Conv nodes are not launched one by
+  // one: they are collected and go out through ogle_hip_conv2d_batch, so that runs
+  // of mutually independent convolutions (the SSD heads) share a grid.  A batch is
+  // launched as soon as anything depends on it: BeforeConv flushes if the coming
+  // convolution reads a deferred output (or the batch is full), every other launch,
+  // copy or wait flushes first.
+  void BeforeConv(const void* input, const void* filter, const void* bias, const void* output);
+  void EnqueueConv(const OgleConvArgs& args);
+  void Flush();
+  void set_batching(bool on) {
+    Flush();
+    batching_ = on;
+  }
 
   void Finish();  // glFinish: waits for the stream
   void Reset() {}
@@ -46,6 +61,9 @@ class Context {
   void* stream_ = nullptr;
   void* workspace_ = nullptr;
   size_t workspace_bytes_ = 0;
+  size_t workspace_used_ = 0;
+  std::vector<OgleConvArgs> pending_;
+  bool batching_ = true;
   std::map<std::string, std::unique_ptr<Program>> programs_;
 };
 

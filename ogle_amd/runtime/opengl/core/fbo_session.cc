@@ -128,6 +128,7 @@ void FBOSession::Setup(const NamedTensorList& inputs_cpu) {
     if (CheckKernelReady(kernel)) {
       // Constants and constant-only subgraphs run once, here (fbo_session.cc:240-244).
       kernel->Compute();
+      context_->Flush();
       UpdateKernelReady(kernel);
     }
   }
@@ -140,6 +141,7 @@ void FBOSession::Compute() {
     if (CheckKernelReady(kernel.get())) continue;
     kernel->Compute();
   }
+  context_->Flush();  // convolutions still deferred at the end of the pass
 }
 
 void FBOSession::Run(const NamedTensorList& inputs_cpu) {
@@ -158,6 +160,7 @@ void FBOSession::RunProfiled(std::vector<NodeTiming>* timings) {
   OGLE_HIP_CALL(hipEventRecord(ev[0], s));
   for (size_t i = 0; i < live.size(); ++i) {
     live[i]->Compute();
+    context_->Flush();  // per-node timing: nothing stays deferred across nodes
     OGLE_HIP_CALL(hipEventRecord(ev[i + 1], s));
   }
   OGLE_HIP_CALL(hipStreamSynchronize(s));

@@ -98,6 +98,7 @@ void Detector::EnqueuePostprocess(const TensorNameList& names, int raw_width, in
   a.kept_score_dev = static_cast<float*>(score_dev_->device_ptr());
   a.kept_box_dev = static_cast<float*>(box_dev_->device_ptr());
   a.kept_rect_dev = static_cast<int32_t*>(rect_dev_->device_ptr());
+  session_->context()->Flush();
   hipStream_t s = static_cast<hipStream_t>(session_->context()->stream());
   const int32_t st = ogle_hip_ssd_detect(&a, s);
   if (st != OGLE_OK) LOG(FATAL) << "ogle_hip_ssd_detect: " << ogle_hip_last_error();

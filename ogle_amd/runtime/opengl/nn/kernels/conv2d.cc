@@ -97,6 +97,7 @@ void Conv2DKernel::InferOutputShape(TensorShapeList& input_shapes, TensorShapeLi
 }
 
 void Conv2DKernel::PackFilter(const Tensor* filter) {
+  context_->Flush();
   const IntList& fs = filter->shape();
   const int layout = variant_ == kDepthwise ? OGLE_FILTER_HWC : OGLE_FILTER_OHWI;
   if (variant_ == kDepthwise) CHECK_EQ(fs[1], 1) << "depthwise filters have one input channel";
@@ -132,6 +133,8 @@ void Conv2DKernel::Compute(TensorList& inputs, TensorList& outputs) {
   a.max_value = max_;
   a.act_variant = act_variant_;
   a.dtype = OGLE_F32;
+  if (variant_ != kDepthwise)
+    context_->BeforeConv(a.input_dev, a.filter_dev, a.bias_dev, a.output_dev);
   if (workspace_need_ < 0) workspace_need_ = static_cast<long>(ogle_hip_conv_workspace_bytes(&a));
   if (workspace_need_ > 0) {
     a.workspace_dev = context_->Workspace(static_cast<size_t>(workspace_need_));

@@ -194,6 +194,52 @@ def test_config3_pointwise_gemm(dtype):
                       "C3 vs oracle")
 
 
+def test_conv_batch_equals_single_launches():
+    """ogle_hip_conv2d_batch: several independent convolutions in grouped launches give exactly
+    what one launch each gives (same kernels, same summation order)."""
+    import ctypes
+    import torch
+    r = rng(2500)
+    cases = [  # n, h, w, c, o, k, s, p
+        (4, 19, 19, 128, 12, 3, 1, 1), (4, 19, 19, 128, 63, 3, 1, 1), (4, 10, 10, 256, 24, 3, 1, 1),
+        (4, 10, 10, 256, 126, 3, 1, 1), (4, 5, 5, 128, 126, 3, 1, 1), (4, 3, 3, 64, 24, 3, 1, 1),
+        (2, 7, 7, 64, 96, 1, 1, 0), (2, 9, 9, 32, 40, 1, 1, 0), (1, 8, 8, 3, 8, 3, 2, 1),
+        (1, 6, 6, 6, 6, 3, 1, 1),
+    ]
+    keep, single, args = [], [], (H.ConvArgs * len(cases))()
+    for i, (n, h, w, c, o, k, st, p) in enumerate(cases):
+        x = torch.from_numpy(r.uniform(-1, 1, (n, h, w, c)).astype(np.float32)).cuda()
+        wt = r.normal(0, 0.2, (o, c, k, k)).astype(np.float32)
+        from util import pack_filter
+        wd = pack_filter(wt, H.FILTER_OHWI)
+        b = torch.from_numpy(r.uniform(-.1, .1, o).astype(np.float32)).cuda()
+        oh, ow = H.out_size(h, k, st, p), H.out_size(w, k, st, p)
+        y1 = torch.full((n, oh, ow, o), float("nan"), device="cuda")
+        y2 = torch.full((n, oh, ow, o), float("nan"), device="cuda")
+        a = H.conv_args(x.data_ptr(), wd.data_ptr(), b.data_ptr(), y1.data_ptr(), n, h, w, c, o, k,
+                        st, p, 1, 1, H.ACT_RELU)
+        need = H.lib().ogle_hip_conv_workspace_bytes(ctypes.byref(a))
+        ws1 = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
+        ws2 = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
+        if need:
+            a.workspace_dev, a.workspace_bytes = ws1.data_ptr(), need
+        H.check(H.lib().ogle_hip_conv2d(ctypes.byref(a), 0))
+        a.output_dev = y2.data_ptr()
+        if need:
+            a.workspace_dev = ws2.data_ptr()
+        args[i] = a
+        keep += [x, wd, b, ws1, ws2]
+        single.append((y1, y2))
+    H.check(H.lib().ogle_hip_conv2d_batch(args, len(cases), 0))
+    torch.cuda.synchronize()
+    for y1, y2 in single:
+        assert torch.isfinite(y2).all()
+        assert torch.equal(y1, y2)
+    # dependent convolutions are refused
+    args[1].input_dev = args[0].output_dev
+    assert H.lib().ogle_hip_conv2d_batch(args, 2, 0) == H.ERR_INVALID_ARG
+
+
 def ssd_anchors():
     """1917 center-size priors: 19/10/5/3/2/1 maps, 3,6,6,6,6,6 anchors, scales 0.2-0.95."""
     maps, counts = [19, 10, 5, 3, 2, 1], [3, 6, 6, 6, 6, 6]
