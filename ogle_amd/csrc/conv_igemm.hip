@@ -82,9 +82,15 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, un
 
 // One workgroup's share of one convolution: output tile / K range number `bid` of
 // the problem.  Shared by the single-problem kernel and the grouped kernel.
+// LDS bytes of one workgroup: two K-slab buffers of BM + BN padded rows.
+template <int BM, int BN, int ROWB>
+constexpr int igemm_lds_bytes() {
+  return 2 * (BM + BN) * (ROWB + 16);
+}
+
 template <typename T, int BM, int BN, int WM, int WN, int ROWB, bool PW>
 __device__ __forceinline__ void igemm_tile(
-    const ConvGeom& g, const T* __restrict__ x, const T* __restrict__ w,
+    unsigned char* __restrict__ lds, const ConvGeom& g, const T* __restrict__ x, const T* __restrict__ w,
     const float* __restrict__ bias, T* __restrict__ y, const Epilogue& ep, int tiles_n,
     int tiles, float* __restrict__ partial, int slabs_per_split, int splits, int bid) {
   static_assert(WM * WN == 4, "four waves per workgroup");
@@ -100,7 +106,7 @@ __device__ __forceinline__ void igemm_tile(
   constexpr int CHUNKS = ROWB / 32;
   constexpr int STAGE = (BM + BN) * LROW;  // one buffer: A rows then B rows
 
-  __shared__ __attribute__((aligned(16))) unsigned char lds[2 * STAGE];
+  static_assert(2 * STAGE == igemm_lds_bytes<BM, BN, ROWB>(), "LDS size");
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -359,11 +365,13 @@ struct IgemmProblem {
   int tiles_n, tiles;
   float* partial;
   int slabs_per_split, splits;
+  int variant;  // mixed-group kernel only: 2 * (tile is 128x32) + (pointwise)
 };
 
 template <typename T, int BM, int BN, int WM, int WN, int ROWB, bool PW>
 __global__ __launch_bounds__(256) void conv_igemm_kernel(IgemmProblem p) {
-  igemm_tile<T, BM, BN, WM, WN, ROWB, PW>(p.g, static_cast<const T*>(p.x),
+  __shared__ __attribute__((aligned(16))) unsigned char lds[igemm_lds_bytes<BM, BN, ROWB>()];
+  igemm_tile<T, BM, BN, WM, WN, ROWB, PW>(lds, p.g, static_cast<const T*>(p.x),
                                           static_cast<const T*>(p.w), p.bias,
                                           static_cast<T*>(p.y), p.ep, p.tiles_n, p.tiles, p.partial,
                                           p.slabs_per_split, p.splits, (int)blockIdx.x);
@@ -381,14 +389,46 @@ struct IgemmGroup {
 
 template <typename T, int BM, int BN, int WM, int WN, int ROWB, bool PW>
 __global__ __launch_bounds__(256) void conv_igemm_group_kernel(IgemmGroup grp) {
+  __shared__ __attribute__((aligned(16))) unsigned char lds[igemm_lds_bytes<BM, BN, ROWB>()];
   int i = 0;
   while (i + 1 < grp.count && (int)blockIdx.x >= grp.first[i + 1]) ++i;
   const IgemmProblem& p = grp.p[i];
-  igemm_tile<T, BM, BN, WM, WN, ROWB, PW>(p.g, static_cast<const T*>(p.x),
+  igemm_tile<T, BM, BN, WM, WN, ROWB, PW>(lds, p.g, static_cast<const T*>(p.x),
                                           static_cast<const T*>(p.w), p.bias,
                                           static_cast<T*>(p.y), p.ep, p.tiles_n, p.tiles, p.partial,
                                           p.slabs_per_split, p.splits,
                                           (int)blockIdx.x - grp.first[i]);
+}
+
+// A group whose members differ in tile shape (64x64 or 128x32) or in being
+// pointwise: each workgroup takes the code path of its own problem.  The branch is
+// uniform over the workgroup; all four paths keep 16 accumulator registers per
+// lane, so the register budget is that of the largest one.
+template <typename T, int ROWB>
+__global__ __launch_bounds__(256) void conv_igemm_mixed_kernel(IgemmGroup grp) {
+  constexpr int kLds = igemm_lds_bytes<128, 32, ROWB>() > igemm_lds_bytes<64, 64, ROWB>()
+                           ? igemm_lds_bytes<128, 32, ROWB>()
+                           : igemm_lds_bytes<64, 64, ROWB>();
+  __shared__ __attribute__((aligned(16))) unsigned char lds[kLds];
+  int i = 0;
+  while (i + 1 < grp.count && (int)blockIdx.x >= grp.first[i + 1]) ++i;
+  const IgemmProblem& p = grp.p[i];
+  const int bid = (int)blockIdx.x - grp.first[i];
+#define OGLE_MIXED_CASE(V, BM, BN, WM, WN, PW)                                                  \
+  case V:                                                                                       \
+    igemm_tile<T, BM, BN, WM, WN, ROWB, PW>(lds, p.g, static_cast<const T*>(p.x),               \
+                                            static_cast<const T*>(p.w), p.bias,                 \
+                                            static_cast<T*>(p.y), p.ep, p.tiles_n, p.tiles,     \
+                                            p.partial, p.slabs_per_split, p.splits, bid);       \
+    break;
+  switch (p.variant) {
+    OGLE_MIXED_CASE(0, 64, 64, 2, 2, false)
+    OGLE_MIXED_CASE(1, 64, 64, 2, 2, true)
+    OGLE_MIXED_CASE(2, 128, 32, 4, 1, false)
+    default:
+      OGLE_MIXED_CASE(3, 128, 32, 4, 1, true)
+  }
+#undef OGLE_MIXED_CASE
 }
 
 struct ReduceProblem {
@@ -398,6 +438,7 @@ struct ReduceProblem {
   long mn;
   int o, splits;
   Epilogue ep;
+  int lanes;  // lanes per output element (1, 2, 4 or 8)
 };
 struct ReduceGroup {
   int count;
@@ -433,11 +474,20 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(ReduceProblem r) {
   splitk_reduce_block<T, LANES>(r, (int)blockIdx.x);
 }
 
-template <typename T, int LANES>
+// The reductions of a whole group in one grid; each workgroup uses the lane count
+// its own problem was planned with.
+template <typename T>
 __global__ __launch_bounds__(256) void splitk_reduce_group_kernel(ReduceGroup grp) {
   int i = 0;
   while (i + 1 < grp.count && (int)blockIdx.x >= grp.first[i + 1]) ++i;
-  splitk_reduce_block<T, LANES>(grp.p[i], (int)blockIdx.x - grp.first[i]);
+  const ReduceProblem& r = grp.p[i];
+  const int bid = (int)blockIdx.x - grp.first[i];
+  switch (r.lanes) {
+    case 8: splitk_reduce_block<T, 8>(r, bid); break;
+    case 4: splitk_reduce_block<T, 4>(r, bid); break;
+    case 2: splitk_reduce_block<T, 2>(r, bid); break;
+    default: splitk_reduce_block<T, 1>(r, bid); break;
+  }
 }
 
 // Tile configurations (BM, BN, waves along M, waves along N).
@@ -573,13 +623,15 @@ Prepared prepare(const OgleConvArgs& a, long m, const IgemmPlan& p) {
   out.prob.partial = p.splits > 1 ? static_cast<float*>(a.workspace_dev) : nullptr;
   out.prob.slabs_per_split = p.slabs_per_split;
   out.prob.splits = p.splits;
+  out.prob.variant = (p.cfg == CFG_128x32 ? 2 : 0) + (is_pointwise(a) ? 1 : 0);
   out.grid = grid_blocks(p, tiles_m, tiles_n);
   if (p.splits > 1) {
     const long mn = (long)g.m_total * g.o;
-    out.red = ReduceProblem{out.prob.partial, a.bias_dev, a.output_dev, mn, g.o, p.splits, out.prob.ep};
     // enough lanes per output that the grid still has about a thousand waves
     int lanes = 1;
     while (lanes < 8 && lanes * 2 <= p.splits && mn * lanes < 64L * 1024) lanes *= 2;
+    out.red = ReduceProblem{out.prob.partial, a.bias_dev, a.output_dev, mn, g.o, p.splits,
+                            out.prob.ep, lanes};
     out.reduce_lanes = lanes;
     out.reduce_grid = (unsigned)((mn * lanes + 255) / 256);
   }
@@ -653,14 +705,16 @@ int32_t launch_conv_igemm(const OgleConvArgs& a, hipStream_t s) {
 }
 
 // Launches `count` mutually independent convolutions.  Those the implicit-GEMM
-// kernel takes are bucketed by kernel instantiation (dtype, tile, pointwise or not)
-// and every bucket goes out as ONE grid (plus one grid for all of its split-K
-// reductions); the others are launched one by one through `fallback`.
+// kernel takes go out as ONE grid (plus one grid for all of their split-K
+// reductions) per storage type: a group whose members share the kernel
+// instantiation uses that instantiation, a mixed group of 64x64 and 128x32 tiles the
+// kernel that branches per workgroup; 128x128-tile problems fill the chip on their
+// own and are launched singly.  The others are launched one by one through `fallback`.
 int32_t launch_conv_batch(const OgleConvArgs* args, int count, hipStream_t s,
                           int32_t (*fallback)(const OgleConvArgs&, hipStream_t)) {
   struct Item {
-    int index;
-    int key;
+    int dtype, cfg;
+    bool pw;
     Prepared pr;
   };
   std::vector<Item> items;
@@ -672,61 +726,60 @@ int32_t launch_conv_batch(const OgleConvArgs* args, int count, hipStream_t s,
       continue;
     }
     const IgemmPlan p = final_plan(args[i], m);
-    Item it;
-    it.index = i;
-    it.key = (args[i].dtype << 8) | (p.cfg << 1) | (is_pointwise(args[i]) ? 1 : 0);
-    it.pr = prepare(args[i], m, p);
-    items.push_back(it);
+    items.push_back(Item{args[i].dtype, p.cfg, is_pointwise(args[i]), prepare(args[i], m, p)});
   }
+  auto mixable = [](const Item& it) { return it.cfg == CFG_64x64 || it.cfg == CFG_128x32; };
   std::vector<bool> done(items.size(), false);
   for (size_t a0 = 0; a0 < items.size(); ++a0) {
     if (done[a0]) continue;
     IgemmGroup grp{};
-    ReduceGroup red[4] = {};  // by log2(lanes)
-    const int key = items[a0].key;
+    ReduceGroup red{};
+    const Item& head = items[a0];
+    bool uniform = true;
     for (size_t b0 = a0; b0 < items.size() && grp.count < kMaxGroup; ++b0) {
-      if (done[b0] || items[b0].key != key) continue;
+      const Item& it = items[b0];
+      if (done[b0] || it.dtype != head.dtype) continue;
+      const bool same = it.cfg == head.cfg && it.pw == head.pw;
+      if (!same && !(mixable(head) && mixable(it))) continue;
+      uniform = uniform && same;
       done[b0] = true;
-      const Prepared& pr = items[b0].pr;
+      const Prepared& pr = it.pr;
       grp.first[grp.count + 1] = grp.first[grp.count] + (int)pr.grid;
       grp.p[grp.count++] = pr.prob;
       if (pr.prob.splits > 1) {
-        int lg = 0;
-        while ((1 << lg) < pr.reduce_lanes) ++lg;
-        ReduceGroup& r = red[lg];
-        r.first[r.count + 1] = r.first[r.count] + (int)pr.reduce_grid;
-        r.p[r.count++] = pr.red;
+        red.first[red.count + 1] = red.first[red.count] + (int)pr.reduce_grid;
+        red.p[red.count++] = pr.red;
       }
     }
-    const int dtype = key >> 8, cfg = (key >> 1) & 0x7f;
-    const bool pw = key & 1;
+    const unsigned grid = (unsigned)grp.first[grp.count];
     if (grp.count == 1) {
-      OGLE_IGEMM_DISPATCH(conv_igemm_kernel, dtype, cfg, pw, (unsigned)grp.first[1], s, grp.p[0]);
+      OGLE_IGEMM_DISPATCH(conv_igemm_kernel, head.dtype, head.cfg, head.pw, grid, s, grp.p[0]);
+    } else if (uniform) {
+      OGLE_IGEMM_DISPATCH(conv_igemm_group_kernel, head.dtype, head.cfg, head.pw, grid, s, grp);
+    } else if (head.dtype == OGLE_F16) {
+      hipLaunchKernelGGL((conv_igemm_mixed_kernel<__half, 128>), dim3(grid), dim3(256), 0, s, grp);
     } else {
-      OGLE_IGEMM_DISPATCH(conv_igemm_group_kernel, dtype, cfg, pw, (unsigned)grp.first[grp.count], s, grp);
+      hipLaunchKernelGGL((conv_igemm_mixed_kernel<float, kRowBytesF32>), dim3(grid), dim3(256), 0,
+                         s, grp);
     }
     int32_t st = check_launch("conv_igemm_group");
     if (st != OGLE_OK) return st;
-    for (int lg = 0; lg < 4; ++lg) {
-      const ReduceGroup& r = red[lg];
-      if (r.count == 0) continue;
-      const dim3 grid((unsigned)r.first[r.count]), block(256);
-#define OGLE_REDUCE_GROUP(T)                                                                         \
-  switch (lg) {                                                                                      \
-    case 3: hipLaunchKernelGGL((splitk_reduce_group_kernel<T, 8>), grid, block, 0, s, r); break;     \
-    case 2: hipLaunchKernelGGL((splitk_reduce_group_kernel<T, 4>), grid, block, 0, s, r); break;     \
-    case 1: hipLaunchKernelGGL((splitk_reduce_group_kernel<T, 2>), grid, block, 0, s, r); break;     \
-    default: hipLaunchKernelGGL((splitk_reduce_group_kernel<T, 1>), grid, block, 0, s, r); break;    \
-  }
-      if (dtype == OGLE_F16) {
-        OGLE_REDUCE_GROUP(__half)
-      } else {
-        OGLE_REDUCE_GROUP(float)
-      }
-#undef OGLE_REDUCE_GROUP
-      st = check_launch("splitk_reduce_group");
-      if (st != OGLE_OK) return st;
+    if (red.count == 0) continue;
+    const dim3 rgrid((unsigned)red.first[red.count]), block(256);
+    if (red.count == 1) {
+      Prepared one{};
+      one.red = red.p[0];
+      one.reduce_grid = rgrid.x;
+      one.reduce_lanes = red.p[0].lanes;
+      if (head.dtype == OGLE_F16) launch_reduce_single<__half>(one, s);
+      else launch_reduce_single<float>(one, s);
+    } else if (head.dtype == OGLE_F16) {
+      hipLaunchKernelGGL((splitk_reduce_group_kernel<__half>), rgrid, block, 0, s, red);
+    } else {
+      hipLaunchKernelGGL((splitk_reduce_group_kernel<float>), rgrid, block, 0, s, red);
     }
+    st = check_launch("splitk_reduce_group");
+    if (st != OGLE_OK) return st;
   }
   return OGLE_OK;
 }

@@ -277,6 +277,21 @@ int64_t ogle_rt_model_debug_string(const void* data, size_t size, char* out, int
 
 int32_t ogle_rt_num_kernels(OgleSession* s) { return s->session->num_kernels(); }
 
+int32_t ogle_rt_set_reorder(OgleSession* s, int32_t on) {
+  return (int32_t)Guard([&]() -> int64_t {
+    s->session->set_reorder(on != 0);
+    return 0;
+  });
+}
+
+const char* ogle_rt_issue_order_name(OgleSession* s, int32_t i) {
+  static thread_local std::string name;
+  const auto names = s->session->IssueOrder();
+  if (i < 0 || i >= (int32_t)names.size()) return nullptr;
+  name = names[i];
+  return name.c_str();
+}
+
 int32_t ogle_rt_registered_kernel_count(void) {
   return (int32_t)opengl::KernelRegistry::Global()->RegisteredNames().size();
 }

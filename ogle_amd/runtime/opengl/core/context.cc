@@ -23,22 +23,32 @@ void* Context::stream() {
   return stream_;
 }
 
+void Context::ReserveWorkspace(size_t bytes) {
+  if (bytes <= workspace_bytes_) return;
+  Finish();  // launches deferred work; earlier launches may still be using the old buffer
+  if (workspace_ != nullptr) (void)hipFree(workspace_);
+  workspace_ = nullptr;
+  workspace_bytes_ = 0;
+  const size_t rounded = (bytes + (1u << 20) - 1) & ~((size_t(1) << 20) - 1);
+  OGLE_HIP_CALL(hipMalloc(&workspace_, rounded));
+  workspace_bytes_ = rounded;
+}
+
 void* Context::Workspace(size_t bytes) {
   const size_t need = (bytes + 255) & ~size_t(255);
   if (workspace_used_ + need > workspace_bytes_) {
-    // Out of room: launch what is deferred (its slices become free), then grow if the
-    // request does not fit even an empty buffer.
+    // Out of room: grow to twice what the batch would have needed unbroken, so
+    // that the next pass keeps it in one piece.
+    const size_t want = 2 * (workspace_used_ + need);
     Flush();
-    if (need > workspace_bytes_) {
-      if (workspace_ != nullptr) {
-        Finish();  // earlier launches may still be using the old buffer
-        (void)hipFree(workspace_);
-        workspace_ = nullptr;
-        workspace_bytes_ = 0;
-      }
-      const size_t rounded = (2 * need + (1u << 20) - 1) & ~((size_t(1) << 20) - 1);
-      OGLE_HIP_CALL(hipMalloc(&workspace_, rounded));
-      workspace_bytes_ = rounded;
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    (void)hipStreamIsCapturing(static_cast<hipStream_t>(stream()), &capturing);
+    if (capturing == hipStreamCaptureStatusNone) {
+      ReserveWorkspace(want);
+    } else {
+      CHECK(need <= workspace_bytes_)
+          << "convolution workspace too small and the stream is being captured; "
+             "run one pass outside the capture or call ReserveWorkspace first";
     }
   }
   void* p = static_cast<char*>(workspace_) + workspace_used_;
@@ -46,14 +56,42 @@ void* Context::Workspace(size_t bytes) {
   return p;
 }
 
+namespace {
+size_t ElemBytes(const OgleConvArgs& a) { return a.dtype == OGLE_F16 ? 2 : 4; }
+bool Inside(const void* p, const void* base, size_t bytes) {
+  const char* q = static_cast<const char*>(p);
+  const char* b = static_cast<const char*>(base);
+  return q >= b && q < b + bytes;
+}
+}  // namespace
+
+bool Context::TouchesPending(const void* p, bool written_only) const {
+  if (p == nullptr) return false;
+  for (const OgleConvArgs& c : pending_) {
+    const size_t esz = ElemBytes(c);
+    if (Inside(p, c.output_dev, static_cast<size_t>(c.n) * c.out_h * c.out_w * c.out_c * esz))
+      return true;
+    if (written_only) continue;
+    if (Inside(p, c.input_dev, static_cast<size_t>(c.n) * c.in_h * c.in_w * c.in_c * esz)) return true;
+    if (p == c.filter_dev || p == c.bias_dev) return true;
+  }
+  return false;
+}
+
 void Context::BeforeConv(const void* input, const void* filter, const void* bias,
                          const void* output) {
-  bool flush = pending_.size() >= 16;
-  for (const OgleConvArgs& p : pending_) {
-    if (p.output_dev == input || p.output_dev == filter || p.output_dev == bias ||
-        p.output_dev == output || p.input_dev == output)
-      flush = true;
-  }
+  // reads of something a deferred convolution writes; a write into anything one touches
+  if (pending_.size() >= 16 || TouchesPending(input, true) || TouchesPending(filter, true) ||
+      TouchesPending(bias, true) || TouchesPending(output, false))
+    Flush();
+}
+
+void Context::BeforeLaunch(const void* const* reads, int n_reads, const void* const* writes,
+                           int n_writes) {
+  if (pending_.empty()) return;
+  bool flush = false;
+  for (int i = 0; i < n_reads && !flush; ++i) flush = TouchesPending(reads[i], true);
+  for (int i = 0; i < n_writes && !flush; ++i) flush = TouchesPending(writes[i], false);
   if (flush) Flush();
 }
 
@@ -171,7 +209,9 @@ void Program::Check(int32_t status, const char* what) const {
 }
 void Program::RunConv2d(const OgleConvArgs& a) const { context_->EnqueueConv(a); }
 void Program::RunDepthwise(const OgleConvArgs& a) const {
-  context_->Flush();
+  const void* reads[] = {a.input_dev, a.filter_dev, a.bias_dev};
+  const void* writes[] = {a.output_dev};
+  context_->BeforeLaunch(reads, 3, writes, 1);
   Check(ogle_hip_dwconv2d(&a, context_->stream()), "ogle_hip_dwconv2d");
 }
 void Program::RunPointwise(const OgleConvArgs& a) const {
@@ -179,19 +219,26 @@ void Program::RunPointwise(const OgleConvArgs& a) const {
   context_->EnqueueConv(a);
 }
 void Program::RunPool(const OglePoolArgs& a) const {
-  context_->Flush();
+  const void* reads[] = {a.input_dev};
+  const void* writes[] = {a.output_dev};
+  context_->BeforeLaunch(reads, 1, writes, 1);
   Check(ogle_hip_pool2d(&a, context_->stream()), "ogle_hip_pool2d");
 }
 void Program::RunConcat(const OgleConcatArgs& a) const {
-  context_->Flush();
+  const void* writes[] = {a.output_dev};
+  context_->BeforeLaunch(a.inputs_dev, a.n_inputs, writes, 1);
   Check(ogle_hip_concat(&a, context_->stream()), "ogle_hip_concat");
 }
 void Program::RunDecode(const OgleDecodeArgs& a) const {
-  context_->Flush();
+  const void* reads[] = {a.prediction_dev, a.anchors_dev};
+  const void* writes[] = {a.boxes_dev};
+  context_->BeforeLaunch(reads, 2, writes, 1);
   Check(ogle_hip_ssd_decode(&a, context_->stream()), "ogle_hip_ssd_decode");
 }
 void Program::RunTranspose(const OgleTransposeArgs& a) const {
-  context_->Flush();
+  const void* reads[] = {a.input_dev};
+  const void* writes[] = {a.output_dev};
+  context_->BeforeLaunch(reads, 1, writes, 1);
   Check(ogle_hip_transpose(&a, context_->stream()), "ogle_hip_transpose");
 }
 

@@ -36,23 +36,29 @@ class Context {
 
   // Scratch memory for the kernels launched on this context's stream.  Each call
   // returns a slice that no other deferred convolution is using; slices are recycled
-  // when the deferred batch is launched.  Grows on demand (first pass only).
+  // when the deferred batch is launched.  A request that does not fit launches the
+  // batch first and, if it still does not fit, waits for the stream and reallocates
+  // (not possible while the stream is being captured: ReserveWorkspace beforehand).
   void* Workspace(size_t bytes);
+  void ReserveWorkspace(size_t bytes);
   size_t workspace_bytes() const { return workspace_bytes_; }
 
   // Deferred convolutions.  Dense and pointwise Conv nodes are not launched one by
-  // one: they are collected and go out through ogle_hip_conv2d_batch, so that runs
-  // of mutually independent convolutions (the SSD heads) share a grid.  A batch is
-  // launched as soon as anything depends on it: BeforeConv flushes if the coming
-  // convolution reads a deferred output (or the batch is full), every other launch,
-  // copy or wait flushes first.
+  // one: they are collected and go out through ogle_hip_conv2d_batch, so that
+  // mutually independent convolutions (the SSD heads next to the feature-extractor
+  // chain) share a grid.  A batch is launched as soon as anything depends on it:
+  // BeforeConv flushes if the coming convolution touches a deferred one's buffers (or
+  // the batch is full), BeforeLaunch does the same for any other kernel given the
+  // buffers it reads and writes; copies and waits always flush.
   void BeforeConv(const void* input, const void* filter, const void* bias, const void* output);
+  void BeforeLaunch(const void* const* reads, int n_reads, const void* const* writes, int n_writes);
   void EnqueueConv(const OgleConvArgs& args);
   void Flush();
   void set_batching(bool on) {
     Flush();
     batching_ = on;
   }
+  size_t pending_convs() const { return pending_.size(); }
 
   void Finish();  // glFinish: waits for the stream
   void Reset() {}
@@ -62,6 +68,9 @@ class Context {
   void* workspace_ = nullptr;
   size_t workspace_bytes_ = 0;
   size_t workspace_used_ = 0;
+  // True if `p` lies inside a buffer a deferred convolution writes (`written`) or
+  // reads or writes (`!written`).
+  bool TouchesPending(const void* p, bool written_only) const;
   std::vector<OgleConvArgs> pending_;
   bool batching_ = true;
   std::map<std::string, std::unique_ptr<Program>> programs_;

@@ -2,7 +2,11 @@
 
 #include <hip/hip_runtime_api.h>
 
+#include <algorithm>
+#include <cstdlib>
 #include <fstream>
+#include <map>
+#include <set>
 #include <sstream>
 
 #include "opengl/core/kernel.h"
@@ -18,7 +22,11 @@ namespace opengl {
     if (e__ != hipSuccess) LOG(FATAL) << #expr << ": " << hipGetErrorString(e__); \
   } while (0)
 
-FBOSession::FBOSession(Context* context) : context_(context) { context_->Reset(); }
+FBOSession::FBOSession(Context* context) : context_(context) {
+  context_->Reset();
+  const char* env = std::getenv("OGLE_FILE_ORDER");
+  if (env != nullptr && env[0] != '\0' && env[0] != '0') reorder_ = false;
+}
 
 FBOSession::~FBOSession() {
   if (graph_exec_ != nullptr) (void)hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph_exec_));
@@ -132,15 +140,167 @@ void FBOSession::Setup(const NamedTensorList& inputs_cpu) {
       UpdateKernelReady(kernel);
     }
   }
+  BuildSchedule();
   finalized_ = true;
+}
+
+// Issue order of a pass.  The context defers convolutions and launches the
+// deferred ones as one grid when something needs a result; in file order the SSD
+// heads all come last and fill the chip by themselves while the chain of small
+// feature-extractor convolutions before them runs one under-filled launch after
+// another.  A head only needs its feature map, so it may be issued any time between
+// that map's launch and its own place in the file.  This pass simulates the
+// context's flush rule over the file order to find the launch groups, then moves
+// each convolution that has such slack to the group (within its window) where it
+// adds least to the estimated pass time: a group costs max(launch floor, work /
+// throughput), so under-filled groups absorb work for free.  A moved node is issued
+// just before the node that triggers its new group's launch.  Data dependencies are
+// still enforced by the context at run time, whatever this order is.
+void FBOSession::BuildSchedule() {
+  order_.clear();
+  std::vector<Kernel*> live;
+  for (auto& kernel : kernels_)
+    if (!CheckKernelReady(kernel.get())) live.push_back(kernel.get());
+  const int n = static_cast<int>(live.size());
+
+  // every deferrable node's scratch fits at once, so a batch is never cut short
+  size_t scratch = 0;
+  for (Kernel* k : live)
+    if (k->Deferrable()) scratch += (k->ScratchBytes() + 255) & ~size_t(255);
+  if (scratch > 0) context_->ReserveWorkspace(scratch);
+
+  if (!reorder_) {
+    order_ = live;
+    return;
+  }
+
+  // producer of every tensor, looking through nodes that only re-interpret memory
+  std::map<int, int> producer;  // tensor index -> position in `live` (views resolved)
+  std::vector<bool> is_view(n, false);
+  std::vector<std::vector<int>> deps(n);
+  for (int i = 0; i < n; ++i) {
+    Kernel* k = live[i];
+    for (int t : k->input_tensor_indexes_) {
+      auto it = producer.find(t);
+      if (it != producer.end()) deps[i].push_back(it->second);
+    }
+    bool view = !k->output_tensor_indexes_.empty();
+    for (size_t j = 0; j < k->output_tensor_indexes_.size(); ++j)
+      if (k->OutputAliasesInput(static_cast<int>(j)) < 0) view = false;
+    is_view[i] = view;
+    for (size_t j = 0; j < k->output_tensor_indexes_.size(); ++j) {
+      int src = i;
+      if (view) {
+        const int in = k->input_tensor_indexes_[k->OutputAliasesInput(static_cast<int>(j))];
+        auto it = producer.find(in);
+        src = it != producer.end() ? it->second : -1;
+      }
+      if (src >= 0) producer[k->output_tensor_indexes_[j]] = src;
+    }
+  }
+
+  // groups under the context's flush rule, in file order
+  constexpr int kMaxBatch = 16;
+  std::vector<int> group(n, -1);
+  std::vector<int> trigger;  // trigger[g]: position whose issue launches group g (n: end of pass)
+  {
+    std::set<int> pending;
+    auto depends_on_pending = [&](int i) {
+      for (int d : deps[i])
+        if (pending.count(d)) return true;
+      return false;
+    };
+    for (int i = 0; i < n; ++i) {
+      if (is_view[i]) continue;
+      const bool defer = live[i]->Deferrable();
+      if (!pending.empty() &&
+          (depends_on_pending(i) || (defer && static_cast<int>(pending.size()) >= kMaxBatch))) {
+        trigger.push_back(i);
+        pending.clear();
+      }
+      if (defer) {
+        pending.insert(i);
+        group[i] = static_cast<int>(trigger.size());
+      }
+    }
+    trigger.push_back(n);  // whatever is left goes out at the end of the pass
+  }
+  const int groups = static_cast<int>(trigger.size());
+
+  // cost model: microseconds at a sustained MFMA rate, with a floor per launch
+  constexpr double kMacPerUs = 45e6;  // ~90 TFLOP/s
+  constexpr double kFloorUs = 8.0;
+  std::vector<double> load(groups, 0.0);
+  std::vector<int> members(groups, 0);
+  for (int i = 0; i < n; ++i)
+    if (group[i] >= 0) {
+      load[group[i]] += live[i]->WorkEstimate() / kMacPerUs;
+      ++members[group[i]];
+    }
+  auto cost = [&](double us) { return std::max(kFloorUs, us); };
+
+  std::vector<int> placed(group);
+  std::vector<std::vector<int>> moved(groups);  // nodes to issue just before trigger[g]
+  for (int i = 0; i < n; ++i) {
+    if (group[i] < 0) continue;
+    int earliest = 0;
+    for (int d : deps[i]) {
+      int g;
+      if (group[d] >= 0) {
+        g = placed[d] + 1;  // after the launch that produces it
+      } else {
+        // a directly launched node at position d is on the stream before every group
+        // whose trigger comes after it
+        g = static_cast<int>(std::upper_bound(trigger.begin(), trigger.end(), d) - trigger.begin());
+      }
+      earliest = std::max(earliest, g);
+    }
+    const int home = group[i];
+    if (earliest >= home) continue;
+    const double w = live[i]->WorkEstimate() / kMacPerUs;
+    int best = home;
+    double best_delta = cost(load[home]) - cost(load[home] - w);
+    for (int g = home - 1; g >= earliest; --g) {
+      if (members[g] >= kMaxBatch) continue;
+      const double delta = cost(load[g] + w) - cost(load[g]);
+      if (delta < best_delta - 1e-9) {
+        best_delta = delta;
+        best = g;
+      }
+    }
+    if (best != home) {
+      load[home] -= w;
+      --members[home];
+      load[best] += w;
+      ++members[best];
+      placed[i] = best;
+      moved[best].push_back(i);
+    }
+  }
+
+  std::vector<bool> is_moved(n, false);
+  for (const auto& list : moved)
+    for (int i : list) is_moved[i] = true;
+  int g = 0;
+  for (int i = 0; i <= n; ++i) {
+    while (g < groups && trigger[g] == i) {
+      for (int m : moved[g]) order_.push_back(live[m]);
+      ++g;
+    }
+    if (i < n && !is_moved[i]) order_.push_back(live[i]);
+  }
+  CHECK_EQ(order_.size(), live.size());
+}
+
+std::vector<std::string> FBOSession::IssueOrder() const {
+  std::vector<std::string> names;
+  for (const Kernel* k : order_) names.push_back(k->kernel_name());
+  return names;
 }
 
 void FBOSession::Compute() {
   CHECK(finalized_) << "Please Setup Session First";
-  for (auto& kernel : kernels_) {
-    if (CheckKernelReady(kernel.get())) continue;
-    kernel->Compute();
-  }
+  for (Kernel* kernel : order_) kernel->Compute();
   context_->Flush();  // convolutions still deferred at the end of the pass
 }
 
@@ -152,9 +312,7 @@ void FBOSession::Run(const NamedTensorList& inputs_cpu) {
 void FBOSession::RunProfiled(std::vector<NodeTiming>* timings) {
   CHECK(finalized_) << "Please Setup Session First";
   hipStream_t s = static_cast<hipStream_t>(context_->stream());
-  std::vector<Kernel*> live;
-  for (auto& kernel : kernels_)
-    if (!CheckKernelReady(kernel.get())) live.push_back(kernel.get());
+  const std::vector<Kernel*>& live = order_;
   std::vector<hipEvent_t> ev(live.size() + 1);
   for (auto& e : ev) OGLE_HIP_CALL(hipEventCreate(&e));
   OGLE_HIP_CALL(hipEventRecord(ev[0], s));

@@ -7,7 +7,11 @@
 // subgraphs are computed once during Setup (the ready_ flags), only the first Run
 // allocates.  Additions for a launch-bound GPU: Compute() replays the kernels
 // without re-uploading inputs, RunProfiled() brackets every node with HIP events,
-// and CaptureGraph()/LaunchGraph() replay the whole run as one hipGraph.
+// CaptureGraph()/LaunchGraph() replay the whole run as one hipGraph, and the
+// convolutions whose results are not needed at once (the SSD heads) are issued
+// earlier than their place in the file, next to a convolution of the serial chain,
+// so that the two share one grid (set_reorder(false) or OGLE_FILE_ORDER=1 keeps
+// strict file order; results are the same either way).
 #ifndef OPENGL_CORE_FBO_SESSION_H_
 #define OPENGL_CORE_FBO_SESSION_H_
 
@@ -61,9 +65,16 @@ class FBOSession {
   void set_allow_resized(bool flag) { allow_resized_ = flag; }
   const IntList& default_input_sizes() const { return default_input_sizes_; }
   int num_kernels() const { return static_cast<int>(kernels_.size()); }
+  // Whether Setup may move deferrable convolutions ahead of their file position.
+  // Takes effect at the first Run.
+  void set_reorder(bool on) { reorder_ = on; }
+  bool reorder() const { return reorder_; }
+  // Node names in the order Compute() issues them (after the first Run).
+  std::vector<std::string> IssueOrder() const;
 
  private:
   bool CheckKernelReady(const Kernel* kernel);
+  void BuildSchedule();
   void UpdateKernelReady(const Kernel* kernel);
 
   Context* context_;
@@ -75,6 +86,8 @@ class FBOSession {
   NamedIndex tensor_name_index_;
   std::vector<bool> ready_;
   bool allow_resized_ = false;
+  bool reorder_ = true;
+  std::vector<Kernel*> order_;  // the per-pass kernels in issue order (not owned)
   IntList default_input_sizes_;
   void* graph_ = nullptr;       // hipGraph_t
   void* graph_exec_ = nullptr;  // hipGraphExec_t

@@ -9,6 +9,7 @@
 #ifndef OPENGL_CORE_KERNEL_H_
 #define OPENGL_CORE_KERNEL_H_
 
+#include <cstddef>
 #include <string>
 #include <vector>
 
@@ -64,6 +65,15 @@ class Kernel {
     (void)i;
     return -1;
   }
+
+  // Scheduling hints, also not in the reference (one draw call per node, in file
+  // order).  The launch of a deferrable node may be held back and merged with other
+  // deferrable nodes into one grid; WorkEstimate is its device work in multiply-adds
+  // including tile padding, ScratchBytes the workspace its launch plan wants.  Valid
+  // once the executor has bound the node's tensors.
+  virtual bool Deferrable() const { return false; }
+  virtual double WorkEstimate() const { return 0.0; }
+  virtual size_t ScratchBytes() const { return 0; }
 
  protected:
   Program* program_ = nullptr;  // not owned (the context owns programs)

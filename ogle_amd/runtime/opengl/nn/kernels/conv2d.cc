@@ -109,30 +109,53 @@ void Conv2DKernel::PackFilter(const Tensor* filter) {
   packed_from_ = filter->device_ptr();
 }
 
+void Conv2DKernel::FillGeometry(const Tensor* image, const Tensor* output, OgleConvArgs* a) const {
+  const IntList& in = image->shape();
+  const IntList& out = output->shape();
+  a->n = in[0]; a->in_h = in[1]; a->in_w = in[2]; a->in_c = in[3];
+  a->out_h = out[1]; a->out_w = out[2]; a->out_c = out[3];
+  a->kernel_size = kernel_size_; a->stride = stride_; a->padding = padding_;
+  a->dilation = dilation_; a->group = group_size_;
+  // "act" uniform: 1 clip, otherwise 2 for any non-empty activation (conv2d.cc:137-147).
+  a->act = activation_type_.empty() ? OGLE_ACT_NONE
+                                    : (activation_type_ == "Clip" ? OGLE_ACT_CLIP : OGLE_ACT_RELU);
+  a->min_value = min_;
+  a->max_value = max_;
+  a->act_variant = act_variant_;
+  a->dtype = OGLE_F32;
+}
+
+size_t Conv2DKernel::ScratchBytes() const {
+  if (workspace_need_ < 0) {
+    CHECK(!input_tensors_.empty() && !output_tensors_.empty()) << "tensors are not bound yet";
+    OgleConvArgs a{};
+    FillGeometry(input_tensors_[0], output_tensors_[0], &a);
+    workspace_need_ = static_cast<long>(ogle_hip_conv_workspace_bytes(&a));
+  }
+  return static_cast<size_t>(workspace_need_);
+}
+
+double Conv2DKernel::WorkEstimate() const {
+  if (input_tensors_.empty() || output_tensors_.empty()) return 0.0;
+  const IntList& in = input_tensors_[0]->shape();
+  const IntList& out = output_tensors_[0]->shape();
+  const double m = static_cast<double>(out[0]) * out[1] * out[2];
+  const double n = 32.0 * ((out[3] + 31) / 32);  // the MFMA tiles are at least 32 channels wide
+  return m * n * kernel_size_ * kernel_size_ * (in[3] / group_size_);
+}
+
 void Conv2DKernel::Compute(TensorList& inputs, TensorList& outputs) {
   program_->Activate();
   const Tensor* image = inputs[0];
   const Tensor* filter = inputs[1];
   if (!packed_filter_ || packed_from_ != filter->device_ptr()) PackFilter(filter);
 
-  const IntList& in = image->shape();
-  const IntList& out = outputs[0]->shape();
   OgleConvArgs a{};
+  FillGeometry(image, outputs[0], &a);
   a.input_dev = image->device_ptr();
   a.filter_dev = packed_filter_->device_ptr();
   a.bias_dev = inputs.size() > 2 ? static_cast<const float*>(inputs[2]->device_ptr()) : nullptr;
   a.output_dev = outputs[0]->device_ptr();
-  a.n = in[0]; a.in_h = in[1]; a.in_w = in[2]; a.in_c = in[3];
-  a.out_h = out[1]; a.out_w = out[2]; a.out_c = out[3];
-  a.kernel_size = kernel_size_; a.stride = stride_; a.padding = padding_;
-  a.dilation = dilation_; a.group = group_size_;
-  // "act" uniform: 1 clip, otherwise 2 for any non-empty activation (conv2d.cc:137-147).
-  a.act = activation_type_.empty() ? OGLE_ACT_NONE
-                                   : (activation_type_ == "Clip" ? OGLE_ACT_CLIP : OGLE_ACT_RELU);
-  a.min_value = min_;
-  a.max_value = max_;
-  a.act_variant = act_variant_;
-  a.dtype = OGLE_F32;
   if (variant_ != kDepthwise)
     context_->BeforeConv(a.input_dev, a.filter_dev, a.bias_dev, a.output_dev);
   if (workspace_need_ < 0) workspace_need_ = static_cast<long>(ogle_hip_conv_workspace_bytes(&a));

@@ -19,10 +19,15 @@ class Conv2DKernel : public Kernel {
   void InferOutputShape(TensorShapeList& inputs, TensorShapeList& outputs) override;
   void SetupAttr(const dlxnet::Attribute& attr) override;
   void SelectKernel(const TensorList& inputs) override;
+  bool Deferrable() const override { return variant_ != kDepthwise; }
+  double WorkEstimate() const override;
+  size_t ScratchBytes() const override;
 
  private:
   enum Variant { kDense, kDepthwise, kPointwise, kGrouped };
   void PackFilter(const Tensor* filter);
+  // Geometry, activation and dtype of the launch (no device pointers).
+  void FillGeometry(const Tensor* image, const Tensor* output, OgleConvArgs* a) const;
 
   int padding_ = 0;
   int stride_ = 1;
@@ -38,7 +43,7 @@ class Conv2DKernel : public Kernel {
   // constant the first time the node computes.
   std::unique_ptr<Tensor> packed_filter_;
   const void* packed_from_ = nullptr;
-  long workspace_need_ = -1;  // bytes of scratch the launch plan wants; -1 until asked
+  mutable long workspace_need_ = -1;  // bytes of scratch the launch plan wants; -1 until asked
 };
 
 }  // namespace opengl

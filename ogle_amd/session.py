@@ -22,6 +22,7 @@ SYMBOLS = [
     "ogle_rt_stream", "ogle_rt_get_output", "ogle_rt_num_kernels",
     "ogle_rt_registered_kernel_count", "ogle_rt_registered_kernel_name", "ogle_rt_detect",
     "ogle_rt_reserialize", "ogle_rt_model_debug_string", "ogle_rt_tensor_dformat",
+    "ogle_rt_set_reorder", "ogle_rt_issue_order_name",
 ]
 
 
@@ -73,6 +74,9 @@ def lib():
         l.ogle_rt_get_output.argtypes = [vp, cp, cp, vp, i64]
         l.ogle_rt_get_output.restype = i64
         l.ogle_rt_num_kernels.argtypes = [vp]
+        l.ogle_rt_set_reorder.argtypes = [vp, i32]
+        l.ogle_rt_issue_order_name.argtypes = [vp, i32]
+        l.ogle_rt_issue_order_name.restype = cp
         l.ogle_rt_registered_kernel_name.argtypes = [i32]
         l.ogle_rt_registered_kernel_name.restype = cp
         l.ogle_rt_detect.argtypes = [vp, vp, ctypes.POINTER(i32), cp, cp, cp, cp, ctypes.c_float,
@@ -206,6 +210,20 @@ class Session:
     @property
     def num_kernels(self):
         return lib().ogle_rt_num_kernels(self._h)
+
+    def set_reorder(self, on):
+        """Before the first run: False keeps the reference's strict file order."""
+        _check(lib().ogle_rt_set_reorder(self._h, 1 if on else 0))
+
+    def issue_order(self):
+        """Node names in the order a pass issues them (after the first run)."""
+        names, i = [], 0
+        while True:
+            p = lib().ogle_rt_issue_order_name(self._h, i)
+            if p is None:
+                return names
+            names.append(p.decode())
+            i += 1
 
     def get_output(self, name, dformat="ANY"):
         shape = self.tensor_shape(name)

@@ -204,7 +204,7 @@ def test_conv_batch_equals_single_launches():
         (4, 19, 19, 128, 12, 3, 1, 1), (4, 19, 19, 128, 63, 3, 1, 1), (4, 10, 10, 256, 24, 3, 1, 1),
         (4, 10, 10, 256, 126, 3, 1, 1), (4, 5, 5, 128, 126, 3, 1, 1), (4, 3, 3, 64, 24, 3, 1, 1),
         (2, 7, 7, 64, 96, 1, 1, 0), (2, 9, 9, 32, 40, 1, 1, 0), (1, 8, 8, 3, 8, 3, 2, 1),
-        (1, 6, 6, 6, 6, 3, 1, 1),
+        (1, 6, 6, 6, 6, 3, 1, 1), (2, 9, 9, 32, 24, 1, 1, 0), (16, 19, 19, 64, 64, 1, 1, 0),
     ]
     keep, single, args = [], [], (H.ConvArgs * len(cases))()
     for i, (n, h, w, c, o, k, st, p) in enumerate(cases):

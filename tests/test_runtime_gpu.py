@@ -256,6 +256,43 @@ def test_graph_replay_equals_eager_batch2():
     assert prof[0][0] == "conv0#Conv#"
 
 
+def test_reordered_issue_equals_file_order():
+    """The executor issues the SSD heads early, next to the feature-extractor chain, so that
+    they share launches.  The issue order must be a dependency-respecting permutation of the
+    file order, and every output must be bit-identical to a strict file-order run (eager and
+    replayed as a graph)."""
+    g, info = models.mobilenet_v1_ssd(2, seed=99, with_weights=True)
+    x = rng(100).uniform(-1, 1, (2, 300, 300, 3)).astype(np.float32)
+    outs = {}
+    orders = {}
+    for reorder in (False, True):
+        sess = session.Session()
+        sess.set_reorder(reorder)
+        sess.load_graph(g)
+        sess.run({"input": x})
+        orders[reorder] = sess.issue_order()
+        eager = {n: sess.get_output(n, "ANY") for n in ("box_preds", "cls_logits", "extra4.conv",
+                                                        "head0.conf", "head5.loc")}
+        sess.compute(graph=True)
+        sess.compute(graph=True)
+        for n, v in eager.items():
+            np.testing.assert_array_equal(sess.get_output(n, "ANY"), v)
+        outs[reorder] = eager
+    for n in outs[False]:
+        np.testing.assert_array_equal(outs[True][n], outs[False][n])
+    file_order, issued = orders[False], orders[True]
+    assert sorted(file_order) == sorted(issued) and file_order != issued
+    pos = {n: i for i, n in enumerate(issued)}
+    # heads move ahead of (part of) the extras chain, never ahead of their feature map
+    assert pos["head0.conf"] < pos["extra4.conv"]
+    for i, feat in enumerate(["block11.pw", "block13.pw", "extra1.conv", "extra2.conv",
+                              "extra3.conv", "extra4.conv"]):
+        assert pos["head%d.loc" % i] > pos[feat] and pos["head%d.conf" % i] > pos[feat]
+    # everything that is not a head keeps its relative order
+    rest = [n for n in issued if not n.startswith("head")]
+    assert rest == [n for n in file_order if not n.startswith("head")]
+
+
 def test_detector_matches_oracle_pipeline():
     """Detector::Detect: graph -> decode + score filter (device) -> top-k -> NMS, against the
     oracle's restatement of GenerateBoxInfo / GetTopK / NMS fed with the device's own logits and
