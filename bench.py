@@ -105,6 +105,127 @@ def read_traffic_summary(kernel_family):
     return None
 
 
+def kernel_table(iters=50, warm=5):
+    """Each kernel of the path on its own, at the shapes the baseline configurations name,
+    called through the C ABI on torch's current stream and timed with events on that stream.
+    FLOPs = 2 x multiply-adds; bytes = input + weights + bias + output once each."""
+    import ctypes
+    import torch
+    from ogle_amd import hip as H
+    L = H.lib()
+    st = torch.cuda.current_stream().cuda_stream
+    rows = []
+
+    def timed(fn):
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(iters):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / iters * 1e3  # microseconds per call
+
+    def row(name, us, flops, nbytes, bound, peak_tflops=MFMA_F32_PEAK_TFLOPS):
+        tf, gb = flops / us / 1e6, nbytes / us / 1e3
+        rows.append(dict(kernel=name, us=round(us, 2), tflops=round(tf, 2), gbs=round(gb, 1),
+                         bound=bound, peak=HBM_PEAK_GBS if bound == "hbm" else peak_tflops,
+                         frac=round(gb / HBM_PEAK_GBS if bound == "hbm" else tf / peak_tflops, 4)))
+
+    def conv_problem(n, h, w, c, o, k, s, p, g=1, dtype=H.F32, act=H.ACT_RELU, maxv=0.0):
+        tdt = torch.float16 if dtype == H.F16 else torch.float32
+        x = torch.rand(n, h, w, c, device="cuda").to(tdt)
+        dw = g == c and g != 1
+        src = torch.randn(o, c // g, k, k, device="cuda") * 0.05
+        wd = torch.empty(src.numel(), dtype=tdt, device="cuda")
+        H.check(L.ogle_hip_pack_filter(src.data_ptr(), wd.data_ptr(),
+                                       H.FILTER_HWC if dw else H.FILTER_OHWI, dtype, o, c // g, k, k, st))
+        b = torch.rand(o, device="cuda")
+        oh, ow = H.out_size(h, k, s, p), H.out_size(w, k, s, p)
+        y = torch.empty(n, oh, ow, o, device="cuda", dtype=tdt)
+        a = H.conv_args(x.data_ptr(), wd.data_ptr(), b.data_ptr(), y.data_ptr(), n, h, w, c, o, k, s,
+                        p, 1, g, act, 0.0, maxv, H.VARIANT_NHWC4, dtype)
+        need = L.ogle_hip_conv_workspace_bytes(ctypes.byref(a))
+        ws = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
+        if need:
+            a.workspace_dev, a.workspace_bytes = ws.data_ptr(), need
+        esz = 2 if dtype == H.F16 else 4
+        flops = 2.0 * n * oh * ow * o * (c // g) * k * k
+        nbytes = esz * (x.numel() + wd.numel() + y.numel()) + 4 * o
+        return a, flops, nbytes, (x, wd, b, y, ws)
+
+    def conv_row(name, entry, bound, *shape, peak=MFMA_F32_PEAK_TFLOPS, **kw):
+        a, flops, nbytes, keep = conv_problem(*shape, **kw)
+        f = getattr(L, entry)
+        row(name, timed(lambda: H.check(f(ctypes.byref(a), st))), flops, nbytes, bound, peak)
+
+    conv_row("dense 3x3 @C1 (1x112x112x32->64)", "ogle_hip_conv2d", "mfma", 1, 112, 112, 32, 64, 3, 1, 1)
+    for b in (1, 8):
+        conv_row("depthwise 3x3 @C2 b%d (38x38x256)" % b, "ogle_hip_dwconv2d", "hbm",
+                 b, 38, 38, 256, 256, 3, 1, 1, g=256, act=H.ACT_CLIP, maxv=6.0)
+        conv_row("pointwise @C2 b%d (M=%d K=256 N=512)" % (b, b * 1444), "ogle_hip_pwconv_gemm", "mfma",
+                 b, 38, 38, 256, 512, 1, 1, 0, act=H.ACT_CLIP, maxv=6.0)
+    conv_row("pointwise GEMM @C3 fp32 (M=11552 K=512 N=1024)", "ogle_hip_pwconv_gemm", "mfma",
+             32, 19, 19, 512, 1024, 1, 1, 0)
+    conv_row("pointwise GEMM @C3 fp16 storage, fp32 accumulate", "ogle_hip_pwconv_gemm", "mfma",
+             32, 19, 19, 512, 1024, 1, 1, 0, dtype=H.F16, peak=2500.0)
+
+    # C4: the twelve SSD head convolutions of 64 images in one grouped call
+    maps = [(19, 512, 3), (10, 1024, 6), (5, 512, 6), (3, 256, 6), (2, 256, 6), (1, 128, 6)]
+    probs = []
+    for m, c, anchors in maps:
+        probs.append(conv_problem(64, m, m, c, anchors * 4, 3, 1, 1, act=H.ACT_NONE))
+        probs.append(conv_problem(64, m, m, c, anchors * 21, 3, 1, 1, act=H.ACT_NONE))
+    arr = (H.ConvArgs * len(probs))(*[q[0] for q in probs])
+    row("SSD heads @C4 b64 (12 convs, one grouped call)",
+        timed(lambda: H.check(L.ogle_hip_conv2d_batch(arr, len(probs), st))),
+        sum(q[1] for q in probs), sum(q[2] for q in probs), "mfma")
+
+    # concat @C4: six maps -> (64, 1917, 4) and (64, 1917, 21)
+    for width, label in ((4, "loc"), (21, "conf")):
+        lens = [m * m * a for m, _, a in maps]
+        ins = [torch.rand(64, n, width, device="cuda") for n in lens]
+        out = torch.empty(64, sum(lens), width, device="cuda")
+        ca = H.ConcatArgs()
+        for i, t in enumerate(ins):
+            ca.inputs_dev[i] = t.data_ptr()
+            ca.axis_len[i] = lens[i]
+        ca.output_dev, ca.n_inputs, ca.outer, ca.inner, ca.dtype = out.data_ptr(), len(ins), 64, width, H.F32
+        row("concat @C4 b64 %s (6 inputs)" % label, timed(lambda: H.check(L.ogle_hip_concat(ctypes.byref(ca), st))),
+            0.0, 2.0 * out.numel() * 4, "hbm")
+
+    # decode + softmax-max + score filter @C4
+    batch, priors, classes = 64, 1917, 21
+    logits = torch.randn(batch, priors, classes, device="cuda") * 2
+    pred = torch.randn(batch, priors, 4, device="cuda")
+    anchors = torch.rand(priors, 4, device="cuda")
+    i32 = dict(dtype=torch.int32, device="cuda")
+    boxes = torch.empty(batch, priors, 4, device="cuda")
+    cnt, kp, kc = torch.zeros(batch, **i32), torch.zeros(batch, priors, **i32), torch.zeros(batch, priors, **i32)
+    ks, kb = torch.empty(batch, priors, device="cuda"), torch.empty(batch, priors, 4, device="cuda")
+    kr = torch.zeros(batch, priors, 4, **i32)
+    da = H.DetectArgs(logits.data_ptr(), pred.data_ptr(), anchors.data_ptr(), boxes.data_ptr(), batch,
+                      priors, classes, 0, (ctypes.c_float * 4)(0.1, 0.1, 0.2, 0.2), 0.3, 300.0, 300.0,
+                      cnt.data_ptr(), kp.data_ptr(), kc.data_ptr(), ks.data_ptr(), kb.data_ptr(),
+                      kr.data_ptr())
+    row("SSD decode + score filter @C4 b64", timed(lambda: H.check(L.ogle_hip_ssd_detect(ctypes.byref(da), st))),
+        0.0, batch * (161028 + 30672 + 30672 + 15336) + 30672, "hbm")
+
+    # pooling parity shapes
+    for name, n, h, c, k, s, p, typ in (("max-pool 3x3 s2 p1 (1x112x112x64)", 1, 112, 64, 3, 2, 1, 0),
+                                        ("max-pool 3x3 s2 p1 (16x112x112x64)", 16, 112, 64, 3, 2, 1, 0),
+                                        ("avg-pool 2x2 s2 (16x112x112x64)", 16, 112, 64, 2, 2, 0, 1)):
+        x = torch.rand(n, h, h, c, device="cuda")
+        oh = H.out_size(h, k, s, p)
+        y = torch.empty(n, oh, oh, c, device="cuda")
+        pa = H.PoolArgs(x.data_ptr(), y.data_ptr(), n, h, h, c, oh, oh, k, s, p, typ, H.F32)
+        row(name, timed(lambda: H.check(L.ogle_hip_pool2d(ctypes.byref(pa), st))), 0.0,
+            4.0 * (x.numel() + y.numel()), "hbm")
+    return rows
+
+
 def cpu_baseline(seed=20240005, images=2, repeats=1):
     """The oracle (CPU restatement of the reference's arithmetic) on the host cores: every conv
     layer of the network, concat and the decode + score filter, for `images` images."""
@@ -158,6 +279,8 @@ def main():
     ap.add_argument("--batch", type=int, default=16)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--eager", action="store_true", help="launch kernel by kernel instead of a hipGraph")
+    ap.add_argument("--skip-kernel-table", action="store_true",
+                    help="leave out the per-kernel leg at the single-kernel configurations")
     ap.add_argument("--skip-b1", action="store_true",
                     help="leave out the batch-1 latency leg (keeps a profiler trace to the batch-16 pass)")
     args = ap.parse_args()
@@ -218,6 +341,8 @@ def main():
         "kernels": fams,
         "non_conv_ms_per_step": round(other_ms, 4),
     }
+    if not args.skip_kernel_table:
+        result["kernel_table"] = kernel_table()
     result["calibration_copy_bytes"] = calibration_copy()
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline()

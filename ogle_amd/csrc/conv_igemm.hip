@@ -533,17 +533,27 @@ IgemmPlan plan_igemm(const OgleConvArgs& a, long m, bool allow_split) {
   }
   p.splits = 1;
   const long t = tiles(p.cfg);
+  long sp = 1;
   if (allow_split && 2 * t <= kComputeUnits && p.ktiles >= 8) {
-    long want = (3 * kComputeUnits + t - 1) / t;   // about three workgroups per unit
-    long most = p.ktiles / 4;                      // at least four slabs per split
-    long sp = want < most ? want : most;
-    if (sp > 64) sp = 64;
-    // the kernel's XCD-aware work layout wants a divisor or a multiple of 8
-    if (sp >= 8) sp -= sp % 8;
-    else if (sp >= 4) sp = 4;
-    else if (sp >= 2) sp = 2;
-    if (sp >= 2) p.splits = (int)sp;
+    // too few tiles to occupy every compute unit: about three workgroups per unit,
+    // at least four slabs per split
+    const long want = (3 * kComputeUnits + t - 1) / t;
+    const long most = p.ktiles / 4;
+    sp = want < most ? want : most;
+  } else if (allow_split && t < 8 * kComputeUnits && p.ktiles >= 128) {
+    // a few long workgroups per unit quantise badly (one unit gets two, its
+    // neighbour one) and leave one wave per SIMD: cut the long contraction so that
+    // about eight shorter workgroups land on every unit, 32 slabs or more each
+    const long want = (8 * kComputeUnits + t - 1) / t;
+    const long most = p.ktiles / 32;
+    sp = want < most ? want : most;
   }
+  if (sp > 64) sp = 64;
+  // the kernel's XCD-aware work layout wants a divisor or a multiple of 8
+  if (sp >= 8) sp -= sp % 8;
+  else if (sp >= 4) sp = 4;
+  else if (sp >= 2) sp = 2;
+  if (sp >= 2) p.splits = (int)sp;
   p.slabs_per_split = (p.ktiles + p.splits - 1) / p.splits;
   if (p.splits > 1) p.slabs_per_split += p.slabs_per_split & 1;  // the K loop runs slab pairs
   // (a split past the end of K would only add zeros; rounding splits down keeps the
