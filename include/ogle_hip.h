@@ -308,6 +308,42 @@ typedef struct OgleDetectArgs {
 
 int32_t ogle_hip_ssd_detect(const OgleDetectArgs* args, ogle_stream_t stream);
 
+/*
+ * Top-k by score, then NMS, per image, on the lists ogle_hip_ssd_detect leaves
+ * on the device: Detector::GetTopK + Detector::NMS
+ * (ogl_runtime/opengl/examples/ssd/detector.cc:114-148) with iou() of
+ * examples/ssd/common.cc:57-77 on the integer rectangles.
+ *   - order: score descending; entries with equal scores keep their order in the
+ *     kept list (ascending prior index).  The reference's std::sort leaves the
+ *     order of equal scores unspecified; this is the stable choice.
+ *   - the first min(count, topk) entries go to NMS: entry j is dropped if any
+ *     earlier entry i has iou(i, j) > nms_threshold (strict), whether or not i
+ *     was itself dropped (detector.cc:130-141).
+ * Inputs are indexed [b*stride + r], r < kept_count_dev[b]; outputs
+ * [b*topk + r], r < final_count_dev[b], in sorted order.  kept_box_dev /
+ * final_box_dev may both be NULL.  1 <= topk <= 1024; stride <= 8192.
+ */
+typedef struct OgleNmsArgs {
+  const int32_t* kept_count_dev;
+  const int32_t* kept_prior_dev;
+  const int32_t* kept_class_dev;
+  const float* kept_score_dev;
+  const float* kept_box_dev;
+  const int32_t* kept_rect_dev;
+  int32_t batch;
+  int32_t stride; /* entries per image in the kept_* arrays (= priors) */
+  int32_t topk;
+  float nms_threshold;
+  int32_t* final_count_dev;
+  int32_t* final_prior_dev;
+  int32_t* final_class_dev;
+  float* final_score_dev;
+  float* final_box_dev;
+  int32_t* final_rect_dev;
+} OgleNmsArgs;
+
+int32_t ogle_hip_ssd_topk_nms(const OgleNmsArgs* args, ogle_stream_t stream);
+
 /* y[i] = exp(x[i]) exactly as ogle_hip_ssd_detect evaluates it; lets a test
  * compare the device exponential with the host's on the same inputs. */
 int32_t ogle_hip_expf(const float* x_dev, float* y_dev, int64_t count, ogle_stream_t stream);

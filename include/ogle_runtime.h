@@ -126,10 +126,14 @@ typedef struct OgleDetection {
 /*
  * Detector::Detect (examples/ssd/detector.cc:275-295) on a loaded session: runs the
  * graph on `images` (host NHWC floats, already preprocessed), decodes and filters
- * on the device, then top-k and NMS.  Tensor names are cls_logits / box_preds /
+ * on the device, then top-k and NMS (device or host, ogle_rt_set_device_nms).  Tensor names are cls_logits / box_preds /
  * anchors unless overridden (NULL keeps the default).  Writes up to `capacity`
  * detections, returns how many there are in total.
  */
+/* Top-k + NMS of ogle_rt_detect / ogle_rt_time_compute on the device (default, 1) or on
+ * the host as in the reference (0).  Same detections either way. */
+int32_t ogle_rt_set_device_nms(OgleSession* s, int32_t on);
+
 int64_t ogle_rt_detect(OgleSession* s, const float* images, const int32_t* dims /* n,h,w,c */,
                        const char* input_name, const char* cls_name, const char* box_name,
                        const char* anchors_name, float score_threshold, float nms_threshold,

@@ -348,6 +348,27 @@ int32_t ogle_hip_ssd_detect(const OgleDetectArgs* a, ogle_stream_t stream) {
   return launch_detect(*a, as_stream(stream));
 }
 
+int32_t ogle_hip_ssd_topk_nms(const OgleNmsArgs* a, ogle_stream_t stream) {
+  if (a == nullptr) return fail(OGLE_ERR_INVALID_ARG, "ssd_topk_nms: null args");
+  if (a->batch < 0 || a->stride < 0) return fail(OGLE_ERR_INVALID_ARG, "ssd_topk_nms: bad size");
+  if (a->topk < 1 || a->topk > 1024)
+    return fail(OGLE_ERR_UNSUPPORTED, "ssd_topk_nms: topk must be in 1..1024");
+  if (a->stride > 8192)  // scores of one image are staged in LDS
+    return fail(OGLE_ERR_UNSUPPORTED, "ssd_topk_nms: more than 8192 entries per image");
+  if (a->batch > 0) {
+    if (!a->kept_count_dev || !a->final_count_dev)
+      return fail(OGLE_ERR_INVALID_ARG, "ssd_topk_nms: count pointers are required");
+    if (a->stride > 0 && (!a->kept_prior_dev || !a->kept_class_dev || !a->kept_score_dev ||
+                          !a->kept_rect_dev))
+      return fail(OGLE_ERR_INVALID_ARG, "ssd_topk_nms: null input list");
+    if (!a->final_prior_dev || !a->final_class_dev || !a->final_score_dev || !a->final_rect_dev)
+      return fail(OGLE_ERR_INVALID_ARG, "ssd_topk_nms: null output list");
+    if ((a->kept_box_dev == nullptr) != (a->final_box_dev == nullptr))
+      return fail(OGLE_ERR_INVALID_ARG, "ssd_topk_nms: kept_box_dev and final_box_dev go together");
+  }
+  return launch_topk_nms(*a, as_stream(stream));
+}
+
 int32_t ogle_hip_expf(const float* x_dev, float* y_dev, int64_t count, ogle_stream_t stream) {
   if (count < 0 || (count > 0 && (!x_dev || !y_dev)))
     return fail(OGLE_ERR_INVALID_ARG, "expf: null pointer or negative count");

@@ -245,7 +245,254 @@ __global__ __launch_bounds__(256) void ssd_compact_kernel(DetectParams p) {
   if (tid == 0) p.kept_count[b] = base;
 }
 
+// Top-k by score and the reference's NMS for one image per workgroup
+// (Detector::GetTopK + Detector::NMS, detector.cc:114-148; iou, common.cc:57-77).
+//   order : score descending; equal scores keep their order in the kept list
+//           (ascending prior index), which is what a stable sort gives
+//   NMS   : entry j is dropped if ANY earlier entry i of the top-k list has
+//           iou(i, j) > threshold, whether or not i was itself dropped
+// IoU is evaluated on the integer rectangles in fp32, operation by operation as the
+// host does (no FMA contraction), so kept sets are bit-identical.
+#pragma clang fp contract(off)
+__device__ __forceinline__ float rect_iou(const int4& a, const int4& b) {
+  const float xmin0 = (float)a.x, ymin0 = (float)a.y;
+  const float xmax0 = (float)(a.x + a.z), ymax0 = (float)(a.y + a.w);
+  const float xmin1 = (float)b.x, ymin1 = (float)b.y;
+  const float xmax1 = (float)(b.x + b.z), ymax1 = (float)(b.y + b.w);
+  const float w = fmaxf(0.0f, fminf(xmax0, xmax1) - fmaxf(xmin0, xmin1));
+  const float h = fmaxf(0.0f, fminf(ymax0, ymax1) - fmaxf(ymin0, ymin1));
+  const float i = w * h;
+  if (i == 0.0f) return 0.0f;  // disjoint: the host gets 0 / u or its u <= 0 case, both 0
+  const float u = (xmax0 - xmin0) * (ymax0 - ymin0) + (xmax1 - xmin1) * (ymax1 - ymin1) - i;
+  if (u <= 0.0f) return 0.0f;
+  return i / u;
+}
+
+struct NmsParams {
+  const int* kept_count;
+  const int* kept_prior;
+  const int* kept_class;
+  const float* kept_score;
+  const float4* kept_box;
+  const int4* kept_rect;
+  int stride, topk;
+  float threshold;
+  int* out_count;
+  int* out_prior;
+  int* out_class;
+  float* out_score;
+  float4* out_box;
+  int4* out_rect;
+};
+
+// Score bits mapped so that unsigned order equals float order (negative values too).
+__device__ __forceinline__ unsigned ordered_bits(float v) {
+  const unsigned b = __float_as_uint(v);
+  return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+
+// Steps of the kernel, one workgroup per image with n kept entries:
+//   1. radix select (four 8-bit passes over the ordered score bits) finds the value
+//      of the k-th largest score and how many entries equal to it belong to the
+//      top k; of equal scores the first ones in list order are taken
+//   2. ordered compaction gathers the min(n, k) selected entries in list order
+//   3. their rank under (score descending, list position ascending) is counted among
+//      the selected entries only, which sorts them
+//   4. NMS over all pairs of the sorted list, then an ordered compaction of the
+//      survivors
+__global__ __launch_bounds__(256) void ssd_topk_nms_kernel(NmsParams p) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char nms_lds[];
+  // keys[stride] | cand_key[topk+4] | cand_idx[topk+4] | sel[topk] | rect[topk] | hist[256] | misc[8]
+  const int tpad = (p.topk + 3) & ~3;
+  unsigned* keys = reinterpret_cast<unsigned*>(nms_lds);
+  unsigned* cand_key = keys + ((p.stride + 3) & ~3);
+  int* cand_idx = reinterpret_cast<int*>(cand_key + tpad);
+  int* sel = cand_idx + tpad;
+  int4* rects = reinterpret_cast<int4*>(sel + tpad);
+  int* hist = reinterpret_cast<int*>(rects + p.topk);
+  int* misc = hist + 256;  // [0..3] wave counts, [4] chosen digit, [5] entries above it
+
+  const int b = blockIdx.x;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const long row0 = (long)b * p.stride;
+  int n = p.kept_count[b];
+  n = n < 0 ? 0 : (n > p.stride ? p.stride : n);
+  for (int i = tid; i < n; i += 256) keys[i] = ordered_bits(p.kept_score[row0 + i]);
+  __syncthreads();
+
+  // 1. the k-th largest key
+  const int m = n < p.topk ? n : p.topk;
+  unsigned prefix = 0, mask = 0;
+  int remaining = m;  // how many of the entries matching `prefix` are still wanted
+  if (n > p.topk) {
+    for (int shift = 24; shift >= 0; shift -= 8) {
+      hist[tid] = 0;
+      __syncthreads();
+      for (int i = tid; i < n; i += 256) {
+        const unsigned k = keys[i];
+        if ((k & mask) == prefix) atomicAdd(&hist[(k >> shift) & 255u], 1);
+      }
+      __syncthreads();
+      // thread t: entries whose digit is above t, and at or above t (suffix sums of
+      // the histogram: a shuffle scan inside each wave plus the totals of later waves)
+      const int mine = hist[tid];
+      int sfx = mine;
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const int v = __shfl_down(sfx, d, 64);
+        if (lane + d < 64) sfx += v;
+      }
+      if (lane == 0) misc[wave] = sfx;
+      __syncthreads();
+      int at_or_above = sfx;
+      for (int wv = wave + 1; wv < 4; ++wv) at_or_above += misc[wv];
+      const int above = at_or_above - mine;
+      if (above < remaining && remaining <= at_or_above) {
+        misc[4] = tid;
+        misc[5] = above;
+      }
+      __syncthreads();
+      prefix |= (unsigned)misc[4] << shift;
+      mask |= 255u << shift;
+      remaining -= misc[5];
+      __syncthreads();  // misc and hist are rewritten by the next pass
+    }
+  }
+  // now: take every key above `prefix`, and the first `remaining` equal to it
+  // (n <= topk: prefix = 0, mask = 0, every key is "above or equal", all are taken)
+
+  // 2. ordered compaction of the selected entries
+  {
+    int taken = 0, equal_seen = 0;
+    for (int start = 0; start < n; start += 256) {
+      const int i = start + tid;
+      const unsigned k = i < n ? keys[i] : 0u;
+      const bool gt = i < n && (n <= p.topk || k > prefix);
+      const bool eq = i < n && n > p.topk && k == prefix;
+      const unsigned long long eq_ballot = __ballot(eq);
+      if (lane == 0) misc[wave] = __popcll(eq_ballot);
+      __syncthreads();
+      int eq_before = equal_seen + __popcll(eq_ballot & ((1ull << lane) - 1ull));
+      for (int wv = 0; wv < wave; ++wv) eq_before += misc[wv];
+      const int eq_total = misc[0] + misc[1] + misc[2] + misc[3];
+      __syncthreads();
+      const bool take = gt || (eq && eq_before < remaining);
+      const unsigned long long ballot = __ballot(take);
+      if (lane == 0) misc[wave] = __popcll(ballot);
+      __syncthreads();
+      int before = taken + __popcll(ballot & ((1ull << lane) - 1ull));
+      for (int wv = 0; wv < wave; ++wv) before += misc[wv];
+      const int total = misc[0] + misc[1] + misc[2] + misc[3];
+      if (take) {
+        cand_key[before] = k;
+        cand_idx[before] = i;
+      }
+      taken += total;
+      equal_seen += eq_total;
+      __syncthreads();
+    }
+  }
+  for (int r = m + tid; r < ((m + 3) & ~3); r += 256) cand_key[r] = 0u;  // padding ranks last
+  __syncthreads();
+
+  // 3. rank among the selected entries (they are in list order, so position breaks ties)
+  const int mpad = (m + 3) & ~3;
+  for (int r = tid; r < m; r += 256) {
+    const unsigned kr = cand_key[r];
+    int rank = 0;
+    for (int j = 0; j < mpad; j += 4) {
+      const uint4 v = *reinterpret_cast<const uint4*>(cand_key + j);
+      rank += (v.x > kr || (v.x == kr && j + 0 < r)) ? 1 : 0;
+      rank += (v.y > kr || (v.y == kr && j + 1 < r)) ? 1 : 0;
+      rank += (v.z > kr || (v.z == kr && j + 2 < r)) ? 1 : 0;
+      rank += (v.w > kr || (v.w == kr && j + 3 < r)) ? 1 : 0;
+    }
+    sel[rank] = cand_idx[r];
+  }
+  __syncthreads();
+  for (int r = tid; r < m; r += 256) rects[r] = p.kept_rect[row0 + sel[r]];
+  __syncthreads();
+
+  // 4. NMS: all (i, j) pairs with i < j are spread over the workgroup; a pair that
+  // overlaps by more than the threshold marks j (every writer stores the same value)
+  int* dropped = cand_idx;  // the candidate list is no longer needed
+  for (int r = tid; r < m; r += 256) dropped[r] = 0;
+  __syncthreads();
+  if (m > 1) {
+    // pair number t = i * m + j, advanced by 256 per step without dividing
+    const int step_i = 256 / m, step_j = 256 - step_i * m;
+    int i = tid / m, j = tid - i * m;
+    for (; i < m; i += step_i, j += step_j) {
+      if (j >= m) {
+        j -= m;
+        ++i;
+        if (i >= m) break;
+      }
+      if (i >= j) continue;
+      if (rect_iou(rects[i], rects[j]) > p.threshold) dropped[j] = 1;
+    }
+  }
+  __syncthreads();
+
+  // ordered compaction of the survivors into the output lists
+  int base = 0;
+  const long out0 = (long)b * p.topk;
+  for (int start = 0; start < m; start += 256) {
+    const int j = start + tid;
+    const bool keep = j < m && dropped[j] == 0;
+    const unsigned long long ballot = __ballot(keep);
+    const int before = __popcll(ballot & ((1ull << lane) - 1ull));
+    if (lane == 0) misc[wave] = __popcll(ballot);
+    __syncthreads();
+    int wave_base = 0;
+    for (int wv = 0; wv < wave; ++wv) wave_base += misc[wv];
+    const int chunk_total = misc[0] + misc[1] + misc[2] + misc[3];
+    if (keep) {
+      const long src = row0 + sel[j];
+      const long dst = out0 + base + wave_base + before;
+      p.out_prior[dst] = p.kept_prior[src];
+      p.out_class[dst] = p.kept_class[src];
+      p.out_score[dst] = p.kept_score[src];
+      if (p.out_box != nullptr) p.out_box[dst] = p.kept_box[src];
+      p.out_rect[dst] = rects[j];
+    }
+    base += chunk_total;
+    __syncthreads();
+  }
+  if (tid == 0) p.out_count[b] = base;
+}
+
 }  // namespace
+
+size_t topk_nms_lds_bytes(int stride, int topk) {
+  const size_t tpad = (size_t)((topk + 3) & ~3);
+  return 4 * (size_t)((stride + 3) & ~3) + 4 * 3 * tpad + sizeof(int4) * (size_t)topk +
+         4 * (256 + 8);
+}
+
+int32_t launch_topk_nms(const OgleNmsArgs& a, hipStream_t s) {
+  if (a.batch == 0) return OGLE_OK;
+  NmsParams p{};
+  p.kept_count = a.kept_count_dev;
+  p.kept_prior = a.kept_prior_dev;
+  p.kept_class = a.kept_class_dev;
+  p.kept_score = a.kept_score_dev;
+  p.kept_box = reinterpret_cast<const float4*>(a.kept_box_dev);
+  p.kept_rect = reinterpret_cast<const int4*>(a.kept_rect_dev);
+  p.stride = a.stride;
+  p.topk = a.topk;
+  p.threshold = a.nms_threshold;
+  p.out_count = a.final_count_dev;
+  p.out_prior = a.final_prior_dev;
+  p.out_class = a.final_class_dev;
+  p.out_score = a.final_score_dev;
+  p.out_box = reinterpret_cast<float4*>(a.final_box_dev);
+  p.out_rect = reinterpret_cast<int4*>(a.final_rect_dev);
+  hipLaunchKernelGGL(ssd_topk_nms_kernel, dim3((unsigned)a.batch), dim3(256),
+                     topk_nms_lds_bytes(a.stride, a.topk), s, p);
+  return check_launch("ssd_topk_nms_kernel");
+}
 
 int32_t launch_decode(const OgleDecodeArgs& a, hipStream_t s) {
   const long total = (long)a.batch * a.priors;

@@ -26,7 +26,7 @@ SYMBOLS = [
     "ogle_hip_convert", "ogle_hip_conv2d", "ogle_hip_dwconv2d", "ogle_hip_pwconv_gemm",
     "ogle_hip_pool2d", "ogle_hip_concat", "ogle_hip_ssd_decode", "ogle_hip_ssd_detect",
     "ogle_hip_expf", "ogle_hip_transpose", "ogle_hip_conv_workspace_bytes",
-    "ogle_hip_conv2d_batch",
+    "ogle_hip_conv2d_batch", "ogle_hip_ssd_topk_nms",
 ]
 
 
@@ -99,6 +99,19 @@ class DetectArgs(ctypes.Structure):
     ]
 
 
+class NmsArgs(ctypes.Structure):
+    _fields_ = [
+        ("kept_count_dev", ctypes.c_void_p), ("kept_prior_dev", ctypes.c_void_p),
+        ("kept_class_dev", ctypes.c_void_p), ("kept_score_dev", ctypes.c_void_p),
+        ("kept_box_dev", ctypes.c_void_p), ("kept_rect_dev", ctypes.c_void_p),
+        ("batch", ctypes.c_int32), ("stride", ctypes.c_int32), ("topk", ctypes.c_int32),
+        ("nms_threshold", ctypes.c_float),
+        ("final_count_dev", ctypes.c_void_p), ("final_prior_dev", ctypes.c_void_p),
+        ("final_class_dev", ctypes.c_void_p), ("final_score_dev", ctypes.c_void_p),
+        ("final_box_dev", ctypes.c_void_p), ("final_rect_dev", ctypes.c_void_p),
+    ]
+
+
 _lib = None
 
 
@@ -128,6 +141,7 @@ def lib():
                           ("ogle_hip_pwconv_gemm", ConvArgs), ("ogle_hip_pool2d", PoolArgs),
                           ("ogle_hip_concat", ConcatArgs), ("ogle_hip_ssd_decode", DecodeArgs),
                           ("ogle_hip_ssd_detect", DetectArgs),
+                          ("ogle_hip_ssd_topk_nms", NmsArgs),
                           ("ogle_hip_transpose", TransposeArgs)):
             getattr(l, name).argtypes = [ctypes.POINTER(typ), ctypes.c_void_p]
         l.ogle_hip_conv2d_batch.argtypes = [ctypes.POINTER(ConvArgs), ctypes.c_int32, ctypes.c_void_p]

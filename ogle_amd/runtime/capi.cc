@@ -22,6 +22,7 @@ struct OgleSession {
   std::unique_ptr<FBOSession> session;
   std::vector<opengl::NodeTiming> timings;
   std::unique_ptr<opengl::Detector> detector;
+  bool device_nms = true;
 };
 
 namespace {
@@ -131,6 +132,7 @@ int32_t ogle_rt_time_compute(OgleSession* s, int32_t warmup, int32_t iters, int3
   return (int32_t)Guard([&]() -> int64_t {
     hipStream_t st = static_cast<hipStream_t>(s->context->stream());
     opengl::DetectorOptions opt;
+    opt.device_nms = s->device_nms;
     if (with_detect && !s->detector) s->detector = opengl::Detector::Create(s->session.get(), opt);
     auto pass = [&]() {
       if (use_graph) {
@@ -139,7 +141,10 @@ int32_t ogle_rt_time_compute(OgleSession* s, int32_t warmup, int32_t iters, int3
       } else {
         s->session->Compute();
       }
-      if (with_detect) s->detector->EnqueuePostprocess(opt.output_names, 300, 300);
+      if (with_detect) {
+        s->detector->EnqueuePostprocess(opt.output_names, 300, 300);
+        if (s->detector->UsesDeviceNms()) s->detector->EnqueueTopkNms();
+      }
       if (sync_each) s->context->Finish();
     };
     for (int i = 0; i < warmup; ++i) pass();
@@ -277,6 +282,12 @@ int64_t ogle_rt_model_debug_string(const void* data, size_t size, char* out, int
 
 int32_t ogle_rt_num_kernels(OgleSession* s) { return s->session->num_kernels(); }
 
+int32_t ogle_rt_set_device_nms(OgleSession* s, int32_t on) {
+  s->device_nms = on != 0;
+  s->detector.reset();
+  return 0;
+}
+
 int32_t ogle_rt_set_reorder(OgleSession* s, int32_t on) {
   return (int32_t)Guard([&]() -> int64_t {
     s->session->set_reorder(on != 0);
@@ -318,6 +329,7 @@ int64_t ogle_rt_detect(OgleSession* s, const float* images, const int32_t* dims,
     opt.score_threshold = score_threshold;
     opt.nms_threshold = nms_threshold;
     opt.topk = topk;
+    opt.device_nms = s->device_nms;
     s->detector = opengl::Detector::Create(s->session.get(), opt);
     opengl::IntList shape(dims, dims + 4);
     Tensor input(Tensor::DT_FLOAT, shape, images, dlxnet::TensorProto::NHWC);

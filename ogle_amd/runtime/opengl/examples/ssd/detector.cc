@@ -63,6 +63,7 @@ void Detector::EnqueuePostprocess(const TensorNameList& names, int raw_width, in
 
   if (batch != batch_ || priors != priors_ || classes != classes_) {
     batch_ = batch; priors_ = priors; classes_ = classes;
+    final_topk_ = 0;
     auto dev = [](IntList shape) {
       return std::unique_ptr<Tensor>(
           new Tensor(Tensor::DT_FLOAT, shape, Tensor::DEVICE_BUFFER, dlxnet::TensorProto::ANY4));
@@ -120,27 +121,105 @@ void Detector::Readback() {
   session_->context()->Finish();
 }
 
+namespace {
+// One BoxInfo from entry `s` of the (prior, class, score, box, rect) arrays
+// (detector.cc:211-225).
+BoxInfo MakeBoxInfo(size_t s, const std::vector<int32_t>& prior, const std::vector<int32_t>& cls,
+                    const std::vector<float>& score, const std::vector<float>& box,
+                    const std::vector<int32_t>& rect) {
+  BoxInfo info;
+  const float xmin = box[s * 4 + 0], ymin = box[s * 4 + 1];
+  const float xmax = box[s * 4 + 2], ymax = box[s * 4 + 3];
+  info.box.x = rect[s * 4 + 0];
+  info.box.y = rect[s * 4 + 1];
+  info.box.width = rect[s * 4 + 2];
+  info.box.height = rect[s * 4 + 3];
+  info.cx = static_cast<float>((xmin + xmax) / 2.0);
+  info.cy = static_cast<float>((ymin + ymax) / 2.0);
+  info.height = static_cast<float>(info.box.height);  // detector.cc:220-221
+  info.width = static_cast<float>(info.box.width);
+  info.score = score[s];
+  info.class_name = cls[s];
+  info.index = prior[s];
+  return info;
+}
+}  // namespace
+
 void Detector::GenerateBoxInfo(int image, std::vector<BoxInfo>* box_infos) const {
   CHECK(image >= 0 && image < batch_);
   box_infos->clear();
   const size_t base = static_cast<size_t>(image) * priors_;
-  for (int r = 0; r < count_[image]; ++r) {
-    const size_t s = base + r;
-    BoxInfo info;
-    const float xmin = box_[s * 4 + 0], ymin = box_[s * 4 + 1];
-    const float xmax = box_[s * 4 + 2], ymax = box_[s * 4 + 3];
-    info.box.x = rect_[s * 4 + 0];
-    info.box.y = rect_[s * 4 + 1];
-    info.box.width = rect_[s * 4 + 2];
-    info.box.height = rect_[s * 4 + 3];
-    info.cx = static_cast<float>((xmin + xmax) / 2.0);
-    info.cy = static_cast<float>((ymin + ymax) / 2.0);
-    info.height = static_cast<float>(info.box.height);  // detector.cc:220-221
-    info.width = static_cast<float>(info.box.width);
-    info.score = score_[s];
-    info.class_name = class_[s];
-    info.index = prior_[s];
-    box_infos->push_back(info);
+  for (int r = 0; r < count_[image]; ++r)
+    box_infos->push_back(MakeBoxInfo(base + r, prior_, class_, score_, box_, rect_));
+}
+
+bool Detector::UsesDeviceNms() const {
+  return options_.device_nms && options_.topk >= 1 && options_.topk <= 1024 && priors_ <= 8192;
+}
+
+void Detector::EnqueueTopkNms() {
+  CHECK(batch_ > 0) << "EnqueuePostprocess first";
+  const int topk = options_.topk;
+  if (final_topk_ != topk) {
+    final_topk_ = topk;
+    auto dev = [](IntList shape) {
+      return std::unique_ptr<Tensor>(
+          new Tensor(Tensor::DT_FLOAT, shape, Tensor::DEVICE_BUFFER, dlxnet::TensorProto::ANY4));
+    };
+    fcount_dev_ = dev({batch_});
+    fprior_dev_ = dev({batch_, topk});
+    fclass_dev_ = dev({batch_, topk});
+    fscore_dev_ = dev({batch_, topk});
+    fbox_dev_ = dev({batch_, topk, 4});
+    frect_dev_ = dev({batch_, topk, 4});
+    fcount_.resize(batch_);
+    fprior_.resize(static_cast<size_t>(batch_) * topk);
+    fclass_.resize(fprior_.size());
+    fscore_.resize(fprior_.size());
+    fbox_.resize(fprior_.size() * 4);
+    frect_.resize(fprior_.size() * 4);
+  }
+  OgleNmsArgs a{};
+  a.kept_count_dev = static_cast<const int32_t*>(count_dev_->device_ptr());
+  a.kept_prior_dev = static_cast<const int32_t*>(prior_dev_->device_ptr());
+  a.kept_class_dev = static_cast<const int32_t*>(class_dev_->device_ptr());
+  a.kept_score_dev = static_cast<const float*>(score_dev_->device_ptr());
+  a.kept_box_dev = static_cast<const float*>(box_dev_->device_ptr());
+  a.kept_rect_dev = static_cast<const int32_t*>(rect_dev_->device_ptr());
+  a.batch = batch_;
+  a.stride = priors_;
+  a.topk = topk;
+  a.nms_threshold = options_.nms_threshold;
+  a.final_count_dev = static_cast<int32_t*>(fcount_dev_->device_ptr());
+  a.final_prior_dev = static_cast<int32_t*>(fprior_dev_->device_ptr());
+  a.final_class_dev = static_cast<int32_t*>(fclass_dev_->device_ptr());
+  a.final_score_dev = static_cast<float*>(fscore_dev_->device_ptr());
+  a.final_box_dev = static_cast<float*>(fbox_dev_->device_ptr());
+  a.final_rect_dev = static_cast<int32_t*>(frect_dev_->device_ptr());
+  hipStream_t s = static_cast<hipStream_t>(session_->context()->stream());
+  const int32_t st = ogle_hip_ssd_topk_nms(&a, s);
+  if (st != OGLE_OK) LOG(FATAL) << "ogle_hip_ssd_topk_nms: " << ogle_hip_last_error();
+}
+
+void Detector::ReadbackFinal(std::vector<std::vector<BoxInfo>>* final_boxes) {
+  CHECK(final_topk_ > 0) << "EnqueueTopkNms first";
+  hipStream_t s = static_cast<hipStream_t>(session_->context()->stream());
+  auto back = [&](void* dst, const Tensor* src, size_t bytes) {
+    const hipError_t e = hipMemcpyAsync(dst, src->device_ptr(), bytes, hipMemcpyDeviceToHost, s);
+    if (e != hipSuccess) LOG(FATAL) << "readback: " << hipGetErrorString(e);
+  };
+  back(fcount_.data(), fcount_dev_.get(), fcount_.size() * 4);
+  back(fprior_.data(), fprior_dev_.get(), fprior_.size() * 4);
+  back(fclass_.data(), fclass_dev_.get(), fclass_.size() * 4);
+  back(fscore_.data(), fscore_dev_.get(), fscore_.size() * 4);
+  back(fbox_.data(), fbox_dev_.get(), fbox_.size() * 4);
+  back(frect_.data(), frect_dev_.get(), frect_.size() * 4);
+  session_->context()->Finish();
+  final_boxes->assign(batch_, {});
+  for (int b = 0; b < batch_; ++b) {
+    const size_t base = static_cast<size_t>(b) * final_topk_;
+    for (int r = 0; r < fcount_[b]; ++r)
+      (*final_boxes)[b].push_back(MakeBoxInfo(base + r, fprior_, fclass_, fscore_, fbox_, frect_));
   }
 }
 
@@ -166,7 +245,13 @@ void Detector::NMS(std::vector<BoxInfo>& boxes, std::vector<BoxInfo>& boxes_left
 void Detector::Detect(const Tensor* images, int raw_width, int raw_height,
                       std::vector<std::vector<BoxInfo>>* final_boxes) {
   Run(images);
-  LoadToOutputTensors(options_.output_names, raw_width, raw_height);
+  EnqueuePostprocess(options_.output_names, raw_width, raw_height);
+  if (UsesDeviceNms()) {
+    EnqueueTopkNms();
+    ReadbackFinal(final_boxes);
+    return;
+  }
+  Readback();
   final_boxes->assign(batch_, {});
   for (int b = 0; b < batch_; ++b) {
     std::vector<BoxInfo> infos;

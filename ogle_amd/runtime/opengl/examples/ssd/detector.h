@@ -1,5 +1,6 @@
-// SSD detector driver: runs the graph, decodes boxes and filters scores on the
-// device, then top-k and NMS on the host.  Counterpart of
+// SSD detector driver: runs the graph, then decode + score filter and top-k + NMS
+// on the device (or, with device_nms off, top-k + NMS on the host as the reference
+// does); one readback of the final lists.  Counterpart of
 // ogl_runtime/opengl/examples/ssd/detector.{h,cc} without the OpenCV image I/O:
 // the caller passes preprocessed float images (NHWC) and the size the boxes are
 // scaled to.  Unlike the reference, which post-processes the first image only
@@ -36,6 +37,10 @@ struct DetectorOptions {
   float nms_threshold = 0.45f;
   float score_threshold = 0.3f;
   int topk = 100;
+  // Top-k + NMS on the device (ogle_hip_ssd_topk_nms) instead of the host loop of
+  // detector.cc:114-148; same results, and only the final lists are read back.
+  // Needs topk <= 1024 and at most 8192 priors; the host path is used otherwise.
+  bool device_nms = true;
   std::vector<float> variances = {0.1f, 0.1f, 0.2f, 0.2f};
   TensorNameList input_names = {"input"};
   TensorNameList output_names = {"cls_logits", "box_preds", "anchors"};
@@ -63,6 +68,11 @@ class Detector {
   // allocated on first use) and the readback of its compacted results (synchronises).
   void EnqueuePostprocess(const TensorNameList& names, int raw_width, int raw_height);
   void Readback();
+  // Device top-k + NMS over what EnqueuePostprocess left on the device
+  // (asynchronous), and the readback of its final lists (synchronises).
+  void EnqueueTopkNms();
+  void ReadbackFinal(std::vector<std::vector<BoxInfo>>* final_boxes);
+  bool UsesDeviceNms() const;
   void GenerateBoxInfo(int image, std::vector<BoxInfo>* box_infos) const;
   static void GetTopK(std::vector<BoxInfo>& input, int top_k);
   static void NMS(std::vector<BoxInfo>& boxes, std::vector<BoxInfo>& boxes_left, float threshold);
@@ -80,6 +90,11 @@ class Detector {
       rect_dev_;
   std::vector<int32_t> count_, prior_, class_, rect_;
   std::vector<float> score_, box_;
+  // final lists of the device top-k + NMS: (batch, topk) each
+  int final_topk_ = 0;
+  std::unique_ptr<Tensor> fcount_dev_, fprior_dev_, fclass_dev_, fscore_dev_, fbox_dev_, frect_dev_;
+  std::vector<int32_t> fcount_, fprior_, fclass_, frect_;
+  std::vector<float> fscore_, fbox_;
 };
 
 float iou(const Rect& box0, const Rect& box1);

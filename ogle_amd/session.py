@@ -22,7 +22,7 @@ SYMBOLS = [
     "ogle_rt_stream", "ogle_rt_get_output", "ogle_rt_num_kernels",
     "ogle_rt_registered_kernel_count", "ogle_rt_registered_kernel_name", "ogle_rt_detect",
     "ogle_rt_reserialize", "ogle_rt_model_debug_string", "ogle_rt_tensor_dformat",
-    "ogle_rt_set_reorder", "ogle_rt_issue_order_name",
+    "ogle_rt_set_reorder", "ogle_rt_issue_order_name", "ogle_rt_set_device_nms",
 ]
 
 
@@ -75,6 +75,7 @@ def lib():
         l.ogle_rt_get_output.restype = i64
         l.ogle_rt_num_kernels.argtypes = [vp]
         l.ogle_rt_set_reorder.argtypes = [vp, i32]
+        l.ogle_rt_set_device_nms.argtypes = [vp, i32]
         l.ogle_rt_issue_order_name.argtypes = [vp, i32]
         l.ogle_rt_issue_order_name.restype = cp
         l.ogle_rt_registered_kernel_name.argtypes = [i32]
@@ -210,6 +211,10 @@ class Session:
     @property
     def num_kernels(self):
         return lib().ogle_rt_num_kernels(self._h)
+
+    def set_device_nms(self, on):
+        """Top-k + NMS of detect() on the device (default) or on the host."""
+        _check(lib().ogle_rt_set_device_nms(self._h, 1 if on else 0))
 
     def set_reorder(self, on):
         """Before the first run: False keeps the reference's strict file order."""

@@ -14,7 +14,8 @@ import pytest
 
 import oracle as O
 from ogle_amd import hip as H
-from util import (assert_conv_close, gpu_concat, gpu_conv, gpu_decode, gpu_detect, gpu_pool, rng)
+from util import (assert_conv_close, gpu_concat, gpu_conv, gpu_decode, gpu_detect, gpu_pool,
+                  gpu_topk_nms, rng)
 
 pytestmark = pytest.mark.gpu
 
@@ -444,3 +445,48 @@ def test_concat_ssd_shapes_batch64():
     for last in (4, 21):
         ins = [r.normal(0, 1, (64, p, last)).astype(np.float32) for p in (1083, 600, 150, 54, 24, 6)]
         np.testing.assert_array_equal(gpu_concat(ins, 1), np.concatenate(ins, 1))
+
+
+@pytest.mark.parametrize("seed,stride,topk,spread", [
+    (1, 1917, 100, 300), (2, 1917, 100, 40), (3, 257, 16, 60), (4, 64, 100, 30), (5, 1917, 1024, 200),
+    (6, 8192, 200, 500), (7, 5, 1, 10),
+])
+def test_topk_nms_matches_oracle(seed, stride, topk, spread):
+    """Device top-k + NMS against the oracle's restatement of GetTopK + NMS (detector.cc:114-148):
+    quantised scores force ties (stable order = prior order), rectangles cluster so that many
+    overlap, include zero-area and negative-size boxes, and one image is empty, one full."""
+    r = rng(9000 + seed)
+    batch = 5
+    counts = np.array([0, stride, min(stride, 3), stride // 2, min(stride, 131)], np.int32)
+    prior = np.zeros((batch, stride), np.int32)
+    cls = r.integers(1, 21, (batch, stride)).astype(np.int32)
+    score = (r.integers(301, 1000, (batch, stride)) / 1000.0).astype(np.float32)   # many equal scores
+    score[3] = r.uniform(0.3, 1.0, stride).astype(np.float32)                      # and one image without ties
+    xy = r.integers(-20, spread, (batch, stride, 2))
+    wh = r.integers(-3, 80, (batch, stride, 2))
+    rect = np.concatenate([xy, wh], -1).astype(np.int32)
+    box = r.uniform(0, 300, (batch, stride, 4)).astype(np.float32)
+    for b in range(batch):
+        prior[b, :counts[b]] = np.sort(r.choice(max(stride, 1) * 3, counts[b], replace=False))
+    got = gpu_topk_nms(counts, prior, cls, score, rect, topk, 0.45, box)
+    for b in range(batch):
+        n = counts[b]
+        keep = O.topk_nms(score[b, :n], rect[b, :n], topk, 0.45)
+        np.testing.assert_array_equal(got[b]["prior"], prior[b, :n][keep])
+        np.testing.assert_array_equal(got[b]["cls"], cls[b, :n][keep])
+        np.testing.assert_array_equal(got[b]["score"], score[b, :n][keep])
+        np.testing.assert_array_equal(got[b]["rect"], rect[b, :n][keep])
+        np.testing.assert_array_equal(got[b]["box"], box[b, :n][keep])
+
+
+def test_topk_nms_rejects_bad_sizes():
+    import ctypes
+    a = H.NmsArgs()
+    a.batch, a.stride, a.topk = 1, 100, 0
+    assert H.lib().ogle_hip_ssd_topk_nms(ctypes.byref(a), 0) == H.ERR_UNSUPPORTED
+    a.topk = 2000
+    assert H.lib().ogle_hip_ssd_topk_nms(ctypes.byref(a), 0) == H.ERR_UNSUPPORTED
+    a.topk, a.stride = 10, 10000
+    assert H.lib().ogle_hip_ssd_topk_nms(ctypes.byref(a), 0) == H.ERR_UNSUPPORTED
+    a.stride = 100
+    assert H.lib().ogle_hip_ssd_topk_nms(ctypes.byref(a), 0) == H.ERR_INVALID_ARG   # null pointers

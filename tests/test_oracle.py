@@ -298,7 +298,9 @@ def test_topk_nms_against_python_restatement():
         u = (ax1 - ax0) * (ay1 - ay0) + (bx1 - bx0) * (by1 - by0) - i
         return 0.0 if u <= 0 else i / u
 
-    for top_k in (100, 25):
+    for top_k, ties in ((100, False), (25, False), (100, True), (7, True)):
+        if ties:  # equal scores keep their input order (the defined choice for std::sort's ties)
+            scores = (r.integers(3, 9, n) / 10.0).astype(np.float32)
         order = sorted(range(n), key=lambda i: (-scores[i], i))[:top_k]
         dropped = [False] * len(order)
         for i in range(len(order) - 1):

@@ -293,14 +293,17 @@ def test_reordered_issue_equals_file_order():
     assert rest == [n for n in file_order if not n.startswith("head")]
 
 
-def test_detector_matches_oracle_pipeline():
-    """Detector::Detect: graph -> decode + score filter (device) -> top-k -> NMS, against the
-    oracle's restatement of GenerateBoxInfo / GetTopK / NMS fed with the device's own logits and
-    box predictions.  Head weights ~N(0, 0.05) give logits wide enough that priors pass."""
+@pytest.mark.parametrize("device_nms", [True, False])
+def test_detector_matches_oracle_pipeline(device_nms):
+    """Detector::Detect: graph -> decode + score filter (device) -> top-k -> NMS (device, or the
+    host loop the reference uses), against the oracle's restatement of GenerateBoxInfo / GetTopK /
+    NMS fed with the device's own logits and box predictions.  Head weights ~N(0, 0.05) give
+    logits wide enough that priors pass."""
     batch = 2
     g, info = models.mobilenet_v1_ssd(batch, seed=31, head_std=0.05)
     x = rng(32).uniform(-1, 1, (batch, 300, 300, 3)).astype(np.float32)
     sess = session.Session()
+    sess.set_device_nms(device_nms)
     sess.load_graph(g)
     dets = sess.detect(x, 640, 480, 0.3, 0.45, 100)
     conf = sess.get_output("cls_logits", "ANY")

@@ -165,6 +165,41 @@ def gpu_detect(logits, pred, anchors, threshold=0.3, image_w=1.0, image_h=1.0,
     return res, boxes.cpu().numpy()
 
 
+def gpu_topk_nms(counts, prior, cls, score, rect, topk, threshold, box=None):
+    """Per-image lists (batch, stride[, 4]) as ogle_hip_ssd_detect leaves them -> per-image dict
+    of the final lists of ogle_hip_ssd_topk_nms."""
+    torch = _torch()
+    batch, stride = prior.shape
+    i32 = dict(dtype=torch.int32, device="cuda")
+    cd, pd, kd = dev(counts.astype(np.int32)), dev(prior.astype(np.int32)), dev(cls.astype(np.int32))
+    sd, rd = dev(score.astype(np.float32)), dev(rect.astype(np.int32))
+    bd = dev(box.astype(np.float32)) if box is not None else None
+    fc = torch.full((batch,), -7, **i32)
+    fp = torch.full((batch, topk), -7, **i32)
+    fk = torch.full((batch, topk), -7, **i32)
+    fs = torch.full((batch, topk), float("nan"), dtype=torch.float32, device="cuda")
+    fr = torch.full((batch, topk, 4), -7, **i32)
+    fb = torch.full((batch, topk, 4), float("nan"), dtype=torch.float32, device="cuda") if box is not None else None
+    a = H.NmsArgs(cd.data_ptr(), pd.data_ptr(), kd.data_ptr(), sd.data_ptr(),
+                  bd.data_ptr() if bd is not None else None, rd.data_ptr(), batch, stride, topk,
+                  threshold, fc.data_ptr(), fp.data_ptr(), fk.data_ptr(), fs.data_ptr(),
+                  fb.data_ptr() if fb is not None else None, fr.data_ptr())
+    H.check(H.lib().ogle_hip_ssd_topk_nms(ctypes.byref(a), stream_ptr()))
+    torch.cuda.synchronize()
+    n = fc.cpu().numpy()
+    out = []
+    for b in range(batch):
+        k = int(n[b])
+        d = dict(prior=fp[b, :k].cpu().numpy(), cls=fk[b, :k].cpu().numpy(),
+                 score=fs[b, :k].cpu().numpy(), rect=fr[b, :k].cpu().numpy())
+        if fb is not None:
+            d["box"] = fb[b, :k].cpu().numpy()
+        # nothing past the count may have been written
+        assert (fp[b, k:] == -7).all() and (fr[b, k:] == -7).all()
+        out.append(d)
+    return out
+
+
 def assert_conv_close(got, ref, scale, rtol, what=""):
     """The fp32 / fp16 parity rule for contractions.
 
