@@ -140,6 +140,14 @@ int64_t ogle_rt_detect(OgleSession* s, const float* images, const int32_t* dims 
                        int32_t topk, int32_t raw_width, int32_t raw_height, OgleDetection* out,
                        int64_t capacity);
 
+/*
+ * The detections of the detector work most recently enqueued on the session's
+ * stream (by ogle_rt_time_compute with with_detect, eagerly or inside its graph):
+ * waits for the stream, reads the lists back and, with host NMS selected, finishes
+ * them on the host.  Same output convention as ogle_rt_detect.
+ */
+int64_t ogle_rt_detect_results(OgleSession* s, OgleDetection* out, int64_t capacity);
+
 #ifdef __cplusplus
 }
 #endif

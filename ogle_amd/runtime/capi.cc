@@ -134,16 +134,26 @@ int32_t ogle_rt_time_compute(OgleSession* s, int32_t warmup, int32_t iters, int3
     opengl::DetectorOptions opt;
     opt.device_nms = s->device_nms;
     if (with_detect && !s->detector) s->detector = opengl::Detector::Create(s->session.get(), opt);
+    auto detect = [&]() {
+      s->detector->EnqueuePostprocess(opt.output_names, 300, 300);
+      if (s->detector->UsesDeviceNms()) s->detector->EnqueueTopkNms();
+    };
+    if (with_detect) {
+      detect();  // first use allocates the result buffers: keep that out of a capture
+      s->context->Finish();
+    }
+    // slot 0: the pass alone; slot 1: the pass followed by the detector's device work
+    const int slot = with_detect ? 1 : 0;
     auto pass = [&]() {
       if (use_graph) {
-        if (!s->session->graph_captured()) s->session->CaptureGraph();
-        s->session->LaunchGraph();
+        if (!s->session->graph_captured(slot)) {
+          if (with_detect) s->session->CaptureGraph(slot, detect);
+          else s->session->CaptureGraph(slot);
+        }
+        s->session->LaunchGraph(slot);
       } else {
         s->session->Compute();
-      }
-      if (with_detect) {
-        s->detector->EnqueuePostprocess(opt.output_names, 300, 300);
-        if (s->detector->UsesDeviceNms()) s->detector->EnqueueTopkNms();
+        if (with_detect) detect();
       }
       if (sync_each) s->context->Finish();
     };
@@ -283,9 +293,12 @@ int64_t ogle_rt_model_debug_string(const void* data, size_t size, char* out, int
 int32_t ogle_rt_num_kernels(OgleSession* s) { return s->session->num_kernels(); }
 
 int32_t ogle_rt_set_device_nms(OgleSession* s, int32_t on) {
-  s->device_nms = on != 0;
-  s->detector.reset();
-  return 0;
+  return (int32_t)Guard([&]() -> int64_t {
+    s->device_nms = on != 0;
+    s->session->DropGraph(1);
+    s->detector.reset();
+    return 0;
+  });
 }
 
 int32_t ogle_rt_set_reorder(OgleSession* s, int32_t on) {
@@ -315,6 +328,27 @@ const char* ogle_rt_registered_kernel_name(int32_t i) {
   return name.c_str();
 }
 
+namespace {
+int64_t CopyDetections(const std::vector<std::vector<opengl::BoxInfo>>& result, OgleDetection* out,
+                       int64_t capacity) {
+  int64_t n = 0;
+  for (size_t b = 0; b < result.size(); ++b)
+    for (const auto& info : result[b]) {
+      if (n < capacity) {
+        OgleDetection& d = out[n];
+        d.image = (int32_t)b;
+        d.prior = info.index;
+        d.class_id = info.class_name;
+        d.score = info.score;
+        d.x = info.box.x; d.y = info.box.y; d.width = info.box.width; d.height = info.box.height;
+        d.cx = info.cx; d.cy = info.cy;
+      }
+      ++n;
+    }
+  return n;
+}
+}  // namespace
+
 int64_t ogle_rt_detect(OgleSession* s, const float* images, const int32_t* dims,
                        const char* input_name, const char* cls_name, const char* box_name,
                        const char* anchors_name, float score_threshold, float nms_threshold,
@@ -330,26 +364,28 @@ int64_t ogle_rt_detect(OgleSession* s, const float* images, const int32_t* dims,
     opt.nms_threshold = nms_threshold;
     opt.topk = topk;
     opt.device_nms = s->device_nms;
+    // a graph recorded with the previous detector's buffers must not outlive them
+    s->session->DropGraph(1);
     s->detector = opengl::Detector::Create(s->session.get(), opt);
     opengl::IntList shape(dims, dims + 4);
     Tensor input(Tensor::DT_FLOAT, shape, images, dlxnet::TensorProto::NHWC);
     std::vector<std::vector<opengl::BoxInfo>> result;
     s->detector->Detect(&input, raw_width, raw_height, &result);
-    int64_t n = 0;
-    for (size_t b = 0; b < result.size(); ++b)
-      for (const auto& info : result[b]) {
-        if (n < capacity) {
-          OgleDetection& d = out[n];
-          d.image = (int32_t)b;
-          d.prior = info.index;
-          d.class_id = info.class_name;
-          d.score = info.score;
-          d.x = info.box.x; d.y = info.box.y; d.width = info.box.width; d.height = info.box.height;
-          d.cx = info.cx; d.cy = info.cy;
-        }
-        ++n;
-      }
-    return n;
+    return CopyDetections(result, out, capacity);
+  });
+}
+
+int64_t ogle_rt_detect_results(OgleSession* s, OgleDetection* out, int64_t capacity) {
+  return Guard([&]() -> int64_t {
+    CHECK(s->detector != nullptr) << "no detector work has been enqueued on this session";
+    std::vector<std::vector<opengl::BoxInfo>> result;
+    if (s->detector->UsesDeviceNms()) {
+      s->detector->ReadbackFinal(&result);
+    } else {
+      s->detector->Readback();
+      s->detector->HostTopkNms(&result);
+    }
+    return CopyDetections(result, out, capacity);
   });
 }
 

@@ -29,8 +29,11 @@ FBOSession::FBOSession(Context* context) : context_(context) {
 }
 
 FBOSession::~FBOSession() {
-  if (graph_exec_ != nullptr) (void)hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph_exec_));
-  if (graph_ != nullptr) (void)hipGraphDestroy(static_cast<hipGraph_t>(graph_));
+  for (int i = 0; i < kGraphSlots; ++i) {
+    if (graph_exec_[i] != nullptr)
+      (void)hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph_exec_[i]));
+    if (graph_[i] != nullptr) (void)hipGraphDestroy(static_cast<hipGraph_t>(graph_[i]));
+  }
   // Views must go before the buffers they alias; both are plain frees, so order
   // only matters for tidiness: release in reverse creation order.
   for (auto it = total_tensors_.rbegin(); it != total_tensors_.rend(); ++it) it->reset();
@@ -332,15 +335,20 @@ void FBOSession::RunProfiled(std::vector<NodeTiming>* timings) {
   for (auto& e : ev) (void)hipEventDestroy(e);
 }
 
-void FBOSession::CaptureGraph() {
+void FBOSession::CaptureGraph(int slot, const std::function<void()>& after_pass) {
   CHECK(finalized_) << "Please Setup Session First";
-  if (graph_exec_ != nullptr) return;
+  CHECK(slot >= 0 && slot < kGraphSlots) << "graph slot";
+  if (graph_exec_[slot] != nullptr) return;
   hipStream_t s = static_cast<hipStream_t>(context_->stream());
   OGLE_HIP_CALL(hipStreamSynchronize(s));
   hipGraph_t graph = nullptr;
   OGLE_HIP_CALL(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal));
   try {
     Compute();
+    if (after_pass) {
+      after_pass();
+      context_->Flush();
+    }
   } catch (...) {
     (void)hipStreamEndCapture(s, &graph);
     if (graph != nullptr) (void)hipGraphDestroy(graph);
@@ -349,13 +357,23 @@ void FBOSession::CaptureGraph() {
   OGLE_HIP_CALL(hipStreamEndCapture(s, &graph));
   hipGraphExec_t exec = nullptr;
   OGLE_HIP_CALL(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0));
-  graph_ = graph;
-  graph_exec_ = exec;
+  graph_[slot] = graph;
+  graph_exec_[slot] = exec;
 }
 
-void FBOSession::LaunchGraph() {
-  CHECK(graph_exec_ != nullptr) << "CaptureGraph first";
-  OGLE_HIP_CALL(hipGraphLaunch(static_cast<hipGraphExec_t>(graph_exec_),
+void FBOSession::DropGraph(int slot) {
+  CHECK(slot >= 0 && slot < kGraphSlots) << "graph slot";
+  if (graph_exec_[slot] == nullptr) return;
+  context_->Finish();
+  (void)hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph_exec_[slot]));
+  (void)hipGraphDestroy(static_cast<hipGraph_t>(graph_[slot]));
+  graph_exec_[slot] = nullptr;
+  graph_[slot] = nullptr;
+}
+
+void FBOSession::LaunchGraph(int slot) {
+  CHECK(slot >= 0 && slot < kGraphSlots && graph_exec_[slot] != nullptr) << "CaptureGraph first";
+  OGLE_HIP_CALL(hipGraphLaunch(static_cast<hipGraphExec_t>(graph_exec_[slot]),
                                static_cast<hipStream_t>(context_->stream())));
 }
 

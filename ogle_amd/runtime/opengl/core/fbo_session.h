@@ -15,6 +15,7 @@
 #ifndef OPENGL_CORE_FBO_SESSION_H_
 #define OPENGL_CORE_FBO_SESSION_H_
 
+#include <functional>
 #include <string>
 #include <vector>
 
@@ -48,10 +49,16 @@ class FBOSession {
   // Compute() with a HIP event pair around every node; returns after the pass.
   void RunProfiled(std::vector<NodeTiming>* timings);
 
-  // Records one Compute() pass into a hipGraph (once) and replays it.
-  void CaptureGraph();
-  void LaunchGraph();
-  bool graph_captured() const { return graph_exec_ != nullptr; }
+  // Records one Compute() pass into a hipGraph (once per slot) and replays it.
+  // `after_pass`, if given, enqueues more work on the context's stream (a detector's
+  // post-processing) that is recorded into the same graph; it must not allocate.
+  static constexpr int kGraphSlots = 2;
+  void CaptureGraph(int slot = 0, const std::function<void()>& after_pass = {});
+  void LaunchGraph(int slot = 0);
+  bool graph_captured(int slot = 0) const { return graph_exec_[slot] != nullptr; }
+  // Forgets a recorded graph (after the stream has drained), e.g. because buffers
+  // its `after_pass` work used are about to be released.
+  void DropGraph(int slot);
 
   void GetOutputs(const TensorNameList& output_names, const StringList& output_dformats,
                   TensorList* outputs);
@@ -89,8 +96,8 @@ class FBOSession {
   bool reorder_ = true;
   std::vector<Kernel*> order_;  // the per-pass kernels in issue order (not owned)
   IntList default_input_sizes_;
-  void* graph_ = nullptr;       // hipGraph_t
-  void* graph_exec_ = nullptr;  // hipGraphExec_t
+  void* graph_[kGraphSlots] = {nullptr, nullptr};       // hipGraph_t
+  void* graph_exec_[kGraphSlots] = {nullptr, nullptr};  // hipGraphExec_t
 };
 
 }  // namespace opengl

@@ -252,6 +252,10 @@ void Detector::Detect(const Tensor* images, int raw_width, int raw_height,
     return;
   }
   Readback();
+  HostTopkNms(final_boxes);
+}
+
+void Detector::HostTopkNms(std::vector<std::vector<BoxInfo>>* final_boxes) const {
   final_boxes->assign(batch_, {});
   for (int b = 0; b < batch_; ++b) {
     std::vector<BoxInfo> infos;

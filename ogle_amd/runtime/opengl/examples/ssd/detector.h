@@ -73,6 +73,9 @@ class Detector {
   void EnqueueTopkNms();
   void ReadbackFinal(std::vector<std::vector<BoxInfo>>* final_boxes);
   bool UsesDeviceNms() const;
+  // The reference's host loop over what Readback() fetched: GenerateBoxInfo, GetTopK,
+  // NMS per image.
+  void HostTopkNms(std::vector<std::vector<BoxInfo>>* final_boxes) const;
   void GenerateBoxInfo(int image, std::vector<BoxInfo>* box_infos) const;
   static void GetTopK(std::vector<BoxInfo>& input, int top_k);
   static void NMS(std::vector<BoxInfo>& boxes, std::vector<BoxInfo>& boxes_left, float threshold);

@@ -23,6 +23,7 @@ SYMBOLS = [
     "ogle_rt_registered_kernel_count", "ogle_rt_registered_kernel_name", "ogle_rt_detect",
     "ogle_rt_reserialize", "ogle_rt_model_debug_string", "ogle_rt_tensor_dformat",
     "ogle_rt_set_reorder", "ogle_rt_issue_order_name", "ogle_rt_set_device_nms",
+    "ogle_rt_detect_results",
 ]
 
 
@@ -83,6 +84,8 @@ def lib():
         l.ogle_rt_detect.argtypes = [vp, vp, ctypes.POINTER(i32), cp, cp, cp, cp, ctypes.c_float,
                                      ctypes.c_float, i32, i32, i32, ctypes.POINTER(Detection), i64]
         l.ogle_rt_detect.restype = i64
+        l.ogle_rt_detect_results.argtypes = [vp, ctypes.POINTER(Detection), i64]
+        l.ogle_rt_detect_results.restype = i64
         l.ogle_rt_reserialize.argtypes = [vp, ctypes.c_size_t, vp, i64]
         l.ogle_rt_reserialize.restype = i64
         l.ogle_rt_model_debug_string.argtypes = [vp, ctypes.c_size_t, vp, i64]
@@ -253,8 +256,18 @@ class Session:
                                         input_name.encode() if input_name else None, names[0],
                                         names[1], names[2], score_threshold, nms_threshold, topk,
                                         raw_width, raw_height, buf, capacity))
-        per_image = [[] for _ in range(images.shape[0])]
+        return self._per_image(buf, n, capacity, images.shape[0])
+
+    @staticmethod
+    def _per_image(buf, n, capacity, batch):
+        per_image = [[] for _ in range(batch)]
         for d in buf[:min(n, capacity)]:
             per_image[d.image].append(dict(prior=d.prior, cls=d.class_id, score=d.score,
                                            rect=(d.x, d.y, d.width, d.height), cx=d.cx, cy=d.cy))
         return per_image
+
+    def detect_results(self, batch, capacity=4096):
+        """Detections of the detector work last enqueued by time_compute(with_detect=True)."""
+        buf = (Detection * capacity)()
+        n = _check(lib().ogle_rt_detect_results(self._h, buf, capacity))
+        return self._per_image(buf, n, capacity, batch)

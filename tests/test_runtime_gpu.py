@@ -322,3 +322,22 @@ def test_detector_matches_oracle_pipeline(device_nms):
         assert np.abs(got_rect - exp_rect).max(initial=0) <= 1   # 1e-4 in coordinates can move a truncation
         total += len(got_prior)
     assert total > 0
+
+
+@pytest.mark.parametrize("device_nms", [True, False])
+def test_detector_inside_graph_equals_eager(device_nms):
+    """time_compute(with_detect) records the detector's device work behind the pass in one
+    hipGraph; its detections after several replays must equal Detector::Detect run eagerly on
+    the same input (time_compute scales boxes to 300x300)."""
+    batch = 3
+    g, info = models.mobilenet_v1_ssd(batch, seed=41, head_std=0.05)
+    x = rng(42).uniform(-1, 1, (batch, 300, 300, 3)).astype(np.float32)
+    sess = session.Session()
+    sess.set_device_nms(device_nms)
+    sess.load_graph(g)
+    eager = sess.detect(x, 300, 300, 0.3, 0.45, 100)
+    assert sum(len(e) for e in eager) > 0
+    for use_graph in (False, True):
+        sess.time_compute(1, 3, graph=use_graph, with_detect=True)
+        got = sess.detect_results(batch)
+        assert got == eager
