@@ -78,6 +78,110 @@ __global__ __launch_bounds__(256) void conv_direct_small_k(
   }
 }
 
+// Stem kernel: few input channels, K = k*k*C <= 32 (the RGB stem has K = 27), on
+// the MFMA units.  A wave owns 32 output pixels x 32 output channels at a time and
+// contracts K with KS = ceil(K/2) v_mfma_f32_32x32x2_f32: lane l supplies
+// A[pixel l%32][k = 2s + l/32] and B[k][channel l%32].  The filter values a lane
+// needs (KS of them) are loaded once and stay in registers while the wave walks
+// over pixel tiles; the lane's KS input taps are gathered straight from global
+// memory (the whole receptive field of a tile is a few KB and is served by the
+// vector cache), all loads of a tile in flight before the first MFMA.  Rows past
+// the end, taps outside the image and the odd K tail contribute zeros.
+typedef float stem_acc_t __attribute__((ext_vector_type(16)));
+
+// 32-bit element offset that no operand reaches (they are kept below 2^31 bytes):
+// a buffer access at it reads zero / is dropped.
+constexpr unsigned kStemOutOfRange = 0x80000000u;
+
+template <typename T>
+__device__ __forceinline__ float stem_load(__amdgpu_buffer_rsrc_t r, unsigned byte_off) {
+  if constexpr (sizeof(T) == 4) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, (int)byte_off, 0, 0));
+  } else {
+    const unsigned short v = __builtin_amdgcn_raw_buffer_load_b16(r, (int)byte_off, 0, 0);
+    return __half2float(__builtin_bit_cast(__half, v));
+  }
+}
+template <typename T>
+__device__ __forceinline__ void stem_store(__amdgpu_buffer_rsrc_t r, unsigned byte_off, float v) {
+  if constexpr (sizeof(T) == 4) {
+    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), r, (int)byte_off, 0, 0);
+  } else {
+    __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(unsigned short, __float2half_rn(v)), r,
+                                          (int)byte_off, 0, 0);
+  }
+}
+
+// What K index kidx means, worked out on the host: the tap's (dy, dx) relative to
+// the pixel's top-left input position and its element offset from there.
+struct StemTaps {
+  int dy[32], dx[32], off[32];
+};
+
+template <typename T, int KS>
+__global__ __launch_bounds__(256) void conv_stem_mfma(
+    const T* __restrict__ x, const T* __restrict__ w, const float* __restrict__ bias,
+    T* __restrict__ y, int h, int wd, int c, int oh, int ow, int o, int stride, Epilogue ep,
+    int ktot, int m_total, int tiles_m, unsigned x_bytes, unsigned y_bytes, StemTaps taps) {
+  constexpr unsigned ESZ = sizeof(T);
+  const int lane = threadIdx.x & 63;
+  const int l32 = lane & 31, lh = lane >> 5;
+  const int wave = (int)(blockIdx.x * 4 + (threadIdx.x >> 6));
+  const int waves = (int)(gridDim.x * 4);
+  const __amdgpu_buffer_rsrc_t rx =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(x), 0, (int)x_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t ry = __builtin_amdgcn_make_buffer_rsrc(y, 0, (int)y_bytes, 0x00020000);
+  // this lane's K indices: kidx = 2s + lane/32 (entries past K never fall inside the image)
+  int tap_dy[KS], tap_dx[KS], tap_off[KS];
+#pragma unroll
+  for (int s = 0; s < KS; ++s) {
+    tap_dy[s] = lh ? taps.dy[2 * s + 1] : taps.dy[2 * s];
+    tap_dx[s] = lh ? taps.dx[2 * s + 1] : taps.dx[2 * s];
+    tap_off[s] = lh ? taps.off[2 * s + 1] : taps.off[2 * s];
+  }
+  for (int n0 = 0; n0 < o; n0 += 32) {
+    const int col = n0 + l32;
+    float bval[KS];
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      const int kidx = 2 * s + lh;
+      bval[s] = (col < o && kidx < ktot) ? to_f32(w[(long)col * ktot + kidx]) : 0.f;
+    }
+    const float bias_v = (bias != nullptr && col < o) ? bias[col] : 0.f;
+    for (int tile = wave; tile < tiles_m; tile += waves) {
+      const int m = tile * 32 + l32;
+      const int ox = m % ow;
+      const int t = m / ow;
+      const int oy = t % oh;
+      const int b = t / oh;
+      const int iy0 = oy * stride, ix0 = ox * stride;
+      const int base = m < m_total ? ((b * h + iy0) * wd + ix0) * c : -0x40000000;
+      float a[KS];
+#pragma unroll
+      for (int s = 0; s < KS; ++s) {
+        const bool in = (unsigned)(iy0 + tap_dy[s]) < (unsigned)h &&
+                        (unsigned)(ix0 + tap_dx[s]) < (unsigned)wd && base >= 0;
+        a[s] = stem_load<T>(rx, in ? (unsigned)(base + tap_off[s]) * ESZ : kStemOutOfRange);
+      }
+      stem_acc_t acc;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+#pragma unroll
+      for (int s = 0; s < KS; ++s) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], bval[s], acc, 0, 0, 0);
+      // register r of lane l: pixel 8*(r/4) + 4*(l/32) + r%4 of the tile, channel l%32
+      const int row0 = tile * 32 + lh * 4;
+      const unsigned off0 = (unsigned)(row0 * o + col);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int dr = (r >> 2) * 8 + (r & 3);
+        const bool ok = row0 + dr < m_total && col < o;
+        stem_store<T>(ry, ok ? (off0 + (unsigned)(dr * o)) * ESZ : kStemOutOfRange,
+                      apply_epilogue(acc[r] + bias_v, ep));
+      }
+    }
+  }
+}
+
 // Fully general kernel: one thread per output element, output channel
 // fastest.  Filter OHWI with I = c/groups.
 template <typename T>
@@ -122,6 +226,38 @@ int32_t run_direct(const OgleConvArgs& a, hipStream_t s) {
   T* y = static_cast<T*>(a.output_dev);
   const int ktot = a.kernel_size * a.kernel_size * a.in_c;
   const size_t lds = sizeof(float) * (size_t)ktot * a.out_c;
+  const long pixels_all = (long)a.n * a.out_h * a.out_w;
+  const long esz = (long)sizeof(T);
+  const long x_bytes = (long)a.n * a.in_h * a.in_w * a.in_c * esz;
+  const long y_bytes = pixels_all * a.out_c * esz;
+  if (a.group == 1 && ktot <= 32 && pixels_all >= 4096 && x_bytes < 0x7fffffffL &&
+      y_bytes < 0x7fffffffL) {
+    const int tiles_m = (int)((pixels_all + 31) / 32);
+    // a wave keeps its filter values while it walks over tiles: one wave per tile
+    // until every compute unit has three workgroups (measured best), then more tiles
+    // per wave
+    int blocks = (tiles_m + 3) / 4;
+    if (blocks > 256 * 3) blocks = 256 * 3;
+    const int ks = (ktot + 1) / 2;
+    StemTaps taps;
+    for (int kidx = 0; kidx < 32; ++kidx) {
+      const int tap = kidx / a.in_c, ci = kidx % a.in_c;
+      taps.dy[kidx] = (tap / a.kernel_size) * a.dilation - a.padding;
+      taps.dx[kidx] = (tap % a.kernel_size) * a.dilation - a.padding;
+      taps.off[kidx] = (taps.dy[kidx] * a.in_w + taps.dx[kidx]) * a.in_c + ci;
+      if (kidx >= ktot) taps.dy[kidx] = -0x40000000;
+    }
+#define OGLE_STEM_CASE(KS)                                                                        \
+  hipLaunchKernelGGL((conv_stem_mfma<T, KS>), dim3(blocks), dim3(256), 0, s, x, w, a.bias_dev, y,  \
+                     a.in_h, a.in_w, a.in_c, a.out_h, a.out_w, a.out_c, a.stride, ep, ktot,       \
+                     (int)pixels_all, tiles_m, (unsigned)x_bytes, (unsigned)y_bytes, taps)
+    if (ks <= 5) OGLE_STEM_CASE(5);
+    else if (ks <= 9) OGLE_STEM_CASE(9);
+    else if (ks <= 14) OGLE_STEM_CASE(14);
+    else OGLE_STEM_CASE(16);
+#undef OGLE_STEM_CASE
+    return check_launch("conv_stem_mfma");
+  }
   if (a.group == 1 && lds <= 48 * 1024 && a.out_c % 4 == 0) {
     // 16 channels per thread when that still leaves enough threads to fill the chip
     const long pixels = (long)a.n * a.out_h * a.out_w;

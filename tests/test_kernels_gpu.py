@@ -104,6 +104,32 @@ def test_conv_shape_sweep_dense_and_depthwise():
                        entry="ogle_hip_dwconv2d", what="dw %d %d" % (size, ch))
 
 
+STEM_CASES = [
+    # n, h, w, c, o, k, s, p, d   (K = k*k*c <= 32 and >= 4096 output pixels: the MFMA stem kernel)
+    (2, 96, 96, 3, 32, 3, 2, 1, 1),     # the RGB stem shape
+    (1, 70, 67, 3, 20, 3, 1, 1, 1),     # ragged pixel count, fewer channels than a tile
+    (1, 65, 66, 1, 40, 3, 1, 0, 1),     # one input channel, two channel tiles, no padding
+    (1, 80, 80, 2, 33, 3, 1, 2, 2),     # dilation 2
+    (1, 64, 70, 3, 8, 2, 1, 0, 1),      # even kernel, K = 12
+    (1, 68, 68, 1, 5, 5, 1, 2, 1),      # 5x5 on one channel, K = 25
+    (1, 64, 64, 8, 16, 2, 2, 0, 1),     # K = 32 exactly
+]
+
+
+@pytest.mark.parametrize("case", STEM_CASES)
+@pytest.mark.parametrize("dtype", [H.F32, H.F16])
+def test_conv_stem_kernel(case, dtype):
+    n, h, w, c, o, k, s, p, d = case
+    r = rng(1500 + STEM_CASES.index(case))
+    x = r.uniform(-1, 1, (n, h, w, c)).astype(np.float32)
+    wt = r.normal(0, 0.5, (o, c, k, k)).astype(np.float32)
+    b = r.uniform(-0.1, 0.1, o).astype(np.float32)
+    if dtype == H.F16:  # the oracle sees the values the device stores
+        x = x.astype(np.float16).astype(np.float32)
+        wt = wt.astype(np.float16).astype(np.float32)
+    check_conv(x, wt, b, s, p, d, 1, act=H.ACT_CLIP, maxv=6.0, dtype=dtype, what=str(case))
+
+
 def test_conv_shape_sweep_mfma_path():
     """Channel counts that take the implicit-GEMM kernel, ragged in every dimension."""
     r = rng(2100)
