@@ -91,6 +91,7 @@ int32_t launch_transpose(const OgleTransposeArgs& a, hipStream_t s);
 int32_t launch_decode(const OgleDecodeArgs& a, hipStream_t s);
 int32_t launch_detect(const OgleDetectArgs& a, hipStream_t s);
 int32_t launch_topk_nms(const OgleNmsArgs& a, hipStream_t s);
+size_t topk_nms_lds_bytes(int stride, int topk);
 int32_t launch_expf(const float* x, float* y, int64_t n, hipStream_t s);
 int32_t launch_pack_filter(const float* src, void* dst, int layout, int dtype, int o, int i,
                            int kh, int kw, hipStream_t s);

@@ -254,16 +254,13 @@ __global__ __launch_bounds__(256) void ssd_compact_kernel(DetectParams p) {
 // IoU is evaluated on the integer rectangles in fp32, operation by operation as the
 // host does (no FMA contraction), so kept sets are bit-identical.
 #pragma clang fp contract(off)
-__device__ __forceinline__ float rect_iou(const int4& a, const int4& b) {
-  const float xmin0 = (float)a.x, ymin0 = (float)a.y;
-  const float xmax0 = (float)(a.x + a.z), ymax0 = (float)(a.y + a.w);
-  const float xmin1 = (float)b.x, ymin1 = (float)b.y;
-  const float xmax1 = (float)(b.x + b.z), ymax1 = (float)(b.y + b.w);
-  const float w = fmaxf(0.0f, fminf(xmax0, xmax1) - fmaxf(xmin0, xmin1));
-  const float h = fmaxf(0.0f, fminf(ymax0, ymax1) - fmaxf(ymin0, ymin1));
+__device__ __forceinline__ float corner_iou(const float4& a, const float4& b) {
+  // a, b = (xmin, ymin, xmax, ymax), the int -> float conversions iou() starts with
+  const float w = fmaxf(0.0f, fminf(a.z, b.z) - fmaxf(a.x, b.x));
+  const float h = fmaxf(0.0f, fminf(a.w, b.w) - fmaxf(a.y, b.y));
   const float i = w * h;
   if (i == 0.0f) return 0.0f;  // disjoint: the host gets 0 / u or its u <= 0 case, both 0
-  const float u = (xmax0 - xmin0) * (ymax0 - ymin0) + (xmax1 - xmin1) * (ymax1 - ymin1) - i;
+  const float u = (a.z - a.x) * (a.w - a.y) + (b.z - b.x) * (b.w - b.y) - i;
   if (u <= 0.0f) return 0.0f;
   return i / u;
 }
@@ -291,7 +288,7 @@ __device__ __forceinline__ unsigned ordered_bits(float v) {
   return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
 }
 
-// Steps of the kernel, one workgroup per image with n kept entries:
+// Steps of the kernel, one workgroup of 1024 threads per image with n kept entries:
 //   1. radix select (four 8-bit passes over the ordered score bits) finds the value
 //      of the k-th largest score and how many entries equal to it belong to the
 //      top k; of equal scores the first ones in list order are taken
@@ -300,17 +297,41 @@ __device__ __forceinline__ unsigned ordered_bits(float v) {
 //      the selected entries only, which sorts them
 //   4. NMS over all pairs of the sorted list, then an ordered compaction of the
 //      survivors
-__global__ __launch_bounds__(256) void ssd_topk_nms_kernel(NmsParams p) {
+constexpr int kNmsThreads = 1024;
+constexpr int kNmsWaves = kNmsThreads / 64;
+
+// Exclusive prefix of `flag` over the workgroup in thread order, and the total.
+// `wave_count` is LDS scratch of kNmsWaves ints; two barriers.
+__device__ __forceinline__ int block_rank(bool flag, int* wave_count, int lane, int wave, int* total) {
+  const unsigned long long ballot = __ballot(flag);
+  if (lane == 0) wave_count[wave] = __popcll(ballot);
+  __syncthreads();
+  int before = __popcll(ballot & ((1ull << lane) - 1ull));
+  int sum = 0;
+#pragma unroll
+  for (int wv = 0; wv < kNmsWaves; ++wv) {
+    const int cnt = wave_count[wv];
+    if (wv < wave) before += cnt;
+    sum += cnt;
+  }
+  __syncthreads();  // wave_count may be rewritten after this
+  *total = sum;
+  return before;
+}
+
+__global__ __launch_bounds__(kNmsThreads) void ssd_topk_nms_kernel(NmsParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char nms_lds[];
-  // keys[stride] | cand_key[topk+4] | cand_idx[topk+4] | sel[topk] | rect[topk] | hist[256] | misc[8]
+  // keys[stride] | cand_key[topk] | cand_idx[topk] | sel[topk] | rect[topk] | frect[topk] |
+  // hist[256] | misc[kNmsWaves + 2]     (topk and stride rounded up to 4)
   const int tpad = (p.topk + 3) & ~3;
   unsigned* keys = reinterpret_cast<unsigned*>(nms_lds);
   unsigned* cand_key = keys + ((p.stride + 3) & ~3);
   int* cand_idx = reinterpret_cast<int*>(cand_key + tpad);
   int* sel = cand_idx + tpad;
   int4* rects = reinterpret_cast<int4*>(sel + tpad);
-  int* hist = reinterpret_cast<int*>(rects + p.topk);
-  int* misc = hist + 256;  // [0..3] wave counts, [4] chosen digit, [5] entries above it
+  float4* frects = reinterpret_cast<float4*>(rects + tpad);
+  int* hist = reinterpret_cast<int*>(frects + tpad);
+  int* misc = hist + 256;  // [0..kNmsWaves) wave counts, then the chosen digit and the count above it
 
   const int b = blockIdx.x;
   const int tid = threadIdx.x;
@@ -318,7 +339,7 @@ __global__ __launch_bounds__(256) void ssd_topk_nms_kernel(NmsParams p) {
   const long row0 = (long)b * p.stride;
   int n = p.kept_count[b];
   n = n < 0 ? 0 : (n > p.stride ? p.stride : n);
-  for (int i = tid; i < n; i += 256) keys[i] = ordered_bits(p.kept_score[row0 + i]);
+  for (int i = tid; i < n; i += kNmsThreads) keys[i] = ordered_bits(p.kept_score[row0 + i]);
   __syncthreads();
 
   // 1. the k-th largest key
@@ -327,78 +348,69 @@ __global__ __launch_bounds__(256) void ssd_topk_nms_kernel(NmsParams p) {
   int remaining = m;  // how many of the entries matching `prefix` are still wanted
   if (n > p.topk) {
     for (int shift = 24; shift >= 0; shift -= 8) {
-      hist[tid] = 0;
+      if (tid < 256) hist[tid] = 0;
       __syncthreads();
-      for (int i = tid; i < n; i += 256) {
+      for (int i = tid; i < n; i += kNmsThreads) {
         const unsigned k = keys[i];
         if ((k & mask) == prefix) atomicAdd(&hist[(k >> shift) & 255u], 1);
       }
       __syncthreads();
-      // thread t: entries whose digit is above t, and at or above t (suffix sums of
-      // the histogram: a shuffle scan inside each wave plus the totals of later waves)
-      const int mine = hist[tid];
+      // thread t < 256: entries whose digit is above t, and at or above t (suffix sums
+      // of the histogram: a shuffle scan inside each wave plus the totals of later waves)
+      const int mine = tid < 256 ? hist[tid] : 0;
       int sfx = mine;
 #pragma unroll
       for (int d = 1; d < 64; d <<= 1) {
         const int v = __shfl_down(sfx, d, 64);
         if (lane + d < 64) sfx += v;
       }
-      if (lane == 0) misc[wave] = sfx;
+      if (lane == 0 && wave < 4) misc[wave] = sfx;
       __syncthreads();
-      int at_or_above = sfx;
-      for (int wv = wave + 1; wv < 4; ++wv) at_or_above += misc[wv];
-      const int above = at_or_above - mine;
-      if (above < remaining && remaining <= at_or_above) {
-        misc[4] = tid;
-        misc[5] = above;
+      if (tid < 256) {
+        int at_or_above = sfx;
+        for (int wv = wave + 1; wv < 4; ++wv) at_or_above += misc[wv];
+        const int above = at_or_above - mine;
+        if (above < remaining && remaining <= at_or_above) {
+          misc[kNmsWaves] = tid;
+          misc[kNmsWaves + 1] = above;
+        }
       }
       __syncthreads();
-      prefix |= (unsigned)misc[4] << shift;
+      prefix |= (unsigned)misc[kNmsWaves] << shift;
       mask |= 255u << shift;
-      remaining -= misc[5];
+      remaining -= misc[kNmsWaves + 1];
       __syncthreads();  // misc and hist are rewritten by the next pass
     }
   }
   // now: take every key above `prefix`, and the first `remaining` equal to it
-  // (n <= topk: prefix = 0, mask = 0, every key is "above or equal", all are taken)
+  // (n <= topk: every entry is taken)
 
   // 2. ordered compaction of the selected entries
   {
     int taken = 0, equal_seen = 0;
-    for (int start = 0; start < n; start += 256) {
+    for (int start = 0; start < n; start += kNmsThreads) {
       const int i = start + tid;
       const unsigned k = i < n ? keys[i] : 0u;
       const bool gt = i < n && (n <= p.topk || k > prefix);
       const bool eq = i < n && n > p.topk && k == prefix;
-      const unsigned long long eq_ballot = __ballot(eq);
-      if (lane == 0) misc[wave] = __popcll(eq_ballot);
-      __syncthreads();
-      int eq_before = equal_seen + __popcll(eq_ballot & ((1ull << lane) - 1ull));
-      for (int wv = 0; wv < wave; ++wv) eq_before += misc[wv];
-      const int eq_total = misc[0] + misc[1] + misc[2] + misc[3];
-      __syncthreads();
+      int eq_total, total;
+      const int eq_before = equal_seen + block_rank(eq, misc, lane, wave, &eq_total);
       const bool take = gt || (eq && eq_before < remaining);
-      const unsigned long long ballot = __ballot(take);
-      if (lane == 0) misc[wave] = __popcll(ballot);
-      __syncthreads();
-      int before = taken + __popcll(ballot & ((1ull << lane) - 1ull));
-      for (int wv = 0; wv < wave; ++wv) before += misc[wv];
-      const int total = misc[0] + misc[1] + misc[2] + misc[3];
+      const int before = taken + block_rank(take, misc, lane, wave, &total);
       if (take) {
         cand_key[before] = k;
         cand_idx[before] = i;
       }
       taken += total;
       equal_seen += eq_total;
-      __syncthreads();
     }
   }
-  for (int r = m + tid; r < ((m + 3) & ~3); r += 256) cand_key[r] = 0u;  // padding ranks last
+  for (int r = m + tid; r < ((m + 3) & ~3); r += kNmsThreads) cand_key[r] = 0u;  // padding ranks last
   __syncthreads();
 
   // 3. rank among the selected entries (they are in list order, so position breaks ties)
   const int mpad = (m + 3) & ~3;
-  for (int r = tid; r < m; r += 256) {
+  for (int r = tid; r < m; r += kNmsThreads) {
     const unsigned kr = cand_key[r];
     int rank = 0;
     for (int j = 0; j < mpad; j += 4) {
@@ -411,17 +423,22 @@ __global__ __launch_bounds__(256) void ssd_topk_nms_kernel(NmsParams p) {
     sel[rank] = cand_idx[r];
   }
   __syncthreads();
-  for (int r = tid; r < m; r += 256) rects[r] = p.kept_rect[row0 + sel[r]];
+  for (int r = tid; r < m; r += kNmsThreads) {
+    const int4 q = p.kept_rect[row0 + sel[r]];
+    rects[r] = q;
+    // corners as the host's iou() forms them: integer sums converted to float
+    frects[r] = make_float4((float)q.x, (float)q.y, (float)(q.x + q.z), (float)(q.y + q.w));
+  }
   __syncthreads();
 
   // 4. NMS: all (i, j) pairs with i < j are spread over the workgroup; a pair that
   // overlaps by more than the threshold marks j (every writer stores the same value)
   int* dropped = cand_idx;  // the candidate list is no longer needed
-  for (int r = tid; r < m; r += 256) dropped[r] = 0;
+  for (int r = tid; r < m; r += kNmsThreads) dropped[r] = 0;
   __syncthreads();
   if (m > 1) {
-    // pair number t = i * m + j, advanced by 256 per step without dividing
-    const int step_i = 256 / m, step_j = 256 - step_i * m;
+    // pair number t = i * m + j, advanced by the thread count per step without dividing
+    const int step_i = kNmsThreads / m, step_j = kNmsThreads - step_i * m;
     int i = tid / m, j = tid - i * m;
     for (; i < m; i += step_i, j += step_j) {
       if (j >= m) {
@@ -429,8 +446,7 @@ __global__ __launch_bounds__(256) void ssd_topk_nms_kernel(NmsParams p) {
         ++i;
         if (i >= m) break;
       }
-      if (i >= j) continue;
-      if (rect_iou(rects[i], rects[j]) > p.threshold) dropped[j] = 1;
+      if (i < j && corner_iou(frects[i], frects[j]) > p.threshold) dropped[j] = 1;
     }
   }
   __syncthreads();
@@ -438,27 +454,21 @@ __global__ __launch_bounds__(256) void ssd_topk_nms_kernel(NmsParams p) {
   // ordered compaction of the survivors into the output lists
   int base = 0;
   const long out0 = (long)b * p.topk;
-  for (int start = 0; start < m; start += 256) {
+  for (int start = 0; start < m; start += kNmsThreads) {
     const int j = start + tid;
     const bool keep = j < m && dropped[j] == 0;
-    const unsigned long long ballot = __ballot(keep);
-    const int before = __popcll(ballot & ((1ull << lane) - 1ull));
-    if (lane == 0) misc[wave] = __popcll(ballot);
-    __syncthreads();
-    int wave_base = 0;
-    for (int wv = 0; wv < wave; ++wv) wave_base += misc[wv];
-    const int chunk_total = misc[0] + misc[1] + misc[2] + misc[3];
+    int total;
+    const int before = block_rank(keep, misc, lane, wave, &total);
     if (keep) {
       const long src = row0 + sel[j];
-      const long dst = out0 + base + wave_base + before;
+      const long dst = out0 + base + before;
       p.out_prior[dst] = p.kept_prior[src];
       p.out_class[dst] = p.kept_class[src];
       p.out_score[dst] = p.kept_score[src];
       if (p.out_box != nullptr) p.out_box[dst] = p.kept_box[src];
       p.out_rect[dst] = rects[j];
     }
-    base += chunk_total;
-    __syncthreads();
+    base += total;
   }
   if (tid == 0) p.out_count[b] = base;
 }
@@ -467,8 +477,8 @@ __global__ __launch_bounds__(256) void ssd_topk_nms_kernel(NmsParams p) {
 
 size_t topk_nms_lds_bytes(int stride, int topk) {
   const size_t tpad = (size_t)((topk + 3) & ~3);
-  return 4 * (size_t)((stride + 3) & ~3) + 4 * 3 * tpad + sizeof(int4) * (size_t)topk +
-         4 * (256 + 8);
+  return 4 * (size_t)((stride + 3) & ~3) + 4 * 3 * tpad + (sizeof(int4) + sizeof(float4)) * tpad +
+         4 * (256 + kNmsWaves + 2);
 }
 
 int32_t launch_topk_nms(const OgleNmsArgs& a, hipStream_t s) {
@@ -489,7 +499,7 @@ int32_t launch_topk_nms(const OgleNmsArgs& a, hipStream_t s) {
   p.out_score = a.final_score_dev;
   p.out_box = reinterpret_cast<float4*>(a.final_box_dev);
   p.out_rect = reinterpret_cast<int4*>(a.final_rect_dev);
-  hipLaunchKernelGGL(ssd_topk_nms_kernel, dim3((unsigned)a.batch), dim3(256),
+  hipLaunchKernelGGL(ssd_topk_nms_kernel, dim3((unsigned)a.batch), dim3(kNmsThreads),
                      topk_nms_lds_bytes(a.stride, a.topk), s, p);
   return check_launch("ssd_topk_nms_kernel");
 }
