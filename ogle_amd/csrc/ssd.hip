@@ -156,27 +156,41 @@ __global__ __launch_bounds__(256) void ssd_detect_kernel(DetectParams p) {
 // image's survivors to the front in place, in prior order.  A slot is only ever
 // overwritten by an entry that came from the same or a later slot, after the chunk
 // holding it has been read, so the in-place pass needs one barrier per chunk.
+constexpr int kScorePriors = 64;  // priors per workgroup of ssd_score_kernel
+
 __global__ __launch_bounds__(256) void ssd_score_kernel(DetectParams p) {
-  extern __shared__ float slab[];  // 256 * classes
+  // Four threads share a prior: each evaluates every fourth exponential (the costly
+  // part) into LDS, then one of them makes the reference's sequential pass over the
+  // row (sum in class order, strict-greater maximum), so the arithmetic and its order
+  // are those of the single-thread form.
+  extern __shared__ float slab[];  // logits, overwritten in place by their exponentials
   const int b = blockIdx.y;
-  const int start = blockIdx.x * 256;
+  const int start = blockIdx.x * kScorePriors;
   const int tid = threadIdx.x;
-  const int rows = min(256, p.priors - start);
+  const int rows = min(kScorePriors, p.priors - start);
   const int count = rows * p.classes;
   const float* src = p.logits + ((long)b * p.priors + start) * p.classes;
   for (int i = tid; i < count; i += 256) slab[i] = src[i];
   __syncthreads();
+  {
+    const int pl = tid >> 2, q = tid & 3;
+    if (pl < rows) {
+      float* l = slab + pl * p.classes;
+      for (int j = q; j < p.classes; j += 4) l[j] = exp_cr(l[j]);
+    }
+  }
+  __syncthreads();
   if (tid >= rows) return;
   const int prior = start + tid;
-  const float* l = slab + tid * p.classes;
-  float total_sum = exp_cr(l[0]);
+  const float* e = slab + tid * p.classes;
+  float total_sum = e[0];
   int max_id = 0;
   float max_prob = 0.f;
   for (int j = 1; j < p.classes; ++j) {
-    const float e = exp_cr(l[j]);
-    total_sum += e;
-    if (max_prob < e) {
-      max_prob = e;
+    const float ej = e[j];
+    total_sum += ej;
+    if (max_prob < ej) {
+      max_prob = ej;
       max_id = j;
     }
   }
@@ -536,8 +550,9 @@ int32_t launch_detect(const OgleDetectArgs& a, hipStream_t s) {
   const size_t lds = sizeof(float) * 256 * (size_t)a.classes;
   const bool all_outputs = p.kept_prior && p.kept_class && p.kept_score && p.kept_box && p.kept_rect;
   if (all_outputs && a.priors > 256 && a.batch <= 65535) {
-    hipLaunchKernelGGL(ssd_score_kernel, dim3((unsigned)((a.priors + 255) / 256), (unsigned)a.batch),
-                       dim3(256), lds, s, p);
+    hipLaunchKernelGGL(ssd_score_kernel,
+                       dim3((unsigned)((a.priors + kScorePriors - 1) / kScorePriors), (unsigned)a.batch),
+                       dim3(256), sizeof(float) * kScorePriors * (size_t)a.classes, s, p);
     const int32_t st = check_launch("ssd_score_kernel");
     if (st != OGLE_OK) return st;
     hipLaunchKernelGGL(ssd_compact_kernel, dim3((unsigned)a.batch), dim3(256), 0, s, p);
