@@ -91,6 +91,7 @@ def encode_pool_attr(kernel, stride, pad):
 # Attribute field numbers (dlxnet.proto:165-187)
 ATTR_CONV2D, ATTR_CONST, ATTR_MAXPOOL, ATTR_AVEPOOL, ATTR_INPUT = 1, 2, 5, 6, 10
 ATTR_TRANSPOSE, ATTR_CONCAT, ATTR_RESHAPE = 12, 16, 17
+ATTR_SHAPE, ATTR_GATHER, ATTR_UNSQUEEZE = 13, 14, 15
 
 
 def encode_node(name, type_, inputs, outputs, attr_field=None, attr_payload=b""):
@@ -154,6 +155,15 @@ class GraphBuilder:
 
     def add_reshape(self, name, x, shape_tensor):
         return self._emit(name, "Reshape", [x, shape_tensor], ATTR_RESHAPE, b"")
+
+    def add_shape(self, name, x):
+        return self._emit(name, "Shape", [x], ATTR_SHAPE, b"")
+
+    def add_gather(self, name, data, index, axis=0):
+        return self._emit(name, "Gather", [data, index], ATTR_GATHER, _int(1, axis))
+
+    def add_unsqueeze(self, name, x, axis):
+        return self._emit(name, "Unsqueeze", [x], ATTR_UNSQUEEZE, _packed_ints(1, [axis]))
 
     def add_decoder(self, name, prediction, anchors):
         return self._emit(name, "Decoder", [prediction, anchors])

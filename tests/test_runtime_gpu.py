@@ -167,6 +167,41 @@ def test_transpose_and_reshape_nodes():
     assert sess.tensor_device_ptr("view") == sess.tensor_device_ptr("input")
 
 
+def test_exported_view_chain_folds_at_setup():
+    """PyTorch exports x.permute(0,2,3,1).view(N, -1, K) with the batch size taken from the
+    tensor: Shape -> Gather(0) -> Unsqueeze -> Concat([n], [-1], [K]) -> Reshape.  The chain runs
+    once while the session is set up (shape.h:19, fbo_session.cc:240-244) and the view aliases
+    its input.  Gather's index counts NCHW positions while the shape vector is NHWC
+    (gather.glsl:10-18)."""
+    r = rng(7600)
+    x = r.normal(0, 1, (3, 5, 4, 8)).astype(np.float32)   # NHWC
+    gb = dlx.GraphBuilder()
+    xi = gb.add_input("input", [3, 8, 5, 4])
+    t0 = gb.add_transpose("perm", xi, [0, 2, 3, 1])
+    shp = gb.add_shape("shape_of", xi)
+    dims = {}
+    for name, idx in (("n", 0), ("c", 1), ("h", 2), ("w", 3)):
+        ci = gb.add_const("idx_" + name, np.array([idx], np.float32), dims=[])
+        gi = gb.add_gather("dim_" + name, shp, ci)
+        dims[name] = gb.add_unsqueeze("dim_" + name + "_1", gi, 0)
+    minus1 = gb.add_const("minus1", np.array([-1], np.float32))
+    four = gb.add_const("four", np.array([4], np.float32))
+    target = gb.add_concat("target", [dims["n"], minus1, four], 0)
+    gb.add_reshape("view", t0, target)
+    alldims = gb.add_concat("nchw", [dims["n"], dims["c"], dims["h"], dims["w"]], 0)
+    sess = session.Session()
+    sess.load_graph(gb)
+    sess.run({"input": x})
+    np.testing.assert_array_equal(sess.get_output("shape_of", "ANY"), [3, 5, 4, 8])
+    np.testing.assert_array_equal(sess.get_output("nchw", "ANY"), [3, 8, 5, 4])
+    np.testing.assert_array_equal(sess.get_output("target", "ANY"), [3, -1, 4])
+    np.testing.assert_array_equal(sess.get_output("view", "ANY"), x.reshape(3, -1, 4))
+    assert sess.tensor_device_ptr("view") == sess.tensor_device_ptr("input")
+    assert sess.tensor_shape("dim_n") == () and sess.tensor_shape("dim_n_1") == (1,)
+    # nothing of the chain is left on the per-pass path
+    assert sess.issue_order() == ["perm", "view"]
+
+
 @pytest.mark.parametrize("batch", [1, 8])
 def test_config2_block_through_session(batch):
     g, w = models.separable_block(batch)
