@@ -248,6 +248,82 @@ typedef struct OgleTransposeArgs {
 int32_t ogle_hip_transpose(const OgleTransposeArgs* args, ogle_stream_t stream);
 
 /* ------------------------------------------------------------------------ */
+/* Elementwise ops and Gemm (classification graphs)                           */
+/* ------------------------------------------------------------------------ */
+
+typedef enum OgleUnaryOp {
+  OGLE_UNARY_RELU = 0, /* relu.glsl:8-10: max(0, x) */
+  OGLE_UNARY_CLIP = 1  /* clip.glsl:7-12: min(max_value, max(min_value, x)) */
+} OgleUnaryOp;
+
+/* ReluKernel / ClipKernel (ogl_runtime/opengl/nn/kernels/{relu,clip}.cc).  `count`
+ * elements of any shape; input and output may be the same buffer.  Pointers must
+ * be 16-byte aligned. */
+typedef struct OgleUnaryArgs {
+  const void* input_dev;
+  void* output_dev;
+  int64_t count;
+  int32_t op; /* OgleUnaryOp */
+  float min_value, max_value;
+  int32_t dtype;
+} OgleUnaryArgs;
+
+int32_t ogle_hip_unary(const OgleUnaryArgs* args, ogle_stream_t stream);
+
+/* BinaryKernel, registered as "Add" (ogl_runtime/opengl/nn/kernels/binary.cc,
+ * binary.glsl:8): y = a + b over two tensors of one shape. */
+typedef struct OgleBinaryArgs {
+  const void* a_dev;
+  const void* b_dev;
+  void* output_dev;
+  int64_t count;
+  int32_t dtype;
+} OgleBinaryArgs;
+
+int32_t ogle_hip_add(const OgleBinaryArgs* args, ogle_stream_t stream);
+
+/* BatchNormKernel (ogl_runtime/opengl/nn/kernels/batchnorm.cc, batchnorm.glsl:33):
+ * y = (x - mean) / sqrt(var + eps) * gamma + beta, the four fp32 parameter vectors
+ * indexed by the last dimension (`channels`); `outer` is the product of the others. */
+typedef struct OgleBatchNormArgs {
+  const void* input_dev;
+  const float* gamma_dev;
+  const float* beta_dev;
+  const float* mean_dev;
+  const float* var_dev;
+  void* output_dev;
+  int64_t outer;
+  int32_t channels;
+  float epsilon;
+  int32_t dtype;
+} OgleBatchNormArgs;
+
+int32_t ogle_hip_batchnorm(const OgleBatchNormArgs* args, ogle_stream_t stream);
+
+/* GemmKernel (ogl_runtime/opengl/nn/kernels/gemm.cc, gemm.glsl:33-95), fp32:
+ * Y(M,N) = alpha * A(M,K) * B' + beta * C, where B' is B(K,N) or, with trans_b, the
+ * transpose of B(N,K).  C is NULL, a row of N values added to every row of Y
+ * (c_rank 1), or (M,N) (c_rank 2) as in GemmCPU (gemm_test.cc:9-40).  The Linear
+ * form (trans_b, alpha 1, C NULL or a row with beta 1, K % 4 == 0) runs on the MFMA
+ * units and may use a workspace of ogle_hip_gemm_workspace_bytes() bytes for its
+ * split-K plans (optional; the library does not allocate). */
+typedef struct OgleGemmArgs {
+  const float* a_dev;
+  const float* b_dev;
+  const float* c_dev;
+  float* y_dev;
+  int32_t m, n, k;
+  int32_t trans_b;
+  int32_t c_rank;
+  float alpha, beta;
+  void* workspace_dev;
+  size_t workspace_bytes;
+} OgleGemmArgs;
+
+size_t ogle_hip_gemm_workspace_bytes(const OgleGemmArgs* args);
+int32_t ogle_hip_gemm(const OgleGemmArgs* args, ogle_stream_t stream);
+
+/* ------------------------------------------------------------------------ */
 /* SSD box decoder and score filter                                           */
 /* ------------------------------------------------------------------------ */
 

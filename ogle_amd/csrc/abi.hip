@@ -31,7 +31,8 @@ namespace {
 // options the reference composes (conv2d.cc:54-62).
 enum Family {
   FAM_CONV = 1, FAM_CONV_DW = 2, FAM_CONV_PW = 3, FAM_CONV_GRP = 4,
-  FAM_POOL = 5, FAM_CONCAT = 6, FAM_DECODER = 7, FAM_TRANSPOSE = 8, FAM_RESHAPE = 9
+  FAM_POOL = 5, FAM_CONCAT = 6, FAM_DECODER = 7, FAM_TRANSPOSE = 8, FAM_RESHAPE = 9,
+  FAM_ELTWISE = 10, FAM_GEMM = 11
 };
 enum Flags { FLAG_BIAS = 1, FLAG_CLIP = 2, FLAG_RELU = 4, FLAG_ANY4 = 8 };
 
@@ -57,6 +58,12 @@ const Entry kRegistry[] = {
     {"transpose_any4", FAM_TRANSPOSE, FLAG_ANY4},
     {"reshape", FAM_RESHAPE, 0},
     {"reshape_any4", FAM_RESHAPE, FLAG_ANY4},
+    {"binary", FAM_ELTWISE, 0},
+    {"relu", FAM_ELTWISE, 0},
+    {"clip", FAM_ELTWISE, 0},
+    {"batchnorm", FAM_ELTWISE, 0},
+    {"batchnorm_any4", FAM_ELTWISE, FLAG_ANY4},
+    {"gemm", FAM_GEMM, 0},
 };
 constexpr int kRegistrySize = sizeof(kRegistry) / sizeof(kRegistry[0]);
 
@@ -346,6 +353,72 @@ int32_t ogle_hip_ssd_detect(const OgleDetectArgs* a, ogle_stream_t stream) {
   if (a->anchors_batch_stride != 0 && a->anchors_batch_stride != (int64_t)a->priors * 4)
     return fail(OGLE_ERR_INVALID_ARG, "ssd_detect: anchors_batch_stride must be 0 or priors*4");
   return launch_detect(*a, as_stream(stream));
+}
+
+namespace {
+bool misaligned(const void* p, uintptr_t bytes) {
+  return (reinterpret_cast<uintptr_t>(p) & (bytes - 1)) != 0;
+}
+bool bad_dtype(int32_t d) { return d != OGLE_F32 && d != OGLE_F16; }
+}  // namespace
+
+int32_t ogle_hip_unary(const OgleUnaryArgs* a, ogle_stream_t stream) {
+  if (a == nullptr) return fail(OGLE_ERR_INVALID_ARG, "unary: null args");
+  if (a->count < 0 || bad_dtype(a->dtype)) return fail(OGLE_ERR_INVALID_ARG, "unary: bad count or dtype");
+  if (a->op != OGLE_UNARY_RELU && a->op != OGLE_UNARY_CLIP)
+    return fail(OGLE_ERR_UNSUPPORTED, "unary: unknown op");
+  if (a->count > 0 && (!a->input_dev || !a->output_dev))
+    return fail(OGLE_ERR_INVALID_ARG, "unary: null device pointer");
+  if (misaligned(a->input_dev, 16) || misaligned(a->output_dev, 16))
+    return fail(OGLE_ERR_INVALID_ARG, "unary: pointers must be 16-byte aligned");
+  return launch_unary(*a, as_stream(stream));
+}
+
+int32_t ogle_hip_add(const OgleBinaryArgs* a, ogle_stream_t stream) {
+  if (a == nullptr) return fail(OGLE_ERR_INVALID_ARG, "add: null args");
+  if (a->count < 0 || bad_dtype(a->dtype)) return fail(OGLE_ERR_INVALID_ARG, "add: bad count or dtype");
+  if (a->count > 0 && (!a->a_dev || !a->b_dev || !a->output_dev))
+    return fail(OGLE_ERR_INVALID_ARG, "add: null device pointer");
+  if (misaligned(a->a_dev, 16) || misaligned(a->b_dev, 16) || misaligned(a->output_dev, 16))
+    return fail(OGLE_ERR_INVALID_ARG, "add: pointers must be 16-byte aligned");
+  return launch_binary(*a, as_stream(stream));
+}
+
+int32_t ogle_hip_batchnorm(const OgleBatchNormArgs* a, ogle_stream_t stream) {
+  if (a == nullptr) return fail(OGLE_ERR_INVALID_ARG, "batchnorm: null args");
+  if (a->outer < 0 || a->channels < 1 || bad_dtype(a->dtype))
+    return fail(OGLE_ERR_INVALID_ARG, "batchnorm: bad size or dtype");
+  if (a->outer > 0 && (!a->input_dev || !a->output_dev || !a->gamma_dev || !a->beta_dev ||
+                       !a->mean_dev || !a->var_dev))
+    return fail(OGLE_ERR_INVALID_ARG, "batchnorm: null device pointer");
+  if (misaligned(a->input_dev, 16) || misaligned(a->output_dev, 16))
+    return fail(OGLE_ERR_INVALID_ARG, "batchnorm: tensors must be 16-byte aligned");
+  return launch_batchnorm(*a, as_stream(stream));
+}
+
+namespace {
+int32_t validate_gemm(const OgleGemmArgs* a) {
+  if (a == nullptr) return fail(OGLE_ERR_INVALID_ARG, "gemm: null args");
+  if (a->m < 0 || a->n < 0 || a->k < 1) return fail(OGLE_ERR_INVALID_ARG, "gemm: bad size");
+  if (a->c_dev != nullptr && a->c_rank != 1 && a->c_rank != 2)
+    return fail(OGLE_ERR_INVALID_ARG, "gemm: c_rank must be 1 or 2");
+  if (a->workspace_dev == nullptr && a->workspace_bytes != 0)
+    return fail(OGLE_ERR_INVALID_ARG, "gemm: workspace_bytes without workspace_dev");
+  return OGLE_OK;
+}
+}  // namespace
+
+size_t ogle_hip_gemm_workspace_bytes(const OgleGemmArgs* a) {
+  if (validate_gemm(a) != OGLE_OK || a->m == 0 || a->n == 0) return 0;
+  return gemm_workspace_bytes(*a);
+}
+
+int32_t ogle_hip_gemm(const OgleGemmArgs* a, ogle_stream_t stream) {
+  const int32_t st = validate_gemm(a);
+  if (st != OGLE_OK) return st;
+  if ((long)a->m * a->n > 0 && (!a->a_dev || !a->b_dev || !a->y_dev))
+    return fail(OGLE_ERR_INVALID_ARG, "gemm: null device pointer");
+  return launch_gemm(*a, as_stream(stream));
 }
 
 int32_t ogle_hip_ssd_topk_nms(const OgleNmsArgs* a, ogle_stream_t stream) {

@@ -90,6 +90,11 @@ int32_t launch_concat(const OgleConcatArgs& a, hipStream_t s);
 int32_t launch_transpose(const OgleTransposeArgs& a, hipStream_t s);
 int32_t launch_decode(const OgleDecodeArgs& a, hipStream_t s);
 int32_t launch_detect(const OgleDetectArgs& a, hipStream_t s);
+int32_t launch_unary(const OgleUnaryArgs& a, hipStream_t s);
+int32_t launch_binary(const OgleBinaryArgs& a, hipStream_t s);
+int32_t launch_batchnorm(const OgleBatchNormArgs& a, hipStream_t s);
+int32_t launch_gemm(const OgleGemmArgs& a, hipStream_t s);
+size_t gemm_workspace_bytes(const OgleGemmArgs& a);
 int32_t launch_topk_nms(const OgleNmsArgs& a, hipStream_t s);
 size_t topk_nms_lds_bytes(int stride, int topk);
 int32_t launch_expf(const float* x, float* y, int64_t n, hipStream_t s);

@@ -26,8 +26,10 @@ SYMBOLS = [
     "ogle_hip_convert", "ogle_hip_conv2d", "ogle_hip_dwconv2d", "ogle_hip_pwconv_gemm",
     "ogle_hip_pool2d", "ogle_hip_concat", "ogle_hip_ssd_decode", "ogle_hip_ssd_detect",
     "ogle_hip_expf", "ogle_hip_transpose", "ogle_hip_conv_workspace_bytes",
-    "ogle_hip_conv2d_batch", "ogle_hip_ssd_topk_nms",
+    "ogle_hip_conv2d_batch", "ogle_hip_ssd_topk_nms", "ogle_hip_unary", "ogle_hip_add",
+    "ogle_hip_batchnorm", "ogle_hip_gemm", "ogle_hip_gemm_workspace_bytes",
 ]
+UNARY_RELU, UNARY_CLIP = 0, 1
 
 
 class OgleError(RuntimeError):
@@ -99,6 +101,33 @@ class DetectArgs(ctypes.Structure):
     ]
 
 
+class UnaryArgs(ctypes.Structure):
+    _fields_ = [("input_dev", ctypes.c_void_p), ("output_dev", ctypes.c_void_p),
+                ("count", ctypes.c_int64), ("op", ctypes.c_int32), ("min_value", ctypes.c_float),
+                ("max_value", ctypes.c_float), ("dtype", ctypes.c_int32)]
+
+
+class BinaryArgs(ctypes.Structure):
+    _fields_ = [("a_dev", ctypes.c_void_p), ("b_dev", ctypes.c_void_p), ("output_dev", ctypes.c_void_p),
+                ("count", ctypes.c_int64), ("dtype", ctypes.c_int32)]
+
+
+class BatchNormArgs(ctypes.Structure):
+    _fields_ = [("input_dev", ctypes.c_void_p), ("gamma_dev", ctypes.c_void_p),
+                ("beta_dev", ctypes.c_void_p), ("mean_dev", ctypes.c_void_p),
+                ("var_dev", ctypes.c_void_p), ("output_dev", ctypes.c_void_p),
+                ("outer", ctypes.c_int64), ("channels", ctypes.c_int32), ("epsilon", ctypes.c_float),
+                ("dtype", ctypes.c_int32)]
+
+
+class GemmArgs(ctypes.Structure):
+    _fields_ = [("a_dev", ctypes.c_void_p), ("b_dev", ctypes.c_void_p), ("c_dev", ctypes.c_void_p),
+                ("y_dev", ctypes.c_void_p), ("m", ctypes.c_int32), ("n", ctypes.c_int32),
+                ("k", ctypes.c_int32), ("trans_b", ctypes.c_int32), ("c_rank", ctypes.c_int32),
+                ("alpha", ctypes.c_float), ("beta", ctypes.c_float),
+                ("workspace_dev", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t)]
+
+
 class NmsArgs(ctypes.Structure):
     _fields_ = [
         ("kept_count_dev", ctypes.c_void_p), ("kept_prior_dev", ctypes.c_void_p),
@@ -141,12 +170,16 @@ def lib():
                           ("ogle_hip_pwconv_gemm", ConvArgs), ("ogle_hip_pool2d", PoolArgs),
                           ("ogle_hip_concat", ConcatArgs), ("ogle_hip_ssd_decode", DecodeArgs),
                           ("ogle_hip_ssd_detect", DetectArgs),
-                          ("ogle_hip_ssd_topk_nms", NmsArgs),
+                          ("ogle_hip_ssd_topk_nms", NmsArgs), ("ogle_hip_unary", UnaryArgs),
+                          ("ogle_hip_add", BinaryArgs), ("ogle_hip_batchnorm", BatchNormArgs),
+                          ("ogle_hip_gemm", GemmArgs),
                           ("ogle_hip_transpose", TransposeArgs)):
             getattr(l, name).argtypes = [ctypes.POINTER(typ), ctypes.c_void_p]
         l.ogle_hip_conv2d_batch.argtypes = [ctypes.POINTER(ConvArgs), ctypes.c_int32, ctypes.c_void_p]
         l.ogle_hip_conv_workspace_bytes.argtypes = [ctypes.POINTER(ConvArgs)]
         l.ogle_hip_conv_workspace_bytes.restype = ctypes.c_size_t
+        l.ogle_hip_gemm_workspace_bytes.argtypes = [ctypes.POINTER(GemmArgs)]
+        l.ogle_hip_gemm_workspace_bytes.restype = ctypes.c_size_t
         l.ogle_hip_expf.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64,
                                     ctypes.c_void_p]
         _lib = l

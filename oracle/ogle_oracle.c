@@ -24,6 +24,10 @@
  *   oracle_fold_bn       conv(x; W', b') == BN(conv(x; W, b)) identity
  *   oracle_nchw_to_hwn4c4 / _inverse   round-trip identity + index formula
  *   oracle_topk_nms      brute-force python restatement on small inputs
+ *   oracle_add / _relu / _clip   numpy add / maximum / clip
+ *   oracle_batchnorm     float64 numpy formula, identity parameters -> x, and
+ *                        BN(conv) == conv with oracle_fold_bn's parameters
+ *   oracle_gemm          numpy float64 matmul (both transB settings, both bias ranks)
  * No function is "parity unpinned".
  *
  * All arithmetic is IEEE binary32 evaluated in the order the reference uses
@@ -456,6 +460,58 @@ int oracle_topk_nms(const float* scores, const int32_t* rects, int count,
   free(idx);
   free(dropped);
   return out;
+}
+
+/* ---- elementwise ops and Gemm of classification graphs ---------------------- */
+
+/* RT/nn/glsl/binary.glsl:8: texel-wise sum of two tensors of one shape. */
+void oracle_add(const float* a, const float* b, float* y, long n) {
+  for (long i = 0; i < n; ++i) y[i] = a[i] + b[i];
+}
+
+/* RT/nn/glsl/relu.glsl:8-10. */
+void oracle_relu(const float* x, float* y, long n) {
+  for (long i = 0; i < n; ++i) y[i] = x[i] > 0.0f ? x[i] : 0.0f;
+}
+
+/* RT/nn/glsl/clip.glsl:7-12: max with min_value first, then min with max_value. */
+void oracle_clip(const float* x, float* y, long n, float minv, float maxv) {
+  for (long i = 0; i < n; ++i) {
+    float v = x[i];
+    v = minv > v ? minv : v;
+    v = maxv < v ? maxv : v;
+    y[i] = v;
+  }
+}
+
+/* RT/nn/glsl/batchnorm.glsl:33: (x - mean) / sqrt(var + eps) * gamma + beta with the
+ * parameters indexed by the last (channel) dimension, evaluated left to right. */
+void oracle_batchnorm(const float* x, const float* gamma, const float* beta, const float* mean,
+                      const float* var, float* y, long outer, int channels, float eps) {
+  for (long i = 0; i < outer; ++i)
+    for (int c = 0; c < channels; ++c) {
+      const float d = x[i * channels + c] - mean[c];
+      const float q = d / sqrtf(var[c] + eps);
+      y[i * channels + c] = q * gamma[c] + beta[c];
+    }
+}
+
+/* RT/nn/glsl/gemm.glsl:33-95 with GemmCPU's reading of C (RT/nn/kernels/gemm_test.cc:9-40):
+ * y[i][j] = sum_m alpha * a[i][m] * b(m, j), terms added for m ascending, then
+ * + beta * c.  b is (N, K) when trans_b, (K, N) otherwise.  c is NULL, a row of N
+ * values broadcast over the rows (c_rank 1), or (M, N) (c_rank 2). */
+void oracle_gemm(const float* a, const float* b, const float* c, float* y, int m_rows, int n_cols,
+                 int k, int trans_b, int c_rank, float alpha, float beta) {
+  for (int i = 0; i < m_rows; ++i)
+    for (int j = 0; j < n_cols; ++j) {
+      float acc = 0.0f;
+      for (int m = 0; m < k; ++m) {
+        const float bv = trans_b ? b[(long)j * k + m] : b[(long)m * n_cols + j];
+        acc += alpha * a[(long)i * k + m] * bv;
+      }
+      if (c != NULL) acc += beta * (c_rank == 2 ? c[(long)i * n_cols + j] : c[j]);
+      y[(long)i * n_cols + j] = acc;
+    }
 }
 
 /* Number of threads the OpenMP loops above will use (for bench.py's report). */

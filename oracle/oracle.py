@@ -186,5 +186,51 @@ def topk_nms(scores, rects, top_k=100, nms_threshold=0.45):
     return order[:n].copy()
 
 
+def add(a, b):
+    a, b = _f32(a), _f32(b)
+    assert a.shape == b.shape
+    y = np.empty_like(a)
+    lib().oracle_add(_p(a), _p(b), _p(y), ctypes.c_long(a.size))
+    return y
+
+
+def relu(x):
+    x = _f32(x)
+    y = np.empty_like(x)
+    lib().oracle_relu(_p(x), _p(y), ctypes.c_long(x.size))
+    return y
+
+
+def clip(x, minv, maxv):
+    x = _f32(x)
+    y = np.empty_like(x)
+    lib().oracle_clip(_p(x), _p(y), ctypes.c_long(x.size), ctypes.c_float(minv), ctypes.c_float(maxv))
+    return y
+
+
+def batchnorm(x, gamma, beta, mean, var, eps):
+    """Parameters index the last dimension of x."""
+    x = _f32(x)
+    gamma, beta, mean, var = _f32(gamma), _f32(beta), _f32(mean), _f32(var)
+    c = x.shape[-1]
+    assert gamma.size == beta.size == mean.size == var.size == c
+    y = np.empty_like(x)
+    lib().oracle_batchnorm(_p(x), _p(gamma), _p(beta), _p(mean), _p(var), _p(y),
+                           ctypes.c_long(x.size // c), c, ctypes.c_float(eps))
+    return y
+
+
+def gemm(a, b, c=None, alpha=1.0, beta=1.0, trans_b=True):
+    a, b = _f32(a), _f32(b)
+    m, k = a.shape
+    n = b.shape[0] if trans_b else b.shape[1]
+    assert (b.shape[1] if trans_b else b.shape[0]) == k
+    c = _f32(c) if c is not None else None
+    y = np.empty((m, n), np.float32)
+    lib().oracle_gemm(_p(a), _p(b), _p(c), _p(y), m, n, k, int(bool(trans_b)),
+                      c.ndim if c is not None else 0, ctypes.c_float(alpha), ctypes.c_float(beta))
+    return y
+
+
 def num_threads():
     return lib().oracle_num_threads()

@@ -309,3 +309,50 @@ def test_topk_nms_against_python_restatement():
                     dropped[j] = True
         expect = [o for o, d in zip(order, dropped) if not d]
         np.testing.assert_array_equal(O.topk_nms(scores, rects, top_k, 0.45), expect)
+
+
+def test_elementwise_against_numpy():
+    r = rng(90)
+    a = r.normal(0, 2, (3, 5, 7, 6)).astype(np.float32)
+    b = r.normal(0, 2, a.shape).astype(np.float32)
+    np.testing.assert_array_equal(O.add(a, b), a + b)
+    np.testing.assert_array_equal(O.relu(a), np.maximum(a, 0))
+    np.testing.assert_array_equal(O.clip(a, -0.5, 1.25), np.clip(a, -0.5, 1.25))
+    # clip.glsl applies max(min_value) first and min(max_value) last: with min > max the result is max
+    np.testing.assert_array_equal(O.clip(a, 2.0, 1.0), np.full_like(a, 1.0))
+
+
+def test_batchnorm_against_float64_and_fold():
+    r = rng(91)
+    c = 10
+    x = r.normal(0, 2, (2, 4, 5, c)).astype(np.float32)
+    gamma, beta = r.uniform(0.5, 1.5, c).astype(np.float32), r.normal(0, 0.1, c).astype(np.float32)
+    mean, var = r.normal(0, 0.3, c).astype(np.float32), r.uniform(0.5, 1.5, c).astype(np.float32)
+    y = O.batchnorm(x, gamma, beta, mean, var, 1e-5)
+    ref = (x.astype(np.float64) - mean) / np.sqrt(var.astype(np.float64) + 1e-5) * gamma + beta
+    np.testing.assert_allclose(y, ref, rtol=2e-6, atol=2e-6)
+    # identity parameters leave x unchanged (sqrt(1 + 0) = 1)
+    one, zero = np.ones(c, np.float32), np.zeros(c, np.float32)
+    np.testing.assert_array_equal(O.batchnorm(x, one, zero, zero, one, 0.0), x)
+    # BN after a convolution equals the convolution with folded parameters (remapper.cc:142-149)
+    w = r.normal(0, 0.3, (c, 6, 3, 3)).astype(np.float32)
+    b0 = r.normal(0, 0.1, c).astype(np.float32)
+    xin = r.normal(0, 1, (1, 6, 6, 6)).astype(np.float32)
+    wf, bf = O.fold_bn(w, b0, gamma, beta, mean, var, 1e-5)
+    lhs = O.batchnorm(O.conv2d(xin, w, b0, 1, 1), gamma, beta, mean, var, 1e-5)
+    np.testing.assert_allclose(lhs, O.conv2d(xin, wf, bf, 1, 1), rtol=1e-4, atol=1e-4)
+
+
+def test_gemm_against_numpy():
+    r = rng(92)
+    for m, n, k in ((1, 7, 5), (4, 10, 33), (3, 1, 8)):
+        a = r.normal(0, 1, (m, k)).astype(np.float32)
+        for trans_b in (True, False):
+            b = r.normal(0, 1, (n, k) if trans_b else (k, n)).astype(np.float32)
+            bm = b.T if trans_b else b
+            for c in (None, r.normal(0, 1, n).astype(np.float32), r.normal(0, 1, (m, n)).astype(np.float32)):
+                got = O.gemm(a, b, c, alpha=0.75, beta=-1.5, trans_b=trans_b)
+                ref = 0.75 * (a.astype(np.float64) @ bm.astype(np.float64))
+                if c is not None:
+                    ref = ref - 1.5 * c
+                np.testing.assert_allclose(got, ref, rtol=1e-5, atol=1e-5)
