@@ -224,6 +224,33 @@ def kernel_table(iters=50, warm=5):
         pa = H.PoolArgs(x.data_ptr(), y.data_ptr(), n, h, h, c, oh, oh, k, s, p, typ, H.F32)
         row(name, timed(lambda: H.check(L.ogle_hip_pool2d(ctypes.byref(pa), st))), 0.0,
             4.0 * (x.numel() + y.numel()), "hbm")
+    # elementwise ops of classification graphs, on a 16x75x75x128 activation (36.9 MB)
+    shape = (16, 75, 75, 128)
+    xe, ye = torch.rand(shape, device="cuda"), torch.rand(shape, device="cuda")
+    oe = torch.empty(shape, device="cuda")
+    ua = H.UnaryArgs(xe.data_ptr(), oe.data_ptr(), xe.numel(), H.UNARY_CLIP, 0.0, 6.0, H.F32)
+    row("clip (16x75x75x128)", timed(lambda: H.check(L.ogle_hip_unary(ctypes.byref(ua), st))), 0.0,
+        8.0 * xe.numel(), "hbm")
+    ba = H.BinaryArgs(xe.data_ptr(), ye.data_ptr(), oe.data_ptr(), xe.numel(), H.F32)
+    row("add (16x75x75x128)", timed(lambda: H.check(L.ogle_hip_add(ctypes.byref(ba), st))), 0.0,
+        12.0 * xe.numel(), "hbm")
+    prm = [torch.rand(128, device="cuda") + 0.5 for _ in range(4)]
+    na = H.BatchNormArgs(xe.data_ptr(), prm[0].data_ptr(), prm[1].data_ptr(), prm[2].data_ptr(),
+                         prm[3].data_ptr(), oe.data_ptr(), xe.numel() // 128, 128, 1e-5, H.F32)
+    row("batchnorm (16x75x75x128)", timed(lambda: H.check(L.ogle_hip_batchnorm(ctypes.byref(na), st))),
+        0.0, 8.0 * xe.numel(), "hbm")
+    # classifier head: (16, 1024) x (1000, 1024)^T + bias, the Linear form on the MFMA kernel
+    ga_, gb_, gc_ = torch.rand(16, 1024, device="cuda"), torch.randn(1000, 1024, device="cuda") * 0.03, \
+        torch.rand(1000, device="cuda")
+    gy = torch.empty(16, 1000, device="cuda")
+    gg = H.GemmArgs(ga_.data_ptr(), gb_.data_ptr(), gc_.data_ptr(), gy.data_ptr(), 16, 1000, 1024, 1, 1,
+                    1.0, 1.0, None, 0)
+    need = L.ogle_hip_gemm_workspace_bytes(ctypes.byref(gg))
+    gws = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
+    if need:
+        gg.workspace_dev, gg.workspace_bytes = gws.data_ptr(), need
+    row("gemm classifier head (M=16 K=1024 N=1000)", timed(lambda: H.check(L.ogle_hip_gemm(ctypes.byref(gg), st))),
+        2.0 * 16 * 1000 * 1024, 4.0 * (16 * 1024 + 1000 * 1024 + 1000 + 16 * 1000), "hbm")
     return rows
 
 

@@ -92,6 +92,7 @@ def encode_pool_attr(kernel, stride, pad):
 ATTR_CONV2D, ATTR_CONST, ATTR_MAXPOOL, ATTR_AVEPOOL, ATTR_INPUT = 1, 2, 5, 6, 10
 ATTR_TRANSPOSE, ATTR_CONCAT, ATTR_RESHAPE = 12, 16, 17
 ATTR_SHAPE, ATTR_GATHER, ATTR_UNSQUEEZE = 13, 14, 15
+ATTR_BATCHNORM, ATTR_RELU, ATTR_FLATTEN, ATTR_BINARY, ATTR_GEMM, ATTR_CLIP = 3, 4, 7, 8, 9, 11
 
 
 def encode_node(name, type_, inputs, outputs, attr_field=None, attr_payload=b""):
@@ -155,6 +156,27 @@ class GraphBuilder:
 
     def add_reshape(self, name, x, shape_tensor):
         return self._emit(name, "Reshape", [x, shape_tensor], ATTR_RESHAPE, b"")
+
+    def add_add(self, name, a, b):
+        return self._emit(name, "Add", [a, b], ATTR_BINARY, b"")
+
+    def add_relu(self, name, x):
+        return self._emit(name, "Relu", [x], ATTR_RELU, b"")
+
+    def add_clip(self, name, x, minv, maxv):
+        return self._emit(name, "Clip", [x], ATTR_CLIP, _float(1, minv) + _float(2, maxv))
+
+    def add_batchnorm(self, name, x, gamma, beta, mean, var, epsilon=1e-5, momentum=0.9):
+        return self._emit(name, "BatchNormalization", [x, gamma, beta, mean, var], ATTR_BATCHNORM,
+                          _float(1, momentum) + _float(2, epsilon))
+
+    def add_gemm(self, name, a, b, c=None, alpha=1.0, beta=1.0, trans_b=True):
+        ins = [a, b] + ([c] if c is not None else [])
+        return self._emit(name, "Gemm", ins, ATTR_GEMM,
+                          _float(1, alpha) + _float(2, beta) + _int(3, int(bool(trans_b))))
+
+    def add_flatten(self, name, x, axis=1):
+        return self._emit(name, "Flatten", [x], ATTR_FLATTEN, _int(1, axis))
 
     def add_shape(self, name, x):
         return self._emit(name, "Shape", [x], ATTR_SHAPE, b"")

@@ -242,4 +242,29 @@ void Program::RunTranspose(const OgleTransposeArgs& a) const {
   Check(ogle_hip_transpose(&a, context_->stream()), "ogle_hip_transpose");
 }
 
+void Program::RunUnary(const OgleUnaryArgs& a) const {
+  const void* reads[] = {a.input_dev};
+  const void* writes[] = {a.output_dev};
+  context_->BeforeLaunch(reads, 1, writes, 1);
+  Check(ogle_hip_unary(&a, context_->stream()), "ogle_hip_unary");
+}
+void Program::RunAdd(const OgleBinaryArgs& a) const {
+  const void* reads[] = {a.a_dev, a.b_dev};
+  const void* writes[] = {a.output_dev};
+  context_->BeforeLaunch(reads, 2, writes, 1);
+  Check(ogle_hip_add(&a, context_->stream()), "ogle_hip_add");
+}
+void Program::RunBatchNorm(const OgleBatchNormArgs& a) const {
+  const void* reads[] = {a.input_dev, a.gamma_dev, a.beta_dev, a.mean_dev, a.var_dev};
+  const void* writes[] = {a.output_dev};
+  context_->BeforeLaunch(reads, 5, writes, 1);
+  Check(ogle_hip_batchnorm(&a, context_->stream()), "ogle_hip_batchnorm");
+}
+void Program::RunGemm(const OgleGemmArgs& a) const {
+  const void* reads[] = {a.a_dev, a.b_dev, a.c_dev};
+  const void* writes[] = {a.y_dev};
+  context_->BeforeLaunch(reads, 3, writes, 1);
+  Check(ogle_hip_gemm(&a, context_->stream()), "ogle_hip_gemm");
+}
+
 }  // namespace opengl

@@ -35,6 +35,10 @@ class Program {
   void RunConcat(const OgleConcatArgs& args) const;
   void RunDecode(const OgleDecodeArgs& args) const;
   void RunTranspose(const OgleTransposeArgs& args) const;
+  void RunUnary(const OgleUnaryArgs& args) const;
+  void RunAdd(const OgleBinaryArgs& args) const;
+  void RunBatchNorm(const OgleBatchNormArgs& args) const;
+  void RunGemm(const OgleGemmArgs& args) const;
 
  private:
   void Check(int32_t status, const char* what) const;
