@@ -38,6 +38,12 @@ struct Vec<float> {
   __device__ static void store(float* p, const float (&v)[4]) {
     *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
   }
+  __device__ static u32x4 pack(const float (&v)[4]) {
+    u32x4 t;
+    t.x = __float_as_uint(v[0]); t.y = __float_as_uint(v[1]);
+    t.z = __float_as_uint(v[2]); t.w = __float_as_uint(v[3]);
+    return t;
+  }
 };
 template <>
 struct Vec<__half> {
@@ -68,47 +74,79 @@ struct Vec<__half> {
     for (int i = 0; i < 4; ++i) h[i] = __floats2half2_rn(v[2 * i], v[2 * i + 1]);
     *reinterpret_cast<uint4*>(p) = t;
   }
+  __device__ static u32x4 pack(const float (&v)[8]) {
+    u32x4 t;
+    __half2* h = reinterpret_cast<__half2*>(&t);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) h[i] = __floats2half2_rn(v[2 * i], v[2 * i + 1]);
+    return t;
+  }
 };
+
+// Unsigned division by a number fixed at launch: q = (mulhi(n, mul) + n) >> shift,
+// exact for every n below 2^31 (Granlund and Montgomery's round-up form).
+struct FastDiv {
+  unsigned mul, shift, d;
+};
+
+__device__ __forceinline__ unsigned fast_div(unsigned n, const FastDiv& f) {
+  return (__umulhi(n, f.mul) + n) >> f.shift;
+}
 
 // 3x3, dilation 1, stride S, channel count a multiple of the vector width.
 // A thread owns a patch of R output rows x Q output columns of one channel vector.
+// Index arithmetic is kept off the vector ALU as far as possible (the kernel issues
+// about as many address instructions as FMAs otherwise): the thread index is split
+// with multiply-high divisions, input offsets are a row term plus a column term, and
+// a tap outside the image just gets the out-of-range bit set in its offset.
 template <typename T, int S, int R, int Q>
 __global__ __launch_bounds__(256) void dwconv3x3_strip(
     const T* __restrict__ x, const T* __restrict__ w, const float* __restrict__ bias,
-    T* __restrict__ y, int n, int h, int wd, int c, int oh, int ow, int pad, Epilogue ep,
-    unsigned x_bytes) {
+    T* __restrict__ y, int h, int wd, int c, int oh, int ow, int pad, Epilogue ep,
+    unsigned x_bytes, unsigned y_bytes, unsigned total, FastDiv div_cv, FastDiv div_cols,
+    FastDiv div_strips) {
   constexpr int V = Vec<T>::N;
   constexpr int IN_ROWS = (R - 1) * S + 3;
   constexpr int IN_COLS = (Q - 1) * S + 3;
-  const int cv = c / V;
-  const int strips = (oh + R - 1) / R;
-  const int colgroups = (ow + Q - 1) / Q;
-  const long total = (long)n * strips * colgroups * cv;
+  constexpr unsigned ESZ = sizeof(T);
+  constexpr unsigned kOut = 0x80000000u;  // offsets at or above this are outside every operand
   // Consecutive logical blocks (neighbouring pixels and strips, which share halo
   // rows) are kept on one XCD so that the re-read rows hit that XCD's L2.
-  const long idx = (long)xcd_swizzle(blockIdx.x, gridDim.x) * blockDim.x + threadIdx.x;
+  const unsigned idx = (unsigned)xcd_swizzle(blockIdx.x, gridDim.x) * 256u + threadIdx.x;
   if (idx >= total) return;
-  const int cg = (int)(idx % cv);
-  long t = idx / cv;
-  const int oxg = (int)(t % colgroups);
-  t /= colgroups;
-  const int strip = (int)(t % strips);
-  const int b = (int)(t / strips);
+  const unsigned t1 = fast_div(idx, div_cv);
+  const int cg = (int)(idx - t1 * div_cv.d);
+  const unsigned t2 = fast_div(t1, div_cols);
+  const int oxg = (int)(t1 - t2 * div_cols.d);
+  const unsigned b = fast_div(t2, div_strips);
+  const int strip = (int)(t2 - b * div_strips.d);
   const int ch = cg * V;
   const int oy0 = strip * R;
   const int ox0 = oxg * Q;
 
   float wt[9][V];
 #pragma unroll
-  for (int tap = 0; tap < 9; ++tap) Vec<T>::load(w + (long)tap * c + ch, wt[tap]);
+  for (int tap = 0; tap < 9; ++tap) Vec<T>::load(w + tap * c + ch, wt[tap]);
 
   float acc[R][Q][V];
+  {
+    float bv[V];
 #pragma unroll
-  for (int r = 0; r < R; ++r)
+    for (int v = 0; v < V; ++v) bv[v] = 0.f;
+    if (bias != nullptr) {
 #pragma unroll
-    for (int q = 0; q < Q; ++q)
+      for (int v = 0; v < V; v += 4) {
+        const float4 t = *reinterpret_cast<const float4*>(bias + ch + v);  // ch % 4 == 0
+        bv[v] = t.x; bv[v + 1] = t.y; bv[v + 2] = t.z; bv[v + 3] = t.w;
+      }
+    }
 #pragma unroll
-      for (int v = 0; v < V; ++v) acc[r][q][v] = bias != nullptr ? bias[ch + v] : 0.f;
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int q = 0; q < Q; ++q)
+#pragma unroll
+        for (int v = 0; v < V; ++v) acc[r][q][v] = bv[v];
+  }
 
   // Every input vector the patch needs is requested up front with buffer loads;
   // taps outside the image get an out-of-range offset and come back as zeros, so
@@ -117,21 +155,29 @@ __global__ __launch_bounds__(256) void dwconv3x3_strip(
   const int ix0 = ox0 * S - pad;
   const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<T*>(x), 0, (int)x_bytes, 0x00020000);
-  const unsigned img = (unsigned)b * (unsigned)(h * wd * c) + (unsigned)ch;
-  u32x4 raw[IN_ROWS][IN_COLS];
+  const unsigned row_bytes = (unsigned)(wd * c) * ESZ;
+  const unsigned img = (b * (unsigned)h) * row_bytes + (unsigned)ch * ESZ;
+  unsigned row_off[IN_ROWS], col_off[IN_COLS];
 #pragma unroll
   for (int j = 0; j < IN_ROWS; ++j) {
     const int iy = iy0 + j;
-    const bool row_ok = iy >= 0 && iy < h;
+    row_off[j] = (unsigned)iy < (unsigned)h ? img + (unsigned)iy * row_bytes : kOut;
+  }
+#pragma unroll
+  for (int s = 0; s < IN_COLS; ++s) {
+    const int ix = ix0 + s;
+    col_off[s] = (unsigned)ix < (unsigned)wd ? (unsigned)(ix * c) * ESZ : kOut;
+  }
+  u32x4 raw[IN_ROWS][IN_COLS];
+#pragma unroll
+  for (int j = 0; j < IN_ROWS; ++j)
 #pragma unroll
     for (int s = 0; s < IN_COLS; ++s) {
-      const int ix = ix0 + s;
-      const bool ok = row_ok && ix >= 0 && ix < wd;
-      const unsigned off =
-          ok ? (img + (unsigned)((iy * wd + ix) * c)) * (unsigned)sizeof(T) : 0x80000000u;
+      // a valid row plus a valid column stays below 2^31; either term being kOut sets
+      // the top bit of the OR, whatever the sum wrapped to
+      const unsigned off = (row_off[j] + col_off[s]) | ((row_off[j] | col_off[s]) & kOut);
       raw[j][s] = __builtin_amdgcn_raw_buffer_load_b128(rx, (int)off, 0, 0);
     }
-  }
 #pragma unroll
   for (int j = 0; j < IN_ROWS; ++j) {
     float in[IN_COLS][V];
@@ -151,18 +197,20 @@ __global__ __launch_bounds__(256) void dwconv3x3_strip(
       }
     }
   }
+  const __amdgpu_buffer_rsrc_t ry = __builtin_amdgcn_make_buffer_rsrc(y, 0, (int)y_bytes, 0x00020000);
+  const unsigned out_row_bytes = (unsigned)(ow * c) * ESZ;
+  const unsigned out0 = (b * (unsigned)oh + (unsigned)oy0) * out_row_bytes +
+                        (unsigned)(ox0 * c + ch) * ESZ;
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    const int oy = oy0 + r;
-    if (oy >= oh) break;
 #pragma unroll
     for (int q = 0; q < Q; ++q) {
-      const int ox = ox0 + q;
-      if (ox >= ow) break;
       float out[V];
 #pragma unroll
       for (int v = 0; v < V; ++v) out[v] = apply_epilogue(acc[r][q][v], ep);
-      Vec<T>::store(y + (((long)b * oh + oy) * ow + ox) * c + ch, out);
+      const bool ok = oy0 + r < oh && ox0 + q < ow;
+      const unsigned off = ok ? out0 + (unsigned)r * out_row_bytes + (unsigned)(q * c) * ESZ : kOut;
+      __builtin_amdgcn_raw_buffer_store_b128(Vec<T>::pack(out), ry, (int)off, 0, 0);
     }
   }
 }
@@ -197,17 +245,29 @@ __global__ __launch_bounds__(256) void dwconv_general(
   }
 }
 
+FastDiv make_fast_div(unsigned d) {
+  FastDiv f{0, 0, d};
+  unsigned l = 0;
+  while ((1ull << l) < d) ++l;
+  f.shift = l;
+  f.mul = (unsigned)(((1ull << 32) * ((1ull << l) - d)) / d + 1);
+  return f;
+}
+
 template <typename T, int S, int R, int Q = 1>
 int32_t launch_strip(const OgleConvArgs& a, hipStream_t s, const Epilogue& ep) {
   constexpr int V = Vec<T>::N;
-  const long total =
-      (long)a.n * ((a.out_h + R - 1) / R) * ((a.out_w + Q - 1) / Q) * (a.in_c / V);
+  const int strips = (a.out_h + R - 1) / R, cols = (a.out_w + Q - 1) / Q, cv = a.in_c / V;
+  const long total = (long)a.n * strips * cols * cv;
   const int blocks = (ceil_div(total, 256) + 7) / 8 * 8;  // whole XCD rounds
   hipLaunchKernelGGL((dwconv3x3_strip<T, S, R, Q>), dim3(blocks), dim3(256), 0, s,
                      static_cast<const T*>(a.input_dev), static_cast<const T*>(a.filter_dev),
-                     a.bias_dev, static_cast<T*>(a.output_dev), a.n, a.in_h, a.in_w, a.in_c,
-                     a.out_h, a.out_w, a.padding, ep,
-                     (unsigned)((long)a.n * a.in_h * a.in_w * a.in_c * sizeof(T)));
+                     a.bias_dev, static_cast<T*>(a.output_dev), a.in_h, a.in_w, a.in_c, a.out_h,
+                     a.out_w, a.padding, ep,
+                     (unsigned)((long)a.n * a.in_h * a.in_w * a.in_c * sizeof(T)),
+                     (unsigned)((long)a.n * a.out_h * a.out_w * a.in_c * sizeof(T)), (unsigned)total,
+                     make_fast_div((unsigned)cv), make_fast_div((unsigned)cols),
+                     make_fast_div((unsigned)strips));
   return check_launch("dwconv3x3_strip");
 }
 
@@ -231,7 +291,10 @@ int32_t run_dw(const OgleConvArgs& a, hipStream_t s) {
   const Epilogue ep = make_epilogue(a.act, a.min_value, a.max_value, a.act_variant);
   constexpr int V = Vec<T>::N;
   // the strip kernel addresses the input with 32-bit byte offsets (buffer loads)
-  const bool fits = (long)a.n * a.in_h * a.in_w * a.in_c * (long)sizeof(T) < 0x7fffffffL;
+  // and the bias with 16-byte loads
+  const bool fits = (long)a.n * a.in_h * a.in_w * a.in_c * (long)sizeof(T) < 0x7fffffffL &&
+                    (long)a.n * a.out_h * a.out_w * a.in_c * (long)sizeof(T) < 0x7fffffffL &&
+                    (reinterpret_cast<uintptr_t>(a.bias_dev) & 15u) == 0;
   if (a.kernel_size == 3 && a.dilation == 1 && a.in_c % V == 0 && fits &&
       (a.stride == 1 || a.stride == 2)) {
     if (a.stride == 1) return pick_strip<T, 1>(a, s, ep);
