@@ -516,3 +516,31 @@ def test_topk_nms_rejects_bad_sizes():
     assert H.lib().ogle_hip_ssd_topk_nms(ctypes.byref(a), 0) == H.ERR_UNSUPPORTED
     a.stride = 100
     assert H.lib().ogle_hip_ssd_topk_nms(ctypes.byref(a), 0) == H.ERR_INVALID_ARG   # null pointers
+
+
+def test_kernels_against_committed_vectors():
+    """The HIP kernels on the inputs stored in tests/golden/oracle_vectors.npz against the
+    outputs stored beside them (written by the oracle, tests/golden/make_golden.py)."""
+    import os
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "oracle_vectors.npz")
+    g = dict(np.load(path))
+    x = g["dense_x"]
+    for name, w, b, kw, ref in (
+            ("dense", g["dense_w"], g["dense_b"], dict(stride=2, pad=1, act=H.ACT_RELU), g["dense_y"]),
+            ("dw", g["dw_w"], g["dw_b"], dict(stride=1, pad=1, groups=8, act=H.ACT_CLIP, maxv=6.0), g["dw_y"]),
+            ("pw", g["pw_w"], g["pw_b"], dict(act=H.ACT_CLIP, minv=-1.0, maxv=0.5, variant=H.VARIANT_PW), g["pw_y"])):
+        got = gpu_conv(x, w, b, **kw)
+        scale = O.conv2d_abs(x, w, b, kw.get("stride", 1), kw.get("pad", 0), 1, kw.get("groups", 1))
+        assert_conv_close(got, ref, scale, FP32_RTOL, name)
+    np.testing.assert_array_equal(gpu_pool(x, 3, 2, 1, O.POOL_MAX), g["maxpool_y"])
+    np.testing.assert_allclose(gpu_pool(x, 2, 2, 0, O.POOL_AVG), g["avgpool_y"], rtol=1e-6, atol=1e-7)
+    np.testing.assert_array_equal(gpu_concat([g["cat_a"], g["cat_b"], g["cat_c"]], 1), g["cat_y"])
+    res, boxes = gpu_detect(g["ssd_logits"], g["ssd_pred"], g["ssd_anchors"], 0.3, 320.0, 240.0)
+    np.testing.assert_allclose(boxes, g["ssd_boxes"], rtol=1e-5, atol=1e-6)
+    for i in range(2):
+        ora = {k: g["info%d_%s" % (i, k)] for k in ("prior", "cls", "score", "box", "rect")}
+        assert_same_detections(res[i], ora, g["ssd_logits"][i], 0.3, "image %d" % i)
+        n = len(ora["prior"])
+        final = gpu_topk_nms(np.array([n], np.int32), ora["prior"][None], ora["cls"][None],
+                             ora["score"][None], ora["rect"][None], 5, 0.45)
+        np.testing.assert_array_equal(final[0]["prior"], ora["prior"][g["info%d_keep" % i]])

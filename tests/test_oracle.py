@@ -356,3 +356,19 @@ def test_gemm_against_numpy():
                 if c is not None:
                     ref = ref - 1.5 * c
                 np.testing.assert_allclose(got, ref, rtol=1e-5, atol=1e-5)
+
+
+def test_oracle_matches_committed_vectors():
+    """tests/golden/oracle_vectors.npz was written by tests/golden/make_golden.py; the oracle
+    built from today's sources must reproduce every array in it bit for bit."""
+    import importlib.util
+    import os
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    spec = importlib.util.spec_from_file_location("make_golden", os.path.join(here, "make_golden.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    now = mod.cases()
+    with np.load(os.path.join(here, "oracle_vectors.npz")) as stored:
+        assert sorted(stored.files) == sorted(now)
+        for k in stored.files:
+            np.testing.assert_array_equal(stored[k], now[k], err_msg=k)
