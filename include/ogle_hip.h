@@ -398,7 +398,7 @@ int32_t ogle_hip_ssd_detect(const OgleDetectArgs* args, ogle_stream_t stream);
  * Inputs are indexed [b*stride + r], r < kept_count_dev[b]; outputs
  * [b*topk + r], r < final_count_dev[b], in sorted order.  kept_box_dev /
  * final_box_dev may both be NULL.  1 <= topk <= 1024, stride <= 8192 and
- * 4*stride + 44*topk + 1.2 KB must fit 64 KB of LDS (OGLE_ERR_UNSUPPORTED otherwise).
+ * 4*stride + 28*topk + 1.2 KB must fit 64 KB of LDS (OGLE_ERR_UNSUPPORTED otherwise).
  */
 typedef struct OgleNmsArgs {
   const int32_t* kept_count_dev;

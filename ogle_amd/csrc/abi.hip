@@ -428,7 +428,7 @@ int32_t ogle_hip_ssd_topk_nms(const OgleNmsArgs* a, ogle_stream_t stream) {
     return fail(OGLE_ERR_UNSUPPORTED, "ssd_topk_nms: topk must be in 1..1024");
   if (a->stride > 8192 || topk_nms_lds_bytes(a->stride, a->topk) > 64 * 1024)
     return fail(OGLE_ERR_UNSUPPORTED,  // scores and candidates of one image are staged in LDS
-                "ssd_topk_nms: more than 8192 entries per image, or stride*4 + topk*44 bytes "
+                "ssd_topk_nms: more than 8192 entries per image, or stride*4 + topk*28 bytes "
                 "exceed 64 KB of LDS");
   if (a->batch > 0) {
     if (!a->kept_count_dev || !a->final_count_dev)

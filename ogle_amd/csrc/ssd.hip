@@ -154,8 +154,8 @@ __global__ __launch_bounds__(256) void ssd_detect_kernel(DetectParams p) {
 // leaves its results UNCOMPACTED in the kept_* arrays at the prior's own slot (prior
 // index, or -1 when the prior is dropped); ssd_compact_kernel then packs each
 // image's survivors to the front in place, in prior order.  A slot is only ever
-// overwritten by an entry that came from the same or a later slot, after the chunk
-// holding it has been read, so the in-place pass needs one barrier per chunk.
+// overwritten by an entry that came from the same or a later slot, after the round
+// holding it has been read.
 constexpr int kScorePriors = 64;  // priors per workgroup of ssd_score_kernel
 
 __global__ __launch_bounds__(256) void ssd_score_kernel(DetectParams p) {
@@ -215,46 +215,70 @@ __global__ __launch_bounds__(256) void ssd_score_kernel(DetectParams p) {
   p.kept_rect[at] = make_int4((int)xmin, (int)ymin, (int)(xmax - xmin), (int)(ymax - ymin));
 }
 
-__global__ __launch_bounds__(256) void ssd_compact_kernel(DetectParams p) {
-  __shared__ int wave_count[4];
+constexpr int kCompactThreads = 1024;
+constexpr int kCompactWaves = kCompactThreads / 64;
+constexpr int kCompactSlots = 2;  // entries per thread and round
+
+__global__ __launch_bounds__(kCompactThreads) void ssd_compact_kernel(DetectParams p) {
+  // A round covers kCompactThreads * kCompactSlots consecutive slots (all 1917 priors
+  // of an SSD300 image in one).  Every entry of the round is read into registers with
+  // all loads in flight, a barrier separates the reads from the writes, and a slot is
+  // only ever overwritten by an entry from the same or a later slot, so the pass can
+  // work in place.
+  __shared__ int wave_count[kCompactSlots][kCompactWaves];
   const int b = blockIdx.x;
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const long row0 = (long)b * p.priors;
   int base = 0;
-  for (int start = 0; start < p.priors; start += 256) {
-    const int prior = start + tid;
-    int kept = -1, cls = 0;
-    float score = 0.f;
-    float4 box = make_float4(0.f, 0.f, 0.f, 0.f);
-    int4 rect = make_int4(0, 0, 0, 0);
-    if (prior < p.priors) {
-      kept = p.kept_prior[row0 + prior];
-      if (kept >= 0) {
-        cls = p.kept_class[row0 + prior];
-        score = p.kept_score[row0 + prior];
-        box = p.kept_box[row0 + prior];
-        rect = p.kept_rect[row0 + prior];
+  for (int start = 0; start < p.priors; start += kCompactThreads * kCompactSlots) {
+    int kept[kCompactSlots], cls[kCompactSlots], before[kCompactSlots];
+    float score[kCompactSlots];
+    float4 box[kCompactSlots];
+    int4 rect[kCompactSlots];
+#pragma unroll
+    for (int u = 0; u < kCompactSlots; ++u) {
+      const int prior = start + u * kCompactThreads + tid;
+      kept[u] = prior < p.priors ? p.kept_prior[row0 + prior] : -1;
+    }
+#pragma unroll
+    for (int u = 0; u < kCompactSlots; ++u) {
+      const int prior = start + u * kCompactThreads + tid;
+      cls[u] = 0;
+      score[u] = 0.f;
+      box[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+      rect[u] = make_int4(0, 0, 0, 0);
+      if (kept[u] >= 0) {
+        cls[u] = p.kept_class[row0 + prior];
+        score[u] = p.kept_score[row0 + prior];
+        box[u] = p.kept_box[row0 + prior];
+        rect[u] = p.kept_rect[row0 + prior];
+      }
+      const unsigned long long ballot = __ballot(kept[u] >= 0);
+      before[u] = __popcll(ballot & ((1ull << lane) - 1ull));
+      if (lane == 0) wave_count[u][wave] = __popcll(ballot);
+    }
+    __syncthreads();  // every read of this round is done; wave counts are visible
+    int round_total = 0;
+#pragma unroll
+    for (int u = 0; u < kCompactSlots; ++u) {
+      int slot = base + round_total + before[u];
+#pragma unroll
+      for (int wv = 0; wv < kCompactWaves; ++wv) {
+        const int cnt = wave_count[u][wv];
+        if (wv < wave) slot += cnt;
+        round_total += cnt;
+      }
+      if (kept[u] >= 0) {
+        p.kept_prior[row0 + slot] = kept[u];
+        p.kept_class[row0 + slot] = cls[u];
+        p.kept_score[row0 + slot] = score[u];
+        p.kept_box[row0 + slot] = box[u];
+        p.kept_rect[row0 + slot] = rect[u];
       }
     }
-    const bool keep = kept >= 0;
-    const unsigned long long ballot = __ballot(keep);
-    const int before = __popcll(ballot & ((1ull << lane) - 1ull));
-    if (lane == 0) wave_count[wave] = __popcll(ballot);
-    __syncthreads();  // every read of this chunk is done; wave counts are visible
-    int wave_base = 0;
-    for (int wv = 0; wv < wave; ++wv) wave_base += wave_count[wv];
-    const int chunk_total = wave_count[0] + wave_count[1] + wave_count[2] + wave_count[3];
-    if (keep) {
-      const long slot = row0 + base + wave_base + before;
-      p.kept_prior[slot] = kept;
-      p.kept_class[slot] = cls;
-      p.kept_score[slot] = score;
-      p.kept_box[slot] = box;
-      p.kept_rect[slot] = rect;
-    }
-    base += chunk_total;
-    __syncthreads();  // wave_count is rewritten by the next chunk
+    base += round_total;
+    __syncthreads();  // wave_count is rewritten by the next round
   }
   if (tid == 0) p.kept_count[b] = base;
 }
@@ -335,15 +359,14 @@ __device__ __forceinline__ int block_rank(bool flag, int* wave_count, int lane, 
 
 __global__ __launch_bounds__(kNmsThreads) void ssd_topk_nms_kernel(NmsParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char nms_lds[];
-  // keys[stride] | cand_key[topk] | cand_idx[topk] | sel[topk] | rect[topk] | frect[topk] |
+  // keys[stride] | cand_key[topk] | cand_idx[topk] | sel[topk] | frect[topk] |
   // hist[256] | misc[kNmsWaves + 2]     (topk and stride rounded up to 4)
   const int tpad = (p.topk + 3) & ~3;
   unsigned* keys = reinterpret_cast<unsigned*>(nms_lds);
   unsigned* cand_key = keys + ((p.stride + 3) & ~3);
   int* cand_idx = reinterpret_cast<int*>(cand_key + tpad);
   int* sel = cand_idx + tpad;
-  int4* rects = reinterpret_cast<int4*>(sel + tpad);
-  float4* frects = reinterpret_cast<float4*>(rects + tpad);
+  float4* frects = reinterpret_cast<float4*>(sel + tpad);
   int* hist = reinterpret_cast<int*>(frects + tpad);
   int* misc = hist + 256;  // [0..kNmsWaves) wave counts, then the chosen digit and the count above it
 
@@ -422,34 +445,40 @@ __global__ __launch_bounds__(kNmsThreads) void ssd_topk_nms_kernel(NmsParams p) 
   for (int r = m + tid; r < ((m + 3) & ~3); r += kNmsThreads) cand_key[r] = 0u;  // padding ranks last
   __syncthreads();
 
-  // 3. rank among the selected entries (they are in list order, so position breaks ties)
+  // 3. thread r owns selected entry r (topk <= the thread count): its record is
+  // requested now, and its rank among the selected entries (they are in list order,
+  // so position breaks ties) is counted while the loads are in flight
   const int mpad = (m + 3) & ~3;
-  for (int r = tid; r < m; r += kNmsThreads) {
-    const unsigned kr = cand_key[r];
-    int rank = 0;
+  const bool owner = tid < m;
+  int my_prior = 0, my_class = 0, my_rank = 0;
+  float my_score = 0.f;
+  float4 my_box = make_float4(0.f, 0.f, 0.f, 0.f);
+  int4 my_rect = make_int4(0, 0, 0, 0);
+  if (owner) {
+    const long src = row0 + cand_idx[tid];
+    my_rect = p.kept_rect[src];
+    my_prior = p.kept_prior[src];
+    my_class = p.kept_class[src];
+    my_score = p.kept_score[src];
+    if (p.kept_box != nullptr) my_box = p.kept_box[src];
+    const unsigned kr = cand_key[tid];
     for (int j = 0; j < mpad; j += 4) {
       const uint4 v = *reinterpret_cast<const uint4*>(cand_key + j);
-      rank += (v.x > kr || (v.x == kr && j + 0 < r)) ? 1 : 0;
-      rank += (v.y > kr || (v.y == kr && j + 1 < r)) ? 1 : 0;
-      rank += (v.z > kr || (v.z == kr && j + 2 < r)) ? 1 : 0;
-      rank += (v.w > kr || (v.w == kr && j + 3 < r)) ? 1 : 0;
+      my_rank += (v.x > kr || (v.x == kr && j + 0 < tid)) ? 1 : 0;
+      my_rank += (v.y > kr || (v.y == kr && j + 1 < tid)) ? 1 : 0;
+      my_rank += (v.z > kr || (v.z == kr && j + 2 < tid)) ? 1 : 0;
+      my_rank += (v.w > kr || (v.w == kr && j + 3 < tid)) ? 1 : 0;
     }
-    sel[rank] = cand_idx[r];
-  }
-  __syncthreads();
-  for (int r = tid; r < m; r += kNmsThreads) {
-    const int4 q = p.kept_rect[row0 + sel[r]];
-    rects[r] = q;
     // corners as the host's iou() forms them: integer sums converted to float
-    frects[r] = make_float4((float)q.x, (float)q.y, (float)(q.x + q.z), (float)(q.y + q.w));
+    frects[my_rank] = make_float4((float)my_rect.x, (float)my_rect.y, (float)(my_rect.x + my_rect.z),
+                                  (float)(my_rect.y + my_rect.w));
   }
+  int* dropped = sel;  // [rank] -> 1 if suppressed
+  for (int r = tid; r < m; r += kNmsThreads) dropped[r] = 0;
   __syncthreads();
 
   // 4. NMS: all (i, j) pairs with i < j are spread over the workgroup; a pair that
   // overlaps by more than the threshold marks j (every writer stores the same value)
-  int* dropped = cand_idx;  // the candidate list is no longer needed
-  for (int r = tid; r < m; r += kNmsThreads) dropped[r] = 0;
-  __syncthreads();
   if (m > 1) {
     // pair number t = i * m + j, advanced by the thread count per step without dividing
     const int step_i = kNmsThreads / m, step_j = kNmsThreads - step_i * m;
@@ -465,33 +494,35 @@ __global__ __launch_bounds__(kNmsThreads) void ssd_topk_nms_kernel(NmsParams p) 
   }
   __syncthreads();
 
-  // ordered compaction of the survivors into the output lists
-  int base = 0;
-  const long out0 = (long)b * p.topk;
-  for (int start = 0; start < m; start += kNmsThreads) {
-    const int j = start + tid;
-    const bool keep = j < m && dropped[j] == 0;
-    int total;
+  // output position of every surviving rank (ordered compaction over the ranks), then
+  // each owner writes its record from registers
+  int* out_pos = cand_idx;  // the candidate list is no longer needed
+  int total;
+  {
+    const bool keep = tid < m && dropped[tid] == 0;
     const int before = block_rank(keep, misc, lane, wave, &total);
-    if (keep) {
-      const long src = row0 + sel[j];
-      const long dst = out0 + base + before;
-      p.out_prior[dst] = p.kept_prior[src];
-      p.out_class[dst] = p.kept_class[src];
-      p.out_score[dst] = p.kept_score[src];
-      if (p.out_box != nullptr) p.out_box[dst] = p.kept_box[src];
-      p.out_rect[dst] = rects[j];
-    }
-    base += total;
+    if (tid < m) out_pos[tid] = keep ? before : -1;
   }
-  if (tid == 0) p.out_count[b] = base;
+  __syncthreads();
+  if (owner) {
+    const int o = out_pos[my_rank];
+    if (o >= 0) {
+      const long dst = (long)b * p.topk + o;
+      p.out_prior[dst] = my_prior;
+      p.out_class[dst] = my_class;
+      p.out_score[dst] = my_score;
+      if (p.out_box != nullptr) p.out_box[dst] = my_box;
+      p.out_rect[dst] = my_rect;
+    }
+  }
+  if (tid == 0) p.out_count[b] = total;
 }
 
 }  // namespace
 
 size_t topk_nms_lds_bytes(int stride, int topk) {
   const size_t tpad = (size_t)((topk + 3) & ~3);
-  return 4 * (size_t)((stride + 3) & ~3) + 4 * 3 * tpad + (sizeof(int4) + sizeof(float4)) * tpad +
+  return 4 * (size_t)((stride + 3) & ~3) + 4 * 3 * tpad + sizeof(float4) * tpad +
          4 * (256 + kNmsWaves + 2);
 }
 
@@ -555,7 +586,7 @@ int32_t launch_detect(const OgleDetectArgs& a, hipStream_t s) {
                        dim3(256), sizeof(float) * kScorePriors * (size_t)a.classes, s, p);
     const int32_t st = check_launch("ssd_score_kernel");
     if (st != OGLE_OK) return st;
-    hipLaunchKernelGGL(ssd_compact_kernel, dim3((unsigned)a.batch), dim3(256), 0, s, p);
+    hipLaunchKernelGGL(ssd_compact_kernel, dim3((unsigned)a.batch), dim3(kCompactThreads), 0, s, p);
     return check_launch("ssd_compact_kernel");
   }
   hipLaunchKernelGGL(ssd_detect_kernel, dim3((unsigned)a.batch), dim3(256), lds, s, p);

@@ -156,7 +156,7 @@ void Detector::GenerateBoxInfo(int image, std::vector<BoxInfo>* box_infos) const
 bool Detector::UsesDeviceNms() const {
   // the device kernel stages one image's scores and candidates in 64 KB of LDS
   return options_.device_nms && options_.topk >= 1 && options_.topk <= 1024 && priors_ <= 8192 &&
-         4L * priors_ + 44L * options_.topk + 2048 <= 64 * 1024;
+         4L * priors_ + 28L * options_.topk + 2048 <= 64 * 1024;
 }
 
 void Detector::EnqueueTopkNms() {
