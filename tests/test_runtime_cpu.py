@@ -143,7 +143,8 @@ def test_runtime_exports_every_declared_symbol():
 def test_registered_op_types():
     names = session.registered_kernels()
     for op in ["Conv", "MaxPool", "AveragePool", "GlobalAveragePool", "Concat", "Decoder", "Const",
-               "Constant", "Transpose", "Reshape"]:
+               "Constant", "Transpose", "Reshape", "Shape", "Gather", "Unsqueeze", "Add", "Relu", "Clip",
+               "BatchNormalization", "Gemm", "Flatten"]:
         assert op in names
 
 
