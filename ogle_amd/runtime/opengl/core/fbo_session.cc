@@ -232,7 +232,7 @@ void FBOSession::BuildSchedule() {
 
   // cost model: microseconds at a sustained MFMA rate, with a floor per launch
   constexpr double kMacPerUs = 45e6;  // ~90 TFLOP/s
-  constexpr double kFloorUs = 8.0;
+  constexpr double kFloorUs = 16.0;  // a dependent launch plus its split-K reduction
   std::vector<double> load(groups, 0.0);
   std::vector<int> members(groups, 0);
   for (int i = 0; i < n; ++i)
