@@ -74,6 +74,103 @@ __global__ __launch_bounds__(256) void pool_kernel(const T* __restrict__ x, T* _
   }
 }
 
+// Unsigned division by a number fixed at launch, exact below 2^31.
+struct PoolDiv {
+  unsigned mul, shift, d;
+};
+__device__ __forceinline__ unsigned pool_div(unsigned n, const PoolDiv& f) {
+  return (__umulhi(n, f.mul) + n) >> f.shift;
+}
+PoolDiv make_pool_div(unsigned d) {
+  PoolDiv f{0, 0, d};
+  unsigned l = 0;
+  while ((1ull << l) < d) ++l;
+  f.shift = l;
+  f.mul = (unsigned)(((1ull << 32) * ((1ull << l) - d)) / d + 1);
+  return f;
+}
+
+// Small windows (K = 2, 3), fp32, channel count a multiple of 4: one thread per
+// 16-byte channel vector of one output pixel; the K*K taps are branch-free buffer
+// loads, all in flight before the first comparison (a tap outside the image gets an
+// out-of-range offset; its lanes are then masked out of the maximum, or add the zeros
+// they read to the average).  Same results as pool_kernel.
+template <int K>
+__global__ __launch_bounds__(256) void pool_small_kernel(
+    const float* __restrict__ x, float* __restrict__ y, int h, int wd, int c, int oh, int ow,
+    int stride, int pad, int pool_type, unsigned total, unsigned x_bytes, unsigned y_bytes,
+    PoolDiv div_cv, PoolDiv div_ow, PoolDiv div_oh) {
+  typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+  constexpr unsigned kOut = 0x80000000u;
+  const unsigned idx = blockIdx.x * 256u + threadIdx.x;
+  if (idx >= total) return;
+  const unsigned t1 = pool_div(idx, div_cv);
+  const unsigned cg = idx - t1 * div_cv.d;
+  const unsigned t2 = pool_div(t1, div_ow);
+  const int ox = (int)(t1 - t2 * div_ow.d);
+  const unsigned b = pool_div(t2, div_oh);
+  const int oy = (int)(t2 - b * div_oh.d);
+  const __amdgpu_buffer_rsrc_t rx =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(x), 0, (int)x_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t ry = __builtin_amdgcn_make_buffer_rsrc(y, 0, (int)y_bytes, 0x00020000);
+  const unsigned row_bytes = (unsigned)(wd * c) * 4u;
+  const unsigned img = b * (unsigned)h * row_bytes + cg * 16u;
+  unsigned row_off[K], col_off[K];
+#pragma unroll
+  for (int j = 0; j < K; ++j) {
+    const int iy = oy * stride + j - pad;
+    row_off[j] = (unsigned)iy < (unsigned)h ? img + (unsigned)iy * row_bytes : kOut;
+    const int ix = ox * stride + j - pad;
+    col_off[j] = (unsigned)ix < (unsigned)wd ? (unsigned)(ix * c) * 4u : kOut;
+  }
+  u32x4 raw[K][K];  // [kx][ky], the shader's tap order
+#pragma unroll
+  for (int i = 0; i < K; ++i)
+#pragma unroll
+    for (int j = 0; j < K; ++j) {
+      const unsigned off = (row_off[j] + col_off[i]) | ((row_off[j] | col_off[i]) & kOut);
+      raw[i][j] = __builtin_amdgcn_raw_buffer_load_b128(rx, (int)off, 0, 0);
+    }
+  float v[4] = {0.f, 0.f, 0.f, 0.f};
+  if (pool_type == OGLE_POOL_MAX) {
+    bool any = false;
+#pragma unroll
+    for (int i = 0; i < K; ++i)
+#pragma unroll
+      for (int j = 0; j < K; ++j) {
+        const bool ok = ((row_off[j] | col_off[i]) & kOut) == 0;
+        const float item[4] = {__uint_as_float(raw[i][j].x), __uint_as_float(raw[i][j].y),
+                               __uint_as_float(raw[i][j].z), __uint_as_float(raw[i][j].w)};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          // the first in-image tap initialises, later ones take the maximum (pool.glsl:48-55)
+          const float m = v[q] > item[q] ? v[q] : item[q];
+          v[q] = ok ? (any ? m : item[q]) : v[q];
+        }
+        any = any || ok;
+      }
+  } else {
+#pragma unroll
+    for (int i = 0; i < K; ++i)
+#pragma unroll
+      for (int j = 0; j < K; ++j) {
+        v[0] += __uint_as_float(raw[i][j].x);
+        v[1] += __uint_as_float(raw[i][j].y);
+        v[2] += __uint_as_float(raw[i][j].z);
+        v[3] += __uint_as_float(raw[i][j].w);
+      }
+    const float denom = (float)(K * K);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) v[q] = v[q] / denom;
+  }
+  u32x4 out;
+  out.x = __float_as_uint(v[0]); out.y = __float_as_uint(v[1]);
+  out.z = __float_as_uint(v[2]); out.w = __float_as_uint(v[3]);
+  const unsigned off = ((b * (unsigned)oh + (unsigned)oy) * (unsigned)ow + (unsigned)ox) *
+                           (unsigned)c * 4u + cg * 16u;
+  __builtin_amdgcn_raw_buffer_store_b128(out, ry, (int)off, 0, 0);
+}
+
 // Global average pooling with large windows: one workgroup per (image, 64
 // channel slab): lanes stride over pixels, partial sums reduced through LDS.
 // The summation order differs from the shader's sequential one; the result
@@ -201,6 +298,23 @@ int32_t run_pool(const OglePoolArgs& a, hipStream_t s) {
     hipLaunchKernelGGL((global_avg_kernel<T>), dim3((a.c + 63) / 64, a.n), dim3(256), 0, s, x, y,
                        a.in_h * a.in_w, a.c);
     return check_launch("global_avg_kernel");
+  }
+  if constexpr (sizeof(T) == 4) {
+    const long total4 = (long)a.n * a.out_h * a.out_w * (a.c / 4);
+    const long x_bytes = (long)a.n * a.in_h * a.in_w * a.c * 4, y_bytes = total4 * 16;
+    if (a.c % 4 == 0 && (a.kernel_size == 2 || a.kernel_size == 3) && total4 < 0x7fffffffL &&
+        x_bytes < 0x7fffffffL && y_bytes < 0x7fffffffL && total4 > 0) {
+      const dim3 grid((unsigned)((total4 + 255) / 256));
+#define OGLE_POOL_SMALL(K)                                                                        \
+  hipLaunchKernelGGL((pool_small_kernel<K>), grid, dim3(256), 0, s, x, y, a.in_h, a.in_w, a.c,    \
+                     a.out_h, a.out_w, a.stride, a.padding, a.pool_type, (unsigned)total4,        \
+                     (unsigned)x_bytes, (unsigned)y_bytes, make_pool_div((unsigned)(a.c / 4)),    \
+                     make_pool_div((unsigned)a.out_w), make_pool_div((unsigned)a.out_h))
+      if (a.kernel_size == 2) OGLE_POOL_SMALL(2);
+      else OGLE_POOL_SMALL(3);
+#undef OGLE_POOL_SMALL
+      return check_launch("pool_small_kernel");
+    }
   }
   if (a.c % 4 == 0) {
     const long total = (long)a.n * a.out_h * a.out_w * (a.c / 4);
