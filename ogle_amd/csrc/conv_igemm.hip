@@ -293,12 +293,12 @@ __device__ __forceinline__ void igemm_tile(
   // contiguous row segments with 16-byte stores; bias and activation are applied
   // on the way out.  Otherwise each lane stores its elements one by one.
   float* const pdst = partial != nullptr ? partial + (long)split * g.m_total * g.o : nullptr;
+  constexpr int SROW = WTN + 4;            // floats per staged row (padded)
+  static_assert(4 * 32 * SROW * 4 <= 2 * STAGE, "epilogue staging exceeds the K-loop LDS");
+  float* const smw = reinterpret_cast<float*>(lds) + wave * 32 * SROW;
   if ((g.o & 3) == 0 && (sizeof(T) == 4 || pdst != nullptr)) {
-    constexpr int SROW = WTN + 4;            // floats per staged row (padded)
     constexpr int LPR = WTN / 4;             // lanes covering one staged row
     constexpr int RPI = 64 / LPR;            // rows one store instruction covers
-    static_assert(4 * 32 * SROW * 4 <= 2 * STAGE, "epilogue staging exceeds the K-loop LDS");
-    float* smw = reinterpret_cast<float*>(lds) + wave * 32 * SROW;
     const int cv = lane % LPR;
     const int rsub = lane / LPR;
     const int col = n0 + wave_n * WTN + cv * 4;
@@ -331,6 +331,52 @@ __device__ __forceinline__ void igemm_tile(
       }
     }
     return;
+  }
+  if constexpr (sizeof(T) == 2) {
+    if ((g.o & 7) == 0) {
+      // fp16 output: the same staging, a lane then takes eight consecutive channels
+      // of a row and stores them as one 16-byte vector of halves
+      constexpr int LPR = WTN / 8;
+      constexpr int RPI = 64 / LPR;
+      const int cv = lane % LPR;
+      const int rsub = lane / LPR;
+      const int col = n0 + wave_n * WTN + cv * 8;
+      float bias8[8];
+#pragma unroll
+      for (int q = 0; q < 8; ++q) bias8[q] = 0.f;
+      if (bias != nullptr && col < g.o) {
+        const float4 b0 = *reinterpret_cast<const float4*>(bias + col);
+        const float4 b1 = *reinterpret_cast<const float4*>(bias + col + 4);
+        bias8[0] = b0.x; bias8[1] = b0.y; bias8[2] = b0.z; bias8[3] = b0.w;
+        bias8[4] = b1.x; bias8[5] = b1.y; bias8[6] = b1.z; bias8[7] = b1.w;
+      }
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            smw[((r >> 2) * 8 + lh * 4 + (r & 3)) * SROW + j * 32 + l32] = acc[i][j][r];
+#pragma unroll
+        for (int it = 0; it < 32 / RPI; ++it) {
+          const int row = it * RPI + rsub;
+          const float4 v0 = *reinterpret_cast<const float4*>(smw + row * SROW + cv * 8);
+          const float4 v1 = *reinterpret_cast<const float4*>(smw + row * SROW + cv * 8 + 4);
+          const int grow = m0 + wave_m * WTM + i * 32 + row;
+          if (grow < g.m_total && col < g.o) {
+            const float f[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+            uint4 packed;
+            __half2* h = reinterpret_cast<__half2*>(&packed);
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+              h[q] = __floats2half2_rn(apply_epilogue(f[2 * q] + bias8[2 * q], ep),
+                                       apply_epilogue(f[2 * q + 1] + bias8[2 * q + 1], ep));
+            *reinterpret_cast<uint4*>(reinterpret_cast<__half*>(y) + (long)grow * g.o + col) = packed;
+          }
+        }
+      }
+      return;
+    }
   }
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
@@ -524,9 +570,13 @@ IgemmPlan plan_igemm(const OgleConvArgs& a, long m, bool allow_split) {
   // the larger tiles on every layer of the network because they quantise better
   // over 256 CUs and hide latency with occupancy; 128x128 only pays off once there
   // are enough tiles for several rounds.
+  // fp16 storage: an MFMA does sixteen times the work per operand byte, so the
+  // 64x64 tile is bound by LDS traffic and instruction issue; 128x128 pays off as soon
+  // as its tiles cover the compute units.
+  const long big_tiles_wanted = a.dtype == OGLE_F16 ? kComputeUnits : 4 * kComputeUnits;
   if (a.out_c <= 32) {
     p.cfg = CFG_128x32;
-  } else if (a.out_c > 64 && tiles(CFG_128x128) >= 4 * kComputeUnits) {
+  } else if (a.out_c > 64 && tiles(CFG_128x128) >= big_tiles_wanted) {
     p.cfg = CFG_128x128;
   } else {
     p.cfg = CFG_64x64;
