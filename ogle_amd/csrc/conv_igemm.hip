@@ -411,7 +411,7 @@ struct IgemmProblem {
   int tiles_n, tiles;
   float* partial;
   int slabs_per_split, splits;
-  int variant;  // mixed-group kernel only: 2 * (tile is 128x32) + (pointwise)
+  int variant;  // mixed-group kernel only: 2 * (tile is 128x32) + (pointwise); 4..7: wave-split 32 / 16
 };
 
 template <typename T, int BM, int BN, int WM, int WN, int ROWB, bool PW>
@@ -446,6 +446,11 @@ __global__ __launch_bounds__(256) void conv_igemm_group_kernel(IgemmGroup grp) {
                                           (int)blockIdx.x - grp.first[i]);
 }
 
+template <typename T, bool PW, int TS, int U>
+__device__ __forceinline__ void igemm_wave_tile(
+    float* __restrict__ red, const ConvGeom& g, const T* __restrict__ x, const T* __restrict__ w,
+    const float* __restrict__ bias, T* __restrict__ y, const Epilogue& ep, int tiles_n, int bid);
+
 // A group whose members differ in tile shape (64x64 or 128x32) or in being
 // pointwise: each workgroup takes the code path of its own problem.  The branch is
 // uniform over the workgroup; all four paths keep 16 accumulator registers per
@@ -471,10 +476,238 @@ __global__ __launch_bounds__(256) void conv_igemm_mixed_kernel(IgemmGroup grp) {
     OGLE_MIXED_CASE(0, 64, 64, 2, 2, false)
     OGLE_MIXED_CASE(1, 64, 64, 2, 2, true)
     OGLE_MIXED_CASE(2, 128, 32, 4, 1, false)
+    OGLE_MIXED_CASE(3, 128, 32, 4, 1, true)
+#define OGLE_MIXED_WAVE(V, PW, TS)                                                               \
+  case V:                                                                                       \
+    /* two steps in flight only: the group kernel's register budget is the 64x64 tile's */      \
+    igemm_wave_tile<T, PW, TS, 2>(reinterpret_cast<float*>(lds), p.g, static_cast<const T*>(p.x), \
+                               static_cast<const T*>(p.w), p.bias, static_cast<T*>(p.y), p.ep,   \
+                               p.tiles_n, bid);                                                 \
+    break;
+    OGLE_MIXED_WAVE(4, false, 32)
+    OGLE_MIXED_WAVE(5, true, 32)
+    OGLE_MIXED_WAVE(6, false, 16)
     default:
-      OGLE_MIXED_CASE(3, 128, 32, 4, 1, true)
+      OGLE_MIXED_WAVE(7, true, 16)
+#undef OGLE_MIXED_WAVE
   }
 #undef OGLE_MIXED_CASE
+}
+
+// ---------------------------------------------------------------------------
+// Small problems: few output tiles, long contraction (the 1x1 ... 19x19 feature
+// maps at batch 1, the extras chain, the SSD heads).  Splitting K across workgroups
+// needs a second launch to add the parts, and a dependent launch costs more than
+// these convolutions themselves.  Here the split stays inside the workgroup: a
+// workgroup owns one 32x32 (or 16x16) output tile, its four waves each contract a quarter of K,
+// and the four partial tiles are added through LDS in wave order (a fixed order, so
+// the result does not depend on timing).  A wave feeds its MFMAs straight from
+// global memory: both operands are K-contiguous, so the 16 bytes a lane loads are
+// exactly its share of an MFMA operand (fp32: four k of an 8-wide group, fp16: eight
+// k of a 16-wide one); no LDS and no barrier in the K loop, and one wave per SIMD
+// can keep its MFMA pipe busy because consecutive MFMAs into one accumulator issue
+// back to back.  Operands are re-read by every tile that shares them, which the L2
+// absorbs at these sizes.
+typedef float floatx4v __attribute__((ext_vector_type(4)));
+
+// MFMA step of the wave-split kernel for a TS x TS tile.  `a` / `b` are the 16 bytes
+// the lane loaded; lanes are grouped by q = lane / TS.
+//   TS 32: q in {0,1};   fp32 4 x 32x32x2 (k = 4q + s), fp16 1 x 32x32x16 (k = 8q..)
+//   TS 16: q in {0..3};  fp32 4 x 16x16x4 (k = 4q + s), fp16 1 x 16x16x32 (k = 8q..)
+template <typename T, int TS>
+struct WaveMma;
+template <>
+struct WaveMma<float, 32> {
+  typedef floatx16 Acc;
+  static constexpr int REGS = 16;
+  __device__ static __forceinline__ void run(const u32x4& a, const u32x4& b, Acc& acc) {
+#pragma unroll
+    for (int s = 0; s < 4; ++s)
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a[s]), __uint_as_float(b[s]), acc, 0, 0, 0);
+  }
+};
+template <>
+struct WaveMma<__half, 32> {
+  typedef floatx16 Acc;
+  static constexpr int REGS = 16;
+  __device__ static __forceinline__ void run(const u32x4& a, const u32x4& b, Acc& acc) {
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(halfx8, a),
+                                                 __builtin_bit_cast(halfx8, b), acc, 0, 0, 0);
+  }
+};
+template <>
+struct WaveMma<float, 16> {
+  typedef floatx4v Acc;
+  static constexpr int REGS = 4;
+  __device__ static __forceinline__ void run(const u32x4& a, const u32x4& b, Acc& acc) {
+#pragma unroll
+    for (int s = 0; s < 4; ++s)
+      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(a[s]), __uint_as_float(b[s]), acc, 0, 0, 0);
+  }
+};
+template <>
+struct WaveMma<__half, 16> {
+  typedef floatx4v Acc;
+  static constexpr int REGS = 4;
+  __device__ static __forceinline__ void run(const u32x4& a, const u32x4& b, Acc& acc) {
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(halfx8, a),
+                                                 __builtin_bit_cast(halfx8, b), acc, 0, 0, 0);
+  }
+};
+
+constexpr int kWaveRedBytes = 4 * 32 * 36 * 4;  // four staged 32x32 partial tiles, padded rows
+
+// U: steps of loads in flight per register set (two sets).
+template <typename T, bool PW, int TS, int U>
+__device__ __forceinline__ void igemm_wave_tile(
+    float* __restrict__ red, const ConvGeom& g, const T* __restrict__ x, const T* __restrict__ w,
+    const float* __restrict__ bias, T* __restrict__ y, const Epilogue& ep, int tiles_n, int bid) {
+  typedef WaveMma<T, TS> M;
+  constexpr int ESZ = (int)sizeof(T);
+  constexpr int VE = 16 / ESZ;          // elements per 16-byte load
+  constexpr int QN = 64 / TS;           // lane groups along k
+  constexpr int KSTEP = QN * VE;        // k covered by one step
+  constexpr int PITCH = TS + 4;         // floats per row of a staged partial tile
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int lt = lane % TS, lq = lane / TS;
+  const int tile_n = bid % tiles_n, tile_m = bid / tiles_n;
+  const int m = tile_m * TS + lt;       // this lane's A row
+  const int col = tile_n * TS + lt;     // this lane's B row (output channel)
+  const __amdgpu_buffer_rsrc_t rx = make_rsrc(x, g.x_bytes);
+  const __amdgpu_buffer_rsrc_t rw = make_rsrc(w, g.w_bytes);
+
+  const int csteps = (g.c + KSTEP - 1) / KSTEP;   // steps per tap
+  const int steps = g.k * g.k * csteps;
+  const int s_begin = (int)(((long)steps * wave) / 4), s_end = (int)(((long)steps * (wave + 1)) / 4);
+
+  // row geometry of this lane
+  int iy0 = 0, ix0 = 0;
+  unsigned img = 0;
+  const bool row_ok = m < g.m_total;
+  if (PW) {
+    img = (unsigned)m * (unsigned)(g.c * ESZ);
+  } else {
+    const int ox = m % g.ow;
+    const int t = m / g.ow;
+    const int oy = t % g.oh;
+    const int b = t / g.oh;
+    img = (unsigned)b * (unsigned)(g.h * g.w * g.c * ESZ);
+    iy0 = oy * g.stride - g.pad;
+    ix0 = ox * g.stride - g.pad;
+  }
+  const unsigned wrow = (unsigned)col * (unsigned)(g.k * g.k * g.c * ESZ);
+  const bool col_ok = col < g.o;
+
+  // load cursor: (tap, channel step) of the next step to request
+  int l_tap = s_begin / csteps, l_cs = s_begin - l_tap * csteps;
+  unsigned a_tap = kOutOfRange, b_tap = kOutOfRange;
+  auto enter_tap = [&](int tap) {
+    if (PW) {
+      a_tap = row_ok ? img : kOutOfRange;
+    } else {
+      const int ky = tap / g.k, kx = tap - ky * g.k;
+      const int iy = iy0 + ky * g.dil, ix = ix0 + kx * g.dil;
+      const bool in = row_ok && iy >= 0 && iy < g.h && ix >= 0 && ix < g.w;
+      a_tap = in ? img + (unsigned)((iy * g.w + ix) * g.c * ESZ) : kOutOfRange;
+    }
+    b_tap = col_ok ? wrow + (unsigned)(tap * g.c * ESZ) : kOutOfRange;
+  };
+  enter_tap(l_tap);
+
+  u32x4 ra[2][U], rb[2][U];
+  int requested = s_begin;
+#define OGLE_WAVE_LOAD(SET)                                                                      \
+  _Pragma("unroll") for (int u = 0; u < U; ++u) {                                                \
+    const int cel = l_cs * KSTEP + lq * VE;                                                      \
+    const bool ok = requested < s_end && cel < g.c;                                              \
+    const unsigned ao = ok && a_tap != kOutOfRange ? a_tap + (unsigned)(cel * ESZ) : kOutOfRange; \
+    const unsigned bo = ok && b_tap != kOutOfRange ? b_tap + (unsigned)(cel * ESZ) : kOutOfRange; \
+    ra[SET][u] = __builtin_amdgcn_raw_buffer_load_b128(rx, (int)ao, 0, 0);                       \
+    rb[SET][u] = __builtin_amdgcn_raw_buffer_load_b128(rw, (int)bo, 0, 0);                       \
+    ++requested;                                                                                 \
+    if (++l_cs == csteps) {                                                                      \
+      l_cs = 0;                                                                                  \
+      ++l_tap;                                                                                   \
+      enter_tap(l_tap);                                                                          \
+    }                                                                                            \
+  }
+#define OGLE_WAVE_MMA(SET) \
+  _Pragma("unroll") for (int u = 0; u < U; ++u) M::run(ra[SET][u], rb[SET][u], acc);
+
+  typename M::Acc acc;
+#pragma unroll
+  for (int r = 0; r < M::REGS; ++r) acc[r] = 0.f;
+
+  // chunks of U steps, two register sets: the next chunk is in flight while the
+  // current one is multiplied; steps past s_end load zeros
+  // (the scheduling barriers keep a whole chunk of loads ahead of the MFMAs that
+  // consume the previous one; left alone the compiler sinks the loads next to their
+  // uses and the wave then waits for memory once per step)
+  OGLE_WAVE_LOAD(0);
+  for (int s = s_begin; s < s_end; s += 2 * U) {
+    OGLE_WAVE_LOAD(1);
+    __builtin_amdgcn_sched_barrier(0);
+    OGLE_WAVE_MMA(0);
+    __builtin_amdgcn_sched_barrier(0);
+    OGLE_WAVE_LOAD(0);
+    __builtin_amdgcn_sched_barrier(0);
+    OGLE_WAVE_MMA(1);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+#undef OGLE_WAVE_LOAD
+#undef OGLE_WAVE_MMA
+
+  // the four partial tiles, then their sum in wave order.  Result layout: register r
+  // of lane l is row 8*(r/4) + 4*(l/32) + r%4 (32x32) or 4*(l/16) + r (16x16), column l % TS.
+  float* mine = red + wave * (TS * PITCH);
+#pragma unroll
+  for (int r = 0; r < M::REGS; ++r) {
+    const int row = TS == 32 ? (r >> 2) * 8 + lq * 4 + (r & 3) : lq * 4 + r;
+    mine[row * PITCH + lt] = acc[r];
+  }
+  __syncthreads();
+  constexpr int VPR = TS / 4;             // 4-element groups per row
+  if (tid >= TS * VPR) return;            // TS 16: 64 threads finish the tile
+  const int orow = tid / VPR, ocol = (tid % VPR) * 4;
+  const float* p0 = red + orow * PITCH + ocol;
+  float4 sum = *reinterpret_cast<const float4*>(p0);
+#pragma unroll
+  for (int wv = 1; wv < 4; ++wv) {
+    const float4 t = *reinterpret_cast<const float4*>(p0 + wv * (TS * PITCH));
+    sum.x += t.x; sum.y += t.y; sum.z += t.z; sum.w += t.w;
+  }
+  const int grow = tile_m * TS + orow;
+  const int gcol = tile_n * TS + ocol;
+  if (grow >= g.m_total || gcol >= g.o) return;
+  float v[4] = {sum.x, sum.y, sum.z, sum.w};
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    if (gcol + q < g.o) v[q] = apply_epilogue(v[q] + (bias != nullptr ? bias[gcol + q] : 0.f), ep);
+  }
+  T* dst = y + (long)grow * g.o + gcol;
+  if ((g.o & 3) == 0) {
+    if constexpr (sizeof(T) == 4) {
+      *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+    } else {
+      const __half2 lo = __floats2half2_rn(v[0], v[1]), hi = __floats2half2_rn(v[2], v[3]);
+      uint2 packed;
+      packed.x = *reinterpret_cast<const unsigned*>(&lo);
+      packed.y = *reinterpret_cast<const unsigned*>(&hi);
+      *reinterpret_cast<uint2*>(dst) = packed;
+    }
+  } else {
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      if (gcol + q < g.o) dst[q] = from_f32<T>(v[q]);
+  }
+}
+
+template <typename T, bool PW, int TS>
+__global__ __launch_bounds__(256) void conv_igemm_wave_kernel(IgemmProblem p) {
+  __shared__ __attribute__((aligned(16))) float red[kWaveRedBytes / 4];
+  igemm_wave_tile<T, PW, TS, 4>(red, p.g, static_cast<const T*>(p.x), static_cast<const T*>(p.w),
+                             p.bias, static_cast<T*>(p.y), p.ep, p.tiles_n, (int)blockIdx.x);
 }
 
 struct ReduceProblem {
@@ -537,9 +770,11 @@ __global__ __launch_bounds__(256) void splitk_reduce_group_kernel(ReduceGroup gr
 }
 
 // Tile configurations (BM, BN, waves along M, waves along N).
-enum TileCfg { CFG_128x128 = 0, CFG_128x64 = 1, CFG_64x64 = 2, CFG_128x32 = 3 };
-constexpr int kCfgBM[] = {128, 128, 64, 128};
-constexpr int kCfgBN[] = {128, 64, 64, 32};
+enum TileCfg {
+  CFG_128x128 = 0, CFG_128x64 = 1, CFG_64x64 = 2, CFG_128x32 = 3, CFG_WAVE32 = 4, CFG_WAVE16 = 5
+};
+constexpr int kCfgBM[] = {128, 128, 64, 128, 32, 16};
+constexpr int kCfgBN[] = {128, 64, 64, 32, 32, 16};
 
 struct IgemmPlan {
   int cfg;
@@ -604,6 +839,25 @@ IgemmPlan plan_igemm(const OgleConvArgs& a, long m, bool allow_split) {
   else if (sp >= 4) sp = 4;
   else if (sp >= 2) sp = 2;
   if (sp >= 2) p.splits = (int)sp;
+  // A small contraction that would be split across workgroups goes to the wave-split
+  // kernel instead (the split stays inside the workgroup: no workspace, no second
+  // launch), whether or not a workspace was offered.  Measured on MI355X against
+  // split-K + reduce: the 32x32 form wins for K <= 512 once its tiles cover half the
+  // chip, the 16x16 form for K <= 1536 on the very small maps; a longer K per wave is
+  // a serial chain of MFMAs and loses to the split across workgroups.
+  {
+    const long k_total = (long)a.kernel_size * a.kernel_size * a.in_c;
+    const bool would_split = (2 * t <= kComputeUnits && p.ktiles >= 8) ||
+                             (t < 8 * kComputeUnits && p.ktiles >= 128);
+    const long t32 = tiles(CFG_WAVE32), t16 = tiles(CFG_WAVE16);
+    if (would_split && k_total <= 512 && t32 >= kComputeUnits / 2 && t32 <= 4 * kComputeUnits) {
+      p.cfg = CFG_WAVE32;
+      p.splits = 1;
+    } else if (would_split && k_total <= 1536 && t16 <= kComputeUnits / 2) {
+      p.cfg = CFG_WAVE16;
+      p.splits = 1;
+    }
+  }
   p.slabs_per_split = (p.ktiles + p.splits - 1) / p.splits;
   if (p.splits > 1) p.slabs_per_split += p.slabs_per_split & 1;  // the K loop runs slab pairs
   // (a split past the end of K would only add zeros; rounding splits down keeps the
@@ -612,6 +866,7 @@ IgemmPlan plan_igemm(const OgleConvArgs& a, long m, bool allow_split) {
   return p;
 }
 
+bool is_wave(int cfg) { return cfg == CFG_WAVE32 || cfg == CFG_WAVE16; }
 int tile_bm(int cfg) { return kCfgBM[cfg]; }
 int tile_bn(int cfg) { return kCfgBN[cfg]; }
 
@@ -683,7 +938,12 @@ Prepared prepare(const OgleConvArgs& a, long m, const IgemmPlan& p) {
   out.prob.partial = p.splits > 1 ? static_cast<float*>(a.workspace_dev) : nullptr;
   out.prob.slabs_per_split = p.slabs_per_split;
   out.prob.splits = p.splits;
-  out.prob.variant = (p.cfg == CFG_128x32 ? 2 : 0) + (is_pointwise(a) ? 1 : 0);
+  out.prob.variant = (p.cfg == CFG_WAVE32 ? 4 : p.cfg == CFG_WAVE16 ? 6 : p.cfg == CFG_128x32 ? 2 : 0) +
+                     (is_pointwise(a) ? 1 : 0);
+  if (is_wave(p.cfg)) {
+    out.grid = (unsigned)(tiles_m * tiles_n);
+    return out;
+  }
   out.grid = grid_blocks(p, tiles_m, tiles_n);
   if (p.splits > 1) {
     const long mn = (long)g.m_total * g.o;
@@ -731,6 +991,25 @@ Prepared prepare(const OgleConvArgs& a, long m, const IgemmPlan& p) {
       break;                                                                                 \
   }
 
+void launch_wave(int dtype, bool pw, int cfg, const Prepared& pr, hipStream_t s) {
+  const dim3 grid(pr.grid), block(256);
+#define OGLE_WAVE_LAUNCH(T, PW, TS) \
+  hipLaunchKernelGGL((conv_igemm_wave_kernel<T, PW, TS>), grid, block, 0, s, pr.prob)
+#define OGLE_WAVE_PICK(T)                                                 \
+  if (cfg == CFG_WAVE32) {                                                \
+    if (pw) OGLE_WAVE_LAUNCH(T, true, 32); else OGLE_WAVE_LAUNCH(T, false, 32); \
+  } else {                                                                \
+    if (pw) OGLE_WAVE_LAUNCH(T, true, 16); else OGLE_WAVE_LAUNCH(T, false, 16); \
+  }
+  if (dtype == OGLE_F16) {
+    OGLE_WAVE_PICK(__half)
+  } else {
+    OGLE_WAVE_PICK(float)
+  }
+#undef OGLE_WAVE_PICK
+#undef OGLE_WAVE_LAUNCH
+}
+
 template <typename T>
 void launch_reduce_single(const Prepared& pr, hipStream_t s) {
   const dim3 grid(pr.reduce_grid), block(256);
@@ -756,6 +1035,10 @@ int32_t launch_conv_igemm(const OgleConvArgs& a, hipStream_t s) {
   const IgemmPlan p = final_plan(a, m);
   const Prepared pr = prepare(a, m, p);
   const bool pw = is_pointwise(a);
+  if (is_wave(p.cfg)) {
+    launch_wave(a.dtype, pw, p.cfg, pr, s);
+    return check_launch("conv_igemm_wave");
+  }
   OGLE_IGEMM_DISPATCH(conv_igemm_kernel, a.dtype, p.cfg, pw, pr.grid, s, pr.prob);
   int32_t st = check_launch("conv_igemm");
   if (st != OGLE_OK || p.splits == 1) return st;
@@ -788,7 +1071,9 @@ int32_t launch_conv_batch(const OgleConvArgs* args, int count, hipStream_t s,
     const IgemmPlan p = final_plan(args[i], m);
     items.push_back(Item{args[i].dtype, p.cfg, is_pointwise(args[i]), prepare(args[i], m, p)});
   }
-  auto mixable = [](const Item& it) { return it.cfg == CFG_64x64 || it.cfg == CFG_128x32; };
+  auto mixable = [](const Item& it) {
+    return it.cfg == CFG_64x64 || it.cfg == CFG_128x32 || is_wave(it.cfg);
+  };
   std::vector<bool> done(items.size(), false);
   for (size_t a0 = 0; a0 < items.size(); ++a0) {
     if (done[a0]) continue;
@@ -812,9 +1097,11 @@ int32_t launch_conv_batch(const OgleConvArgs* args, int count, hipStream_t s,
       }
     }
     const unsigned grid = (unsigned)grp.first[grp.count];
-    if (grp.count == 1) {
+    if (grp.count == 1 && is_wave(head.cfg)) {
+      launch_wave(head.dtype, head.pw, head.cfg, head.pr, s);
+    } else if (grp.count == 1) {
       OGLE_IGEMM_DISPATCH(conv_igemm_kernel, head.dtype, head.cfg, head.pw, grid, s, grp.p[0]);
-    } else if (uniform) {
+    } else if (uniform && !is_wave(head.cfg)) {
       OGLE_IGEMM_DISPATCH(conv_igemm_group_kernel, head.dtype, head.cfg, head.pw, grid, s, grp);
     } else if (head.dtype == OGLE_F16) {
       hipLaunchKernelGGL((conv_igemm_mixed_kernel<__half, 128>), dim3(grid), dim3(256), 0, s, grp);

@@ -130,8 +130,6 @@ def test_gemm(case):
     for workspace in (True, False):
         got, need = gpu_gemm(a, b, c, alpha, beta, trans_b, workspace)
         assert np.all(np.abs(got - ref) <= 1e-4 * scale + 1e-30), case
-    if m <= 16 and trans_b and k % 4 == 0 and k >= 512 and alpha == 1.0:
-        assert need > 0   # the small-M Linear form plans a split-K
 
 
 def test_eltwise_argument_checks():
