@@ -130,6 +130,42 @@ def test_conv_stem_kernel(case, dtype):
     check_conv(x, wt, b, s, p, d, 1, act=H.ACT_CLIP, maxv=6.0, dtype=dtype, what=str(case))
 
 
+WAVE_CASES = [
+    # n, h, w, c, o, k, s, p, d   small problems with a long enough K: the wave-split kernel
+    (1, 19, 19, 512, 512, 1, 1, 0, 1),    # 32x32 tiles, pointwise (a batch-1 MobileNet layer)
+    (1, 38, 38, 256, 250, 1, 1, 0, 1),    # 32x32 tiles, ragged N with 2-element tail
+    (2, 40, 40, 20, 64, 3, 1, 1, 1),      # 32x32 tiles, 3x3, C % 8 == 4 (half-filled last step)
+    (1, 45, 41, 36, 33, 3, 2, 1, 1),      # 32x32 tiles, stride 2, N not a multiple of 4
+    (1, 10, 10, 1024, 256, 1, 1, 0, 1),   # 16x16 tiles, pointwise
+    (1, 3, 3, 128, 256, 3, 2, 1, 1),      # 16x16 tiles, one output pixel per image
+    (3, 5, 5, 64, 21, 3, 1, 2, 2),        # 16x16 tiles, dilation 2, odd N
+    (1, 1, 1, 1024, 1000, 1, 1, 0, 1),    # 16x16 tiles, M = 1 (a classifier head)
+    (1, 7, 9, 128, 10, 3, 1, 1, 1),       # 16x16 tiles, fewer channels than a tile
+]
+
+
+@pytest.mark.parametrize("case", WAVE_CASES)
+@pytest.mark.parametrize("dtype", [H.F32, H.F16])
+def test_conv_wave_split_kernel(case, dtype):
+    n, h, w, c, o, k, s, p, d = case
+    r = rng(1700 + WAVE_CASES.index(case))
+    x = r.uniform(-1, 1, (n, h, w, c)).astype(np.float32)
+    wt = r.normal(0, 0.2, (o, c, k, k)).astype(np.float32)
+    b = r.uniform(-0.1, 0.1, o).astype(np.float32)
+    if dtype == H.F16:
+        if c % 8 != 0:
+            pytest.skip("fp16 storage needs C % 8 == 0 for the MFMA kernels")
+        x = x.astype(np.float16).astype(np.float32)
+        wt = wt.astype(np.float16).astype(np.float32)
+    variant = H.VARIANT_PW if (k == 1 and s == 1 and p == 0) else H.VARIANT_NHWC4
+    # with and without a workspace: the plan must not depend on it
+    for entry_ws in (True, False):
+        ref = O.conv2d(x, wt, b, s, p, d, 1, O.ACT_CLIP, 0.0, 6.0, variant)
+        scale = O.conv2d_abs(x, wt, b, s, p, d, 1)
+        got = gpu_conv(x, wt, b, s, p, d, 1, H.ACT_CLIP, 0.0, 6.0, variant, dtype, None, entry_ws)
+        assert_conv_close(got, ref, scale, FP16_RTOL if dtype == H.F16 else FP32_RTOL, str(case))
+
+
 def test_conv_shape_sweep_mfma_path():
     """Channel counts that take the implicit-GEMM kernel, ragged in every dimension."""
     r = rng(2100)
