@@ -570,10 +570,19 @@ __device__ __forceinline__ void igemm_wave_tile(
   constexpr int PITCH = TS + 4;         // floats per row of a staged partial tile
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
-  const int lt = lane % TS, lq = lane / TS;
+  // MFMA operand order: lane = q * TS + row.  Pointwise loads use the other order,
+  // lane = row * QN + q, so that the QN lanes of a row read one contiguous run (the
+  // vector cache takes one access per contiguous run, and one per lane otherwise, which
+  // is what bounds the pointwise problems); a lane permute puts the data into MFMA
+  // order.  The other problems sent here are tiny maps that wait on latency, not on the
+  // cache, and the permutes only lengthen their chain: they load in MFMA order.
+  const int mt = lane % TS, mq = lane / TS;        // MFMA order (also the result layout)
+  constexpr bool PERM = PW;
+  const int lt = PERM ? lane / QN : mt, lq = PERM ? lane % QN : mq;        // load order
+  const int permute_from = (mt * QN + mq) * 4;     // byte address for ds_bpermute
   const int tile_n = bid % tiles_n, tile_m = bid / tiles_n;
-  const int m = tile_m * TS + lt;       // this lane's A row
-  const int col = tile_n * TS + lt;     // this lane's B row (output channel)
+  const int m = tile_m * TS + lt;       // the A row this lane loads
+  const int col = tile_n * TS + lt;     // the B row (output channel) this lane loads
   const __amdgpu_buffer_rsrc_t rx = make_rsrc(x, g.x_bytes);
   const __amdgpu_buffer_rsrc_t rw = make_rsrc(w, g.w_bytes);
 
@@ -632,8 +641,15 @@ __device__ __forceinline__ void igemm_wave_tile(
       enter_tap(l_tap);                                                                          \
     }                                                                                            \
   }
-#define OGLE_WAVE_MMA(SET) \
-  _Pragma("unroll") for (int u = 0; u < U; ++u) M::run(ra[SET][u], rb[SET][u], acc);
+#define OGLE_WAVE_MMA(SET)                                                                       \
+  _Pragma("unroll") for (int u = 0; u < U; ++u) {                                                \
+    u32x4 av, bv;                                                                                \
+    _Pragma("unroll") for (int e = 0; e < 4; ++e) {                                              \
+      av[e] = PERM ? (unsigned)__builtin_amdgcn_ds_bpermute(permute_from, (int)ra[SET][u][e]) : ra[SET][u][e]; \
+      bv[e] = PERM ? (unsigned)__builtin_amdgcn_ds_bpermute(permute_from, (int)rb[SET][u][e]) : rb[SET][u][e]; \
+    }                                                                                            \
+    M::run(av, bv, acc);                                                                         \
+  }
 
   typename M::Acc acc;
 #pragma unroll
@@ -663,8 +679,8 @@ __device__ __forceinline__ void igemm_wave_tile(
   float* mine = red + wave * (TS * PITCH);
 #pragma unroll
   for (int r = 0; r < M::REGS; ++r) {
-    const int row = TS == 32 ? (r >> 2) * 8 + lq * 4 + (r & 3) : lq * 4 + r;
-    mine[row * PITCH + lt] = acc[r];
+    const int row = TS == 32 ? (r >> 2) * 8 + mq * 4 + (r & 3) : mq * 4 + r;
+    mine[row * PITCH + mt] = acc[r];
   }
   __syncthreads();
   constexpr int VPR = TS / 4;             // 4-element groups per row
@@ -788,6 +804,8 @@ struct IgemmPlan {
 constexpr long kComputeUnits = 256;
 constexpr int kRowBytesF32 = 64;   // bytes of K per tile row per slab, fp32
 
+bool is_pointwise(const OgleConvArgs& a);
+
 // Picks the output tile and the K split.  Problems with few output
 // tiles but a long contraction (the SSD heads, the small feature maps) are split
 // along K until the grid fills the chip, provided a workspace was supplied.
@@ -842,18 +860,24 @@ IgemmPlan plan_igemm(const OgleConvArgs& a, long m, bool allow_split) {
   // A small contraction that would be split across workgroups goes to the wave-split
   // kernel instead (the split stays inside the workgroup: no workspace, no second
   // launch), whether or not a workspace was offered.  Measured on MI355X against
-  // split-K + reduce: the 32x32 form wins for K <= 512 once its tiles cover half the
-  // chip, the 16x16 form for K <= 1536 on the very small maps; a longer K per wave is
-  // a serial chain of MFMAs and loses to the split across workgroups.
+  // split-K + reduce: the 32x32 form wins once its tiles cover half the chip, for
+  // K <= 1024 pointwise and K <= 512 otherwise; the 16x16 form wins for pointwise
+  // K <= 1024 while its tiles stay under two per compute unit, and for K <= 1536 on the
+  // very small maps; a longer K per wave is a serial chain of MFMAs and loses to the
+  // split across workgroups.
   {
     const long k_total = (long)a.kernel_size * a.kernel_size * a.in_c;
+    const bool pw = is_pointwise(a);
     const bool would_split = (2 * t <= kComputeUnits && p.ktiles >= 8) ||
                              (t < 8 * kComputeUnits && p.ktiles >= 128);
     const long t32 = tiles(CFG_WAVE32), t16 = tiles(CFG_WAVE16);
-    if (would_split && k_total <= 512 && t32 >= kComputeUnits / 2 && t32 <= 4 * kComputeUnits) {
+    const bool small16 = (pw && k_total <= 1024 && t16 <= 2 * kComputeUnits) ||
+                         (k_total <= 1536 && t16 <= kComputeUnits / 2);
+    if (would_split && !small16 && k_total <= (pw ? 1024 : 512) && t32 >= kComputeUnits / 2 &&
+        t32 <= 4 * kComputeUnits) {
       p.cfg = CFG_WAVE32;
       p.splits = 1;
-    } else if (would_split && k_total <= 1536 && t16 <= kComputeUnits / 2) {
+    } else if (would_split && small16) {
       p.cfg = CFG_WAVE16;
       p.splits = 1;
     }

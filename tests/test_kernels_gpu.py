@@ -141,6 +141,9 @@ WAVE_CASES = [
     (3, 5, 5, 64, 21, 3, 1, 2, 2),        # 16x16 tiles, dilation 2, odd N
     (1, 1, 1, 1024, 1000, 1, 1, 0, 1),    # 16x16 tiles, M = 1 (a classifier head)
     (1, 7, 9, 128, 10, 3, 1, 1, 1),       # 16x16 tiles, fewer channels than a tile
+    (1, 10, 10, 1024, 1024, 1, 1, 0, 1),  # 16x16 tiles, pointwise, two tiles per compute unit
+    (1, 9, 11, 504, 130, 1, 1, 0, 1),     # 16x16 tiles, pointwise, ragged M, N and last K step
+    (2, 10, 10, 1024, 1024, 1, 1, 0, 1),  # 32x32 tiles, pointwise, K = 1024
 ]
 
 
