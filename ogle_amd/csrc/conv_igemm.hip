@@ -184,28 +184,20 @@ __device__ __forceinline__ void igemm_tile(
   // being requested into the other, so a load has two slabs of MFMA work to land.
   u32x4 ra[2][AP], rb[2][BP];
 
-  // Issues the global loads of K slab `kt` into ra / rb (no waiting).
-#define OGLE_LOAD_SLAB(kt, SET)                                                                 \
+  // Issues the global loads of the next K slab into ra / rb (no waiting) and moves
+  // the load cursor on.  The cursor (slab number, its tap, channel chunk and tap
+  // offsets) advances by increments: slabs are requested strictly in order, so the
+  // two integer divisions that locate a slab are paid once, not per slab.
+#define OGLE_LOAD_SLAB(SET)                                                                  \
   {                                                                                          \
-    int tap_ = 0, cc_ = (kt);                                                                \
-    if (!PW) {                                                                               \
-      tap_ = (kt) / g.cchunks;                                                               \
-      cc_ = (kt) - tap_ * g.cchunks;                                                         \
-    }                                                                                        \
-    const int cbyte_ = cc_ * ROWB + vcol * 16;                                               \
-    const bool c_ok_ = cbyte_ < g.c * ESZ && (kt) < kt_end; /* past the end: zeros */       \
-    int dy_ = 0, dx_ = 0;                                                                    \
-    if (!PW) {                                                                               \
-      const int ky_ = tap_ / g.k;                                                            \
-      dy_ = ky_ * g.dil;                                                                     \
-      dx_ = (tap_ - ky_ * g.k) * g.dil;                                                      \
-    }                                                                                        \
+    const int cbyte_ = l_cc * ROWB + vcol * 16;                                              \
+    const bool c_ok_ = cbyte_ < g.c * ESZ && l_kt < kt_end; /* past the end: zeros */        \
     _Pragma("unroll") for (int p = 0; p < AP; ++p) {                                         \
       unsigned off_;                                                                         \
       if (PW) {                                                                              \
         off_ = c_ok_ ? a_base[p] + (unsigned)cbyte_ : kOutOfRange;                           \
       } else {                                                                               \
-        const int iy_ = a_iy[p] + dy_, ix_ = a_ix[p] + dx_;                                  \
+        const int iy_ = a_iy[p] + l_dy, ix_ = a_ix[p] + l_dx;                                \
         const bool in_ = c_ok_ && iy_ >= 0 && iy_ < g.h && ix_ >= 0 && ix_ < g.w;            \
         off_ = in_ ? a_base[p] + (unsigned)((iy_ * g.w + ix_) * g.c * ESZ + cbyte_)          \
                    : kOutOfRange;                                                            \
@@ -213,9 +205,19 @@ __device__ __forceinline__ void igemm_tile(
       ra[SET][p] = __builtin_amdgcn_raw_buffer_load_b128(rx, (int)off_, 0, 0);               \
     }                                                                                        \
     _Pragma("unroll") for (int p = 0; p < BP; ++p) {                                         \
-      const unsigned off_ =                                                                  \
-          c_ok_ ? b_base[p] + (unsigned)(tap_ * g.c * ESZ + cbyte_) : kOutOfRange;           \
+      const unsigned off_ = c_ok_ ? b_base[p] + l_tapbyte + (unsigned)cbyte_ : kOutOfRange;  \
       rb[SET][p] = __builtin_amdgcn_raw_buffer_load_b128(rw, (int)off_, 0, 0);               \
+    }                                                                                        \
+    ++l_kt;                                                                                  \
+    if (++l_cc == g.cchunks) {                                                               \
+      l_cc = 0;                                                                              \
+      l_tapbyte += (unsigned)(g.c * ESZ);                                                    \
+      l_dx += g.dil;                                                                         \
+      if (++l_kx == g.k) {                                                                   \
+        l_kx = 0;                                                                            \
+        l_dx = 0;                                                                            \
+        l_dy += g.dil;                                                                       \
+      }                                                                                      \
     }                                                                                        \
   }
 
@@ -263,22 +265,35 @@ __device__ __forceinline__ void igemm_tile(
     }                                                                                        \
   }
 
+  // The load cursor starts at slab kt_begin.
+  int l_kt = kt_begin, l_cc = kt_begin, l_kx = 0, l_dy = 0, l_dx = 0;
+  unsigned l_tapbyte = 0;
+  if (!PW) {
+    const int tap = kt_begin / g.cchunks;
+    const int ky = tap / g.k;
+    l_cc = kt_begin - tap * g.cchunks;
+    l_kx = tap - ky * g.k;
+    l_dy = ky * g.dil;
+    l_dx = l_kx * g.dil;
+    l_tapbyte = (unsigned)(tap * g.c * ESZ);
+  }
+
   // Software pipeline, unrolled by two so that the register sets and LDS buffers
   // are compile-time: while slab kt is multiplied out of one LDS buffer, slab kt+1
   // (requested one step earlier) is moved from its registers into the other buffer
   // and slab kt+2 is requested.  Requests past kt_end return zeros and are dropped.
-  OGLE_LOAD_SLAB(kt_begin, 0);
-  OGLE_LOAD_SLAB(kt_begin + 1, 1);
+  OGLE_LOAD_SLAB(0);
+  OGLE_LOAD_SLAB(1);
   OGLE_STORE_SLAB(0, 0);
   __syncthreads();
   for (int kt = kt_begin; kt < kt_end; kt += 2) {
     // An odd slab count runs one extra all-zero slab through the second half: a
     // loop without early exits keeps the accumulators in one set of registers.
-    OGLE_LOAD_SLAB(kt + 2, 0);
+    OGLE_LOAD_SLAB(0);
     OGLE_COMPUTE_SLAB(0);
     OGLE_STORE_SLAB(1, 1);
     __syncthreads();
-    OGLE_LOAD_SLAB(kt + 3, 1);
+    OGLE_LOAD_SLAB(1);
     OGLE_COMPUTE_SLAB(1);
     OGLE_STORE_SLAB(0, 0);
     __syncthreads();
@@ -570,14 +585,15 @@ __device__ __forceinline__ void igemm_wave_tile(
   constexpr int PITCH = TS + 4;         // floats per row of a staged partial tile
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
-  // MFMA operand order: lane = q * TS + row.  Pointwise loads use the other order,
-  // lane = row * QN + q, so that the QN lanes of a row read one contiguous run (the
-  // vector cache takes one access per contiguous run, and one per lane otherwise, which
-  // is what bounds the pointwise problems); a lane permute puts the data into MFMA
-  // order.  The other problems sent here are tiny maps that wait on latency, not on the
-  // cache, and the permutes only lengthen their chain: they load in MFMA order.
+  // MFMA operand order: lane = q * TS + row.  Loads use the other order, lane =
+  // row * QN + q, so that the QN lanes of a row read one contiguous run (the vector
+  // cache takes one access per contiguous run, and one per lane otherwise, which is
+  // what bounds these problems); a lane permute puts the data into MFMA order.  The
+  // 16x16 form of a non-pointwise problem is only chosen for tiny maps that wait on
+  // latency, not on the cache, and the permutes only lengthen their chain: those load
+  // in MFMA order.
   const int mt = lane % TS, mq = lane / TS;        // MFMA order (also the result layout)
-  constexpr bool PERM = PW;
+  constexpr bool PERM = PW || TS == 32;
   const int lt = PERM ? lane / QN : mt, lq = PERM ? lane % QN : mq;        // load order
   const int permute_from = (mt * QN + mq) * 4;     // byte address for ds_bpermute
   const int tile_n = bid % tiles_n, tile_m = bid / tiles_n;
