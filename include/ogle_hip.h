@@ -212,7 +212,10 @@ int32_t ogle_hip_pool2d(const OglePoolArgs* args, ogle_stream_t stream);
  * of concat_multi.glsl:14-114 (numpy.concatenate).  Each input i is viewed as
  * (outer, axis_len[i], inner) row-major and lands at its running offset along
  * the axis of the (outer, sum axis_len, inner) output.  One launch for all
- * inputs.  n_inputs <= OGLE_CONCAT_MAX_INPUTS.
+ * inputs.  n_inputs <= OGLE_CONCAT_MAX_INPUTS.  With outer == 1 the output is the
+ * inputs back to back: if every input already lies at its place inside the output
+ * (the runtime lets the producers write there), nothing is launched; an input may
+ * not overlap the output in any other way.
  */
 typedef struct OgleConcatArgs {
   const void* inputs_dev[OGLE_CONCAT_MAX_INPUTS];

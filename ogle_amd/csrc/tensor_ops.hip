@@ -354,6 +354,16 @@ int32_t launch_concat(const OgleConcatArgs& a, hipStream_t s) {
   }
   p.out_run = off;
   if (off == 0 || a.outer == 0) return OGLE_OK;
+  if (a.outer == 1) {
+    // a single outer slice: the output is the inputs back to back, and a caller may
+    // have had them produced in place; then there is nothing to move
+    bool in_place = true;
+    for (int i = 0; i < a.n_inputs; ++i)
+      if (p.run[i] > 0 &&
+          a.inputs_dev[i] != static_cast<const unsigned char*>(a.output_dev) + p.start[i] * esz)
+        in_place = false;
+    if (in_place) return OGLE_OK;
+  }
   if (vec_ok) {
     for (int i = 0; i < a.n_inputs; ++i) {
       p.run[i] /= vec;

@@ -143,8 +143,69 @@ void FBOSession::Setup(const NamedTensorList& inputs_cpu) {
       UpdateKernelReady(kernel);
     }
   }
+  PlaceInputsInOutputs();
   BuildSchedule();
   finalized_ = true;
+}
+
+// Where a node's output is nothing but its inputs back to back (a Concat with a single
+// slice before its axis: the SSD box and class concats at batch 1), the producers of
+// those inputs are pointed at their places inside the output, so that the node has
+// nothing left to copy (ogle_hip_concat then launches nothing).  An input qualifies if,
+// looking through nodes that only re-interpret memory, it is the whole output of a live
+// node with its own allocation that has not been placed already; its place must be
+// 16-byte aligned unless the producer is a convolution whose channel count is not a
+// multiple of four (those store element by element).  All inputs of the node must
+// qualify.  Every tensor that aliases a moved allocation is re-pointed with it.
+void FBOSession::PlaceInputsInOutputs() {
+  std::map<int, std::pair<Kernel*, int>> producer;  // tensor index -> (kernel, output slot)
+  for (auto& k : kernels_)
+    for (size_t j = 0; j < k->output_tensor_indexes_.size(); ++j)
+      producer[k->output_tensor_indexes_[j]] = {k.get(), static_cast<int>(j)};
+  std::set<int> placed;
+  for (auto& kp : kernels_) {
+    Kernel* k = kp.get();
+    if (CheckKernelReady(k)) continue;
+    const std::vector<size_t> offsets = k->InputOffsetsInOutput();
+    if (offsets.empty() || offsets.size() != k->input_tensor_indexes_.size()) continue;
+    Tensor* out = k->output_tensors_[0];
+    if (!out->owns_device_buffer()) continue;
+    std::vector<int> roots;
+    bool ok = true;
+    for (size_t i = 0; i < offsets.size() && ok; ++i) {
+      int idx = k->input_tensor_indexes_[i];
+      Kernel* pk = nullptr;
+      for (;;) {
+        auto it = producer.find(idx);
+        if (it == producer.end()) { ok = false; break; }  // a graph input
+        pk = it->second.first;
+        const int alias = pk->OutputAliasesInput(it->second.second);
+        if (alias < 0) break;
+        idx = pk->input_tensor_indexes_[alias];
+      }
+      if (!ok) break;
+      Tensor* root = total_tensors_[idx].get();
+      const uintptr_t place = reinterpret_cast<uintptr_t>(out->device_ptr()) + offsets[i];
+      const bool by_element = pk->kernel_type() == "Conv" && root->shape().back() % 4 != 0;
+      ok = !CheckKernelReady(pk) && root->owns_device_buffer() && placed.count(idx) == 0 &&
+           std::find(roots.begin(), roots.end(), idx) == roots.end() &&
+           root->num_elements() == k->input_tensors_[i]->num_elements() &&
+           (place % 16 == 0 || (by_element && place % 4 == 0));
+      roots.push_back(idx);
+    }
+    if (!ok) continue;
+    for (size_t i = 0; i < offsets.size(); ++i) {
+      Tensor* root = total_tensors_[roots[i]].get();
+      void* const old = root->device_ptr();
+      void* const place = static_cast<unsigned char*>(out->device_ptr()) + offsets[i];
+      for (auto& t : total_tensors_)
+        if (t && t.get() != root && t->mem_type() == Tensor::DEVICE_BUFFER &&
+            !t->owns_device_buffer() && t->device_ptr() == old)
+          t->Rebind(place);
+      root->Rebind(place);
+      placed.insert(roots[i]);
+    }
+  }
 }
 
 // Issue order of a pass.  The context defers convolutions and launches the

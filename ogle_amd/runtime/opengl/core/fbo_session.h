@@ -81,6 +81,7 @@ class FBOSession {
 
  private:
   bool CheckKernelReady(const Kernel* kernel);
+  void PlaceInputsInOutputs();
   void BuildSchedule();
   void UpdateKernelReady(const Kernel* kernel);
 

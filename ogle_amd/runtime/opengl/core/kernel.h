@@ -61,7 +61,11 @@ class Kernel {
   // re-interpretation of dense memory), or -1.  Not in the reference, where every
   // layout change is a draw call; with linear NHWC buffers Reshape and an identity
   // Transpose move no data.  Consulted by the executor after InferOutputShape.
-  virtual int OutputAliasesInput(int i) const {
+// If output 0 is nothing but the inputs placed back to back, the byte offset of
+  // every input inside it (the session may then have the inputs produced in place);
+  // empty otherwise.  Valid after InferOutputShape.
+  virtual std::vector<size_t> InputOffsetsInOutput() const { return {}; }
+    virtual int OutputAliasesInput(int i) const {
     (void)i;
     return -1;
   }

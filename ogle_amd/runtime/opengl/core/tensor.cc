@@ -83,6 +83,14 @@ Tensor::Tensor(const Tensor* other, IntList shape, DataFormat dformat)
   allocated_size_ = other->AllocatedSize();
 }
 
+void Tensor::Rebind(void* ptr) {
+  CHECK(mem_type_ != HOST_MEMORY && device_ != nullptr) << "only device tensors can be rebound";
+  DeviceBuffer* buf = device<DeviceBuffer>();
+  if (buf->owned && buf->ptr != nullptr) (void)hipFree(buf->ptr);
+  buf->ptr = ptr;
+  buf->owned = false;
+}
+
 Tensor::~Tensor() {
   if (host_ != nullptr) std::free(host_);
   if (device_ != nullptr) {

@@ -67,6 +67,11 @@ class Tensor {
   T* host() const { return reinterpret_cast<T*>(host_); }
   // Raw device address of the first element.
   void* device_ptr() const { return device_ ? device<DeviceBuffer>()->ptr : nullptr; }
+  // True when this tensor's device memory is its own allocation (not a view).
+  bool owns_device_buffer() const { return device_ != nullptr && device<DeviceBuffer>()->owned; }
+  // Makes this device tensor a view of memory owned elsewhere, starting at `ptr`
+  // (its own allocation, if any, is released).  The contents are not moved.
+  void Rebind(void* ptr);
 
   const IntList& shape() const { return shape_; }
   size_t num_elements() const;

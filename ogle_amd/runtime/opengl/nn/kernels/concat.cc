@@ -41,6 +41,22 @@ void ConcatKernel::InferOutputShape(const TensorList& input_tensors, TensorShape
   }
 }
 
+// With a single slice before the axis (batch 1 on axis 1, or axis 0) the output is the
+// inputs back to back.
+std::vector<size_t> ConcatKernel::InputOffsetsInOutput() const {
+  if (input_tensors_.empty() || output_tensors_.empty()) return {};
+  const IntList& out = output_tensors_[0]->shape();
+  for (int d = 0; d < axis_; ++d)
+    if (out[d] != 1) return {};
+  std::vector<size_t> offsets;
+  size_t at = 0;
+  for (const Tensor* t : input_tensors_) {
+    offsets.push_back(at);
+    at += t->num_elements() * sizeof(float);
+  }
+  return offsets;
+}
+
 void ConcatKernel::Compute(TensorList& inputs, TensorList& outputs) {
   program_->Activate();
   const IntList& out = outputs[0]->shape();

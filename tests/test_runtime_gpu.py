@@ -266,6 +266,35 @@ def test_mobilenet_ssd_every_layer_matches_oracle():
     np.testing.assert_array_equal(sess.get_output("anchors", "ANY"), info["anchors"])
 
 
+def test_concat_inputs_are_produced_in_place_at_batch1():
+    """With a single slice before the concat axis (batch 1) the heads write straight into the
+    concat outputs: every head output sits at its running offset inside box_preds / cls_logits
+    (the class heads at offsets that are only 4-byte aligned: 63 and 126 channels are stored
+    element by element), the concat has nothing to copy, and a replay after new input still gives
+    the concatenation.  At batch 2 the outputs interleave per image and nothing is placed."""
+    sess, info, x = _run_ssd(1)
+    for out_name, suffix, last in (("box_preds", "loc", 4), ("cls_logits", "conf", 21)):
+        base = sess.tensor_device_ptr(out_name)
+        off = 0
+        for i in range(6):
+            assert sess.tensor_device_ptr("head%d.%s" % (i, suffix)) == base + off, (out_name, i)
+            assert sess.tensor_device_ptr("head%d.%s.view" % (i, suffix)) == base + off
+            off += int(np.prod(sess.tensor_shape("head%d.%s" % (i, suffix)))) * 4
+        assert off == 1917 * last * 4
+    x2 = rng(77).uniform(-1, 1, x.shape).astype(np.float32)
+    sess.run({"input": x2})
+    for out_name, suffix, last in (("box_preds", "loc", 4), ("cls_logits", "conf", 21)):
+        parts = [sess.get_output("head%d.%s" % (i, suffix), "NHWC").reshape(1, -1, last) for i in range(6)]
+        np.testing.assert_array_equal(sess.get_output(out_name, "ANY"), np.concatenate(parts, 1))
+    # the same network at batch 1 and as image 0 of a batch of 2 (nothing placed there)
+    sess2, _, xb = _run_ssd(2)
+    assert sess2.tensor_device_ptr("head0.loc") != sess2.tensor_device_ptr("box_preds")
+    sess.run({"input": xb[:1]})
+    for name in ("box_preds", "cls_logits"):
+        a, b = sess.get_output(name, "ANY"), sess2.get_output(name, "ANY")[:1]
+        assert np.all(np.abs(a - b) <= 1e-4 * (np.abs(b) + 1.0)), name
+
+
 def test_graph_replay_equals_eager_batch2():
     """The captured hipGraph is replayed several times with eager work and synchronisations in
     between; every replay must reproduce the eager result bit for bit."""
