@@ -365,6 +365,13 @@ int32_t ogle_hip_ssd_decode(const OgleDecodeArgs* args, ogle_stream_t stream);
  * (what the reference reads back).  If prediction_dev is NULL, boxes_dev is an
  * INPUT holding already decoded boxes.  Any kept_* pointer except
  * kept_count_dev may be NULL.
+ *
+ * kept_count_dev == NULL asks for the lists IN PLACE instead: no compaction pass,
+ * every prior's record stays at its own slot [b*priors + i] and kept_prior_dev holds
+ * i for a kept prior and -1 for a dropped one (the other lists are written for every
+ * prior).  All five lists are then required.  ogle_hip_ssd_topk_nms takes such lists
+ * when its kept_count_dev is NULL; a caller that only wants the final detections
+ * saves one launch per pass this way.
  */
 typedef struct OgleDetectArgs {
   const float* logits_dev;     /* (batch, priors, classes) */
@@ -398,6 +405,9 @@ int32_t ogle_hip_ssd_detect(const OgleDetectArgs* args, ogle_stream_t stream);
  *   - the first min(count, topk) entries go to NMS: entry j is dropped if any
  *     earlier entry i has iou(i, j) > nms_threshold (strict), whether or not i
  *     was itself dropped (detector.cc:130-141).
+ * kept_count_dev == NULL: the lists are in place as ogle_hip_ssd_detect leaves them
+ * without kept_count_dev (all `stride` slots are looked at, kept_prior_dev < 0 marks
+ * an empty one); the results are the same.
  * Inputs are indexed [b*stride + r], r < kept_count_dev[b]; outputs
  * [b*topk + r], r < final_count_dev[b], in sorted order.  kept_box_dev /
  * final_box_dev may both be NULL.  1 <= topk <= 1024, stride <= 8192 and

@@ -341,8 +341,12 @@ int32_t ogle_hip_ssd_detect(const OgleDetectArgs* a, ogle_stream_t stream) {
     return fail(OGLE_ERR_INVALID_ARG, "ssd_detect: bad size");
   if (a->classes > 40)  // the logit slab of 256 priors must fit LDS
     return fail(OGLE_ERR_UNSUPPORTED, "ssd_detect: more than 40 classes");
-  if (!a->kept_count_dev && a->batch > 0)
-    return fail(OGLE_ERR_INVALID_ARG, "ssd_detect: kept_count_dev is required");
+  if (!a->kept_count_dev && a->batch > 0 &&
+      (!a->kept_prior_dev || !a->kept_class_dev || !a->kept_score_dev || !a->kept_box_dev ||
+       !a->kept_rect_dev || a->batch > 65535))
+    return fail(OGLE_ERR_INVALID_ARG,
+                "ssd_detect: without kept_count_dev (lists left in place) every other list is "
+                "required and batch <= 65535");
   if ((long)a->batch * a->priors > 0) {
     if (!a->logits_dev) return fail(OGLE_ERR_INVALID_ARG, "ssd_detect: null logits");
     if (a->prediction_dev && !a->anchors_dev)
@@ -431,8 +435,8 @@ int32_t ogle_hip_ssd_topk_nms(const OgleNmsArgs* a, ogle_stream_t stream) {
                 "ssd_topk_nms: more than 8192 entries per image, or stride*4 + topk*28 bytes "
                 "exceed 64 KB of LDS");
   if (a->batch > 0) {
-    if (!a->kept_count_dev || !a->final_count_dev)
-      return fail(OGLE_ERR_INVALID_ARG, "ssd_topk_nms: count pointers are required");
+    if (!a->final_count_dev)
+      return fail(OGLE_ERR_INVALID_ARG, "ssd_topk_nms: final_count_dev is required");
     if (a->stride > 0 && (!a->kept_prior_dev || !a->kept_class_dev || !a->kept_score_dev ||
                           !a->kept_rect_dev))
       return fail(OGLE_ERR_INVALID_ARG, "ssd_topk_nms: null input list");

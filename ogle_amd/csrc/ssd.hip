@@ -357,10 +357,16 @@ __device__ __forceinline__ int block_rank(bool flag, int* wave_count, int lane, 
   return before;
 }
 
+//
+// SPARSE: the lists are not compacted (ogle_hip_ssd_detect without kept_count_dev): all
+// `stride` slots of an image are looked at and a slot with kept_prior < 0 is empty.  An
+// empty slot gets key 0, which no kept score has (scores that passed `> threshold` are
+// not negative, and the key of +0 is 0x80000000), so it is never selected.
+template <bool SPARSE>
 __global__ __launch_bounds__(kNmsThreads) void ssd_topk_nms_kernel(NmsParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char nms_lds[];
   // keys[stride] | cand_key[topk] | cand_idx[topk] | sel[topk] | frect[topk] |
-  // hist[256] | misc[kNmsWaves + 2]     (topk and stride rounded up to 4)
+  // hist[256] | misc[kNmsWaves + 4]     (topk and stride rounded up to 4)
   const int tpad = (p.topk + 3) & ~3;
   unsigned* keys = reinterpret_cast<unsigned*>(nms_lds);
   unsigned* cand_key = keys + ((p.stride + 3) & ~3);
@@ -374,22 +380,43 @@ __global__ __launch_bounds__(kNmsThreads) void ssd_topk_nms_kernel(NmsParams p) 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const long row0 = (long)b * p.stride;
-  int n = p.kept_count[b];
-  n = n < 0 ? 0 : (n > p.stride ? p.stride : n);
-  for (int i = tid; i < n; i += kNmsThreads) keys[i] = ordered_bits(p.kept_score[row0 + i]);
-  __syncthreads();
+  int n;   // slots looked at
+  int nv;  // entries among them
+  if constexpr (SPARSE) {
+    n = p.stride;
+    if (tid == 0) misc[kNmsWaves + 2] = 0;
+    int mine = 0;
+    for (int i = tid; i < n; i += kNmsThreads) {
+      const bool live = p.kept_prior[row0 + i] >= 0;
+      keys[i] = live ? ordered_bits(p.kept_score[row0 + i]) : 0u;
+      mine += live ? 1 : 0;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) mine += __shfl_xor(mine, d, 64);
+    if (lane == 0 && mine > 0) atomicAdd(&misc[kNmsWaves + 2], mine);
+    __syncthreads();
+    nv = misc[kNmsWaves + 2];
+  } else {
+    n = p.kept_count[b];
+    n = n < 0 ? 0 : (n > p.stride ? p.stride : n);
+    nv = n;
+    for (int i = tid; i < n; i += kNmsThreads) keys[i] = ordered_bits(p.kept_score[row0 + i]);
+    __syncthreads();
+  }
 
   // 1. the k-th largest key
-  const int m = n < p.topk ? n : p.topk;
+  const int m = nv < p.topk ? nv : p.topk;
   unsigned prefix = 0, mask = 0;
   int remaining = m;  // how many of the entries matching `prefix` are still wanted
-  if (n > p.topk) {
+  if (nv > p.topk) {
     for (int shift = 24; shift >= 0; shift -= 8) {
       if (tid < 256) hist[tid] = 0;
       __syncthreads();
       for (int i = tid; i < n; i += kNmsThreads) {
         const unsigned k = keys[i];
-        if ((k & mask) == prefix) atomicAdd(&hist[(k >> shift) & 255u], 1);
+        // (empty slots stay out: they would all hit one counter, and cannot be chosen)
+        if ((!SPARSE || k != 0u) && (k & mask) == prefix) atomicAdd(&hist[(k >> shift) & 255u], 1);
       }
       __syncthreads();
       // thread t < 256: entries whose digit is above t, and at or above t (suffix sums
@@ -420,7 +447,7 @@ __global__ __launch_bounds__(kNmsThreads) void ssd_topk_nms_kernel(NmsParams p) 
     }
   }
   // now: take every key above `prefix`, and the first `remaining` equal to it
-  // (n <= topk: every entry is taken)
+  // (nv <= topk: every entry is taken)
 
   // 2. ordered compaction of the selected entries
   {
@@ -428,8 +455,9 @@ __global__ __launch_bounds__(kNmsThreads) void ssd_topk_nms_kernel(NmsParams p) 
     for (int start = 0; start < n; start += kNmsThreads) {
       const int i = start + tid;
       const unsigned k = i < n ? keys[i] : 0u;
-      const bool gt = i < n && (n <= p.topk || k > prefix);
-      const bool eq = i < n && n > p.topk && k == prefix;
+      const bool live = i < n && (!SPARSE || k != 0u);
+      const bool gt = live && (nv <= p.topk || k > prefix);
+      const bool eq = live && nv > p.topk && k == prefix;
       int eq_total, total;
       const int eq_before = equal_seen + block_rank(eq, misc, lane, wave, &eq_total);
       const bool take = gt || (eq && eq_before < remaining);
@@ -523,7 +551,7 @@ __global__ __launch_bounds__(kNmsThreads) void ssd_topk_nms_kernel(NmsParams p) 
 size_t topk_nms_lds_bytes(int stride, int topk) {
   const size_t tpad = (size_t)((topk + 3) & ~3);
   return 4 * (size_t)((stride + 3) & ~3) + 4 * 3 * tpad + sizeof(float4) * tpad +
-         4 * (256 + kNmsWaves + 2);
+         4 * (256 + kNmsWaves + 4);
 }
 
 int32_t launch_topk_nms(const OgleNmsArgs& a, hipStream_t s) {
@@ -544,8 +572,13 @@ int32_t launch_topk_nms(const OgleNmsArgs& a, hipStream_t s) {
   p.out_score = a.final_score_dev;
   p.out_box = reinterpret_cast<float4*>(a.final_box_dev);
   p.out_rect = reinterpret_cast<int4*>(a.final_rect_dev);
-  hipLaunchKernelGGL(ssd_topk_nms_kernel, dim3((unsigned)a.batch), dim3(kNmsThreads),
-                     topk_nms_lds_bytes(a.stride, a.topk), s, p);
+  if (a.kept_count_dev == nullptr) {
+    hipLaunchKernelGGL(ssd_topk_nms_kernel<true>, dim3((unsigned)a.batch), dim3(kNmsThreads),
+                       topk_nms_lds_bytes(a.stride, a.topk), s, p);
+  } else {
+    hipLaunchKernelGGL(ssd_topk_nms_kernel<false>, dim3((unsigned)a.batch), dim3(kNmsThreads),
+                       topk_nms_lds_bytes(a.stride, a.topk), s, p);
+  }
   return check_launch("ssd_topk_nms_kernel");
 }
 
@@ -580,12 +613,14 @@ int32_t launch_detect(const OgleDetectArgs& a, hipStream_t s) {
   p.kept_rect = reinterpret_cast<int4*>(a.kept_rect_dev);
   const size_t lds = sizeof(float) * 256 * (size_t)a.classes;
   const bool all_outputs = p.kept_prior && p.kept_class && p.kept_score && p.kept_box && p.kept_rect;
-  if (all_outputs && a.priors > 256 && a.batch <= 65535) {
+  const bool sparse = p.kept_count == nullptr;  // validated: all outputs given, batch <= 65535
+  if (sparse && a.priors == 0) return OGLE_OK;
+  if (sparse || (all_outputs && a.priors > 256 && a.batch <= 65535)) {
     hipLaunchKernelGGL(ssd_score_kernel,
                        dim3((unsigned)((a.priors + kScorePriors - 1) / kScorePriors), (unsigned)a.batch),
                        dim3(256), sizeof(float) * kScorePriors * (size_t)a.classes, s, p);
     const int32_t st = check_launch("ssd_score_kernel");
-    if (st != OGLE_OK) return st;
+    if (st != OGLE_OK || sparse) return st;
     hipLaunchKernelGGL(ssd_compact_kernel, dim3((unsigned)a.batch), dim3(kCompactThreads), 0, s, p);
     return check_launch("ssd_compact_kernel");
   }

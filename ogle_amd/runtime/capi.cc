@@ -135,8 +135,7 @@ int32_t ogle_rt_time_compute(OgleSession* s, int32_t warmup, int32_t iters, int3
     opt.device_nms = s->device_nms;
     if (with_detect && !s->detector) s->detector = opengl::Detector::Create(s->session.get(), opt);
     auto detect = [&]() {
-      s->detector->EnqueuePostprocess(opt.output_names, 300, 300);
-      if (s->detector->UsesDeviceNms()) s->detector->EnqueueTopkNms();
+      s->detector->EnqueueDetect(opt.output_names, 300, 300);
     };
     if (with_detect) {
       detect();  // first use allocates the result buffers: keep that out of a capture

@@ -44,7 +44,9 @@ void Detector::LoadToOutputTensors(const TensorNameList& names, int raw_width, i
   Readback();
 }
 
-void Detector::EnqueuePostprocess(const TensorNameList& names, int raw_width, int raw_height) {
+void Detector::EnqueuePostprocess(const TensorNameList& names, int raw_width, int raw_height,
+                                  bool lists_in_place) {
+  lists_in_place_ = lists_in_place;
   CHECK_EQ(names.size(), 3u);
   Tensor* cls_logits = session_->FindTensorByName(names[0]);
   Tensor* box_preds = session_->FindTensorByName(names[1]);
@@ -53,6 +55,7 @@ void Detector::EnqueuePostprocess(const TensorNameList& names, int raw_width, in
   CHECK_EQ(cls_logits->shape().size(), 3u);
   CHECK_EQ(box_preds->shape().size(), 3u);
   const int batch = box_preds->shape()[0], priors = box_preds->shape()[1];
+  priors_for_nms_ = priors;
   const int classes = cls_logits->shape()[2];
   CHECK_EQ(box_preds->shape()[2], 4);
   CHECK_EQ(cls_logits->shape()[0], batch);
@@ -93,7 +96,8 @@ void Detector::EnqueuePostprocess(const TensorNameList& names, int raw_width, in
   a.score_threshold = options_.score_threshold;
   a.image_width = static_cast<float>(raw_width);
   a.image_height = static_cast<float>(raw_height);
-  a.kept_count_dev = static_cast<int32_t*>(count_dev_->device_ptr());
+  // in place: no compaction launch; only the device top-k + NMS can read such lists
+  a.kept_count_dev = lists_in_place ? nullptr : static_cast<int32_t*>(count_dev_->device_ptr());
   a.kept_prior_dev = static_cast<int32_t*>(prior_dev_->device_ptr());
   a.kept_class_dev = static_cast<int32_t*>(class_dev_->device_ptr());
   a.kept_score_dev = static_cast<float*>(score_dev_->device_ptr());
@@ -107,6 +111,7 @@ void Detector::EnqueuePostprocess(const TensorNameList& names, int raw_width, in
 
 void Detector::Readback() {
   CHECK(batch_ > 0) << "EnqueuePostprocess first";
+  CHECK(!lists_in_place_) << "the kept lists were left in place for the device top-k + NMS";
   hipStream_t s = static_cast<hipStream_t>(session_->context()->stream());
   auto back = [&](void* dst, const Tensor* src, size_t bytes) {
     const hipError_t e = hipMemcpyAsync(dst, src->device_ptr(), bytes, hipMemcpyDeviceToHost, s);
@@ -155,8 +160,22 @@ void Detector::GenerateBoxInfo(int image, std::vector<BoxInfo>* box_infos) const
 
 bool Detector::UsesDeviceNms() const {
   // the device kernel stages one image's scores and candidates in 64 KB of LDS
-  return options_.device_nms && options_.topk >= 1 && options_.topk <= 1024 && priors_ <= 8192 &&
-         4L * priors_ + 28L * options_.topk + 2048 <= 64 * 1024;
+  const int priors = priors_for_nms_;
+  return options_.device_nms && options_.topk >= 1 && options_.topk <= 1024 && priors <= 8192 &&
+         4L * priors + 28L * options_.topk + 2048 <= 64 * 1024;
+}
+
+// Everything Detect does on the device after the network: with device top-k + NMS the
+// score filter leaves its lists in place (no compaction launch) and the top-k + NMS
+// launch reads them there; without, the score filter compacts them for the host.
+void Detector::EnqueueDetect(const TensorNameList& names, int raw_width, int raw_height) {
+  // whether the device kernel fits depends on the output shapes: look before launching
+  const Tensor* box_preds = session_->FindTensorByName(names.size() == 3 ? names[1] : "");
+  CHECK(box_preds != nullptr && box_preds->shape().size() == 3u) << "detector outputs were not produced";
+  priors_for_nms_ = box_preds->shape()[1];
+  const bool device = UsesDeviceNms();
+  EnqueuePostprocess(names, raw_width, raw_height, device);
+  if (device) EnqueueTopkNms();
 }
 
 void Detector::EnqueueTopkNms() {
@@ -182,7 +201,8 @@ void Detector::EnqueueTopkNms() {
     frect_.resize(fprior_.size() * 4);
   }
   OgleNmsArgs a{};
-  a.kept_count_dev = static_cast<const int32_t*>(count_dev_->device_ptr());
+  a.kept_count_dev =
+      lists_in_place_ ? nullptr : static_cast<const int32_t*>(count_dev_->device_ptr());
   a.kept_prior_dev = static_cast<const int32_t*>(prior_dev_->device_ptr());
   a.kept_class_dev = static_cast<const int32_t*>(class_dev_->device_ptr());
   a.kept_score_dev = static_cast<const float*>(score_dev_->device_ptr());
@@ -247,9 +267,8 @@ void Detector::NMS(std::vector<BoxInfo>& boxes, std::vector<BoxInfo>& boxes_left
 void Detector::Detect(const Tensor* images, int raw_width, int raw_height,
                       std::vector<std::vector<BoxInfo>>* final_boxes) {
   Run(images);
-  EnqueuePostprocess(options_.output_names, raw_width, raw_height);
+  EnqueueDetect(options_.output_names, raw_width, raw_height);
   if (UsesDeviceNms()) {
-    EnqueueTopkNms();
     ReadbackFinal(final_boxes);
     return;
   }

@@ -66,13 +66,20 @@ class Detector {
   void LoadToOutputTensors(const TensorNameList& names, int raw_width, int raw_height);
   // The two halves of LoadToOutputTensors: the device launch (asynchronous, buffers
   // allocated on first use) and the readback of its compacted results (synchronises).
-  void EnqueuePostprocess(const TensorNameList& names, int raw_width, int raw_height);
+  // lists_in_place: skip the compaction launch and leave every prior's record at its own
+  // slot (kept prior index or -1); only EnqueueTopkNms can read such lists.
+  void EnqueuePostprocess(const TensorNameList& names, int raw_width, int raw_height,
+                          bool lists_in_place = false);
   void Readback();
   // Device top-k + NMS over what EnqueuePostprocess left on the device
   // (asynchronous), and the readback of its final lists (synchronises).
   void EnqueueTopkNms();
   void ReadbackFinal(std::vector<std::vector<BoxInfo>>* final_boxes);
   bool UsesDeviceNms() const;
+  // Everything Detect does on the device after the network (asynchronous): the score
+  // filter, and with device top-k + NMS that launch too (ReadbackFinal fetches its
+  // lists; otherwise Readback + HostTopkNms finish on the host).
+  void EnqueueDetect(const TensorNameList& names, int raw_width, int raw_height);
   // The reference's host loop over what Readback() fetched: GenerateBoxInfo, GetTopK,
   // NMS per image.
   void HostTopkNms(std::vector<std::vector<BoxInfo>>* final_boxes) const;
@@ -88,6 +95,8 @@ class Detector {
   FBOSession* session_;
   bool owns_session_;
   int batch_ = 0, priors_ = 0, classes_ = 0;
+  int priors_for_nms_ = 0;       // prior count of the outputs last looked at
+  bool lists_in_place_ = false;  // how the last EnqueuePostprocess left the kept lists
   // device results of the fused decode + score filter, and their host copies
   std::unique_ptr<Tensor> boxes_dev_, count_dev_, prior_dev_, class_dev_, score_dev_, box_dev_,
       rect_dev_;

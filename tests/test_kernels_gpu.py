@@ -544,6 +544,79 @@ def test_topk_nms_matches_oracle(seed, stride, topk, spread):
         np.testing.assert_array_equal(got[b]["box"], box[b, :n][keep])
 
 
+@pytest.mark.parametrize("batch,priors,topk,sigma", [(1, 1917, 100, 0.9), (16, 1917, 100, 0.9),
+                                                     (3, 1917, 100, 0.35), (2, 1917, 1024, 2.0),
+                                                     (4, 300, 16, 1.0), (2, 70, 200, 1.0)])
+def test_detect_lists_in_place_then_topk_nms(batch, priors, topk, sigma):
+    """ogle_hip_ssd_detect without kept_count_dev leaves every prior's record at its own slot
+    (kept_prior = index or -1, no compaction launch); ogle_hip_ssd_topk_nms without
+    kept_count_dev reads such lists.  The final lists must equal, bit for bit, those of the
+    compacted path, which other tests hold to the oracle."""
+    import ctypes
+    import torch
+    r = rng(9700 + batch + priors + topk)
+    classes = 21
+    logits = r.normal(0, sigma, (batch, priors, classes)).astype(np.float32)
+    logits[0] = np.round(logits[0] * 4) / 4      # frequent equal scores in image 0
+    pred = r.normal(0, 1.0, (batch, priors, 4)).astype(np.float32)
+    anchors = ssd_anchors() if priors == 1917 else np.concatenate(
+        [r.uniform(.1, .9, (priors, 2)), r.uniform(.05, .5, (priors, 2))], 1).astype(np.float32)
+    kept, boxes = gpu_detect(logits, pred, anchors, 0.3, 300.0, 300.0)
+    counts = np.array([len(k["prior"]) for k in kept], np.int32)
+
+    def padded(key, shape, dtype):
+        out = np.zeros((batch,) + shape, dtype)
+        for b in range(batch):
+            out[b, :counts[b]] = kept[b][key]
+        return out
+    ref = gpu_topk_nms(counts, padded("prior", (priors,), np.int32), padded("cls", (priors,), np.int32),
+                       padded("score", (priors,), np.float32), padded("rect", (priors, 4), np.int32),
+                       topk, 0.45, padded("box", (priors, 4), np.float32))
+    i32 = dict(dtype=torch.int32, device="cuda")
+    f32 = dict(dtype=torch.float32, device="cuda")
+    ld, pd, ad = (torch.from_numpy(a).cuda() for a in (logits, pred, anchors))
+    bx = torch.empty((batch, priors, 4), **f32)
+    kp = torch.full((batch, priors), -5, **i32)
+    kc = torch.full((batch, priors), -5, **i32)
+    ks = torch.full((batch, priors), float("nan"), **f32)
+    kb = torch.full((batch, priors, 4), float("nan"), **f32)
+    kr = torch.full((batch, priors, 4), -5, **i32)
+    st = torch.cuda.current_stream().cuda_stream
+    da = H.DetectArgs(ld.data_ptr(), pd.data_ptr(), ad.data_ptr(), bx.data_ptr(), batch, priors, classes,
+                      0, (ctypes.c_float * 4)(.1, .1, .2, .2), 0.3, 300.0, 300.0, None, kp.data_ptr(),
+                      kc.data_ptr(), ks.data_ptr(), kb.data_ptr(), kr.data_ptr())
+    H.check(H.lib().ogle_hip_ssd_detect(ctypes.byref(da), st))
+    fc = torch.full((batch,), -7, **i32)
+    fp = torch.full((batch, topk), -7, **i32)
+    fk = torch.full((batch, topk), -7, **i32)
+    fs = torch.full((batch, topk), float("nan"), **f32)
+    fb = torch.full((batch, topk, 4), float("nan"), **f32)
+    fr = torch.full((batch, topk, 4), -7, **i32)
+    na = H.NmsArgs(None, kp.data_ptr(), kc.data_ptr(), ks.data_ptr(), kb.data_ptr(), kr.data_ptr(), batch,
+                   priors, topk, 0.45, fc.data_ptr(), fp.data_ptr(), fk.data_ptr(), fs.data_ptr(),
+                   fb.data_ptr(), fr.data_ptr())
+    H.check(H.lib().ogle_hip_ssd_topk_nms(ctypes.byref(na), st))
+    torch.cuda.synchronize()
+    # the in-place lists: kept priors carry their index, dropped ones -1
+    kpn = kp.cpu().numpy()
+    for b in range(batch):
+        np.testing.assert_array_equal(np.nonzero(kpn[b] >= 0)[0], kept[b]["prior"])
+        assert np.all((kpn[b] == -1) | (kpn[b] == np.arange(priors)))
+    n = fc.cpu().numpy()
+    for b in range(batch):
+        k = int(n[b])
+        assert k == len(ref[b]["prior"]), (b, k)
+        np.testing.assert_array_equal(fp[b, :k].cpu().numpy(), ref[b]["prior"])
+        np.testing.assert_array_equal(fk[b, :k].cpu().numpy(), ref[b]["cls"])
+        np.testing.assert_array_equal(fs[b, :k].cpu().numpy(), ref[b]["score"])
+        np.testing.assert_array_equal(fr[b, :k].cpu().numpy(), ref[b]["rect"])
+        np.testing.assert_array_equal(fb[b, :k].cpu().numpy(), ref[b]["box"])
+        assert (fp[b, k:] == -7).all()
+    # in-place lists need every list
+    da.kept_rect_dev = None
+    assert H.lib().ogle_hip_ssd_detect(ctypes.byref(da), st) == H.ERR_INVALID_ARG
+
+
 def test_topk_nms_rejects_bad_sizes():
     import ctypes
     a = H.NmsArgs()
