@@ -63,6 +63,20 @@ int32_t ogle_rt_time_compute(OgleSession* s, int32_t warmup, int32_t iters, int3
                              float* total_ms);
 
 /*
+ * Throughput of `n` sessions that hold the same graph, run as a pipeline: every session
+ * replays its pass (network, and with_detect the detector's device work) as a hipGraph
+ * on its own stream, and `iters` passes are dealt round-robin over the sessions from the
+ * calling thread, so that one session's launch gaps and under-filled kernels are
+ * covered by the others' work.  Each session must have run once (inputs resident).
+ * `warmup` untimed passes first; total_ms is the time from the common start (all
+ * streams idle) until the last stream is idle again.  The reference executes one
+ * graph on one GL context (fbo_session.cc:127-153); this is what a server that keeps
+ * several batches in flight does with it.
+ */
+int32_t ogle_rt_time_pipelined(OgleSession** sessions, int32_t n, int32_t warmup, int32_t iters,
+                               int32_t with_detect, float* total_ms);
+
+/*
  * One pass with an event pair around every node (the reference's per-node TraceMe
  * with sync, fbo_session.cc:140-153).  Returns the number of nodes timed, or a
  * negative status.  ogle_rt_profile_entry then reads entry i: its

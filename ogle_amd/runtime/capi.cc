@@ -3,6 +3,7 @@
 
 #include <hip/hip_runtime_api.h>
 
+#include <chrono>
 #include <cstring>
 #include <exception>
 #include <memory>
@@ -173,6 +174,42 @@ int32_t ogle_rt_time_compute(OgleSession* s, int32_t warmup, int32_t iters, int3
     if (ms_each)
       for (int i = 0; i < iters; ++i) (void)hipEventElapsedTime(&ms_each[i], ev[i], ev[i + 1]);
     for (auto& e : ev) (void)hipEventDestroy(e);
+    return 0;
+  });
+}
+
+int32_t ogle_rt_time_pipelined(OgleSession** sessions, int32_t n, int32_t warmup, int32_t iters,
+                               int32_t with_detect, float* total_ms) {
+  return (int32_t)Guard([&]() -> int64_t {
+    CHECK(sessions != nullptr && n >= 1 && n <= 16) << "1..16 sessions";
+    const int slot = with_detect ? 1 : 0;
+    for (int i = 0; i < n; ++i) {
+      OgleSession* s = sessions[i];
+      CHECK(s != nullptr && s->session != nullptr) << "null session";
+      if (with_detect) {
+        opengl::DetectorOptions opt;
+        opt.device_nms = s->device_nms;
+        if (!s->detector) s->detector = opengl::Detector::Create(s->session.get(), opt);
+        auto detect = [s, opt]() { s->detector->EnqueueDetect(opt.output_names, 300, 300); };
+        if (!s->session->graph_captured(slot)) {
+          detect();  // first use allocates the result buffers: keep that out of the capture
+          s->context->Finish();
+          s->session->CaptureGraph(slot, detect);
+        }
+      } else if (!s->session->graph_captured(slot)) {
+        s->session->CaptureGraph(slot);
+      }
+    }
+    auto idle = [&]() {
+      for (int i = 0; i < n; ++i) sessions[i]->context->Finish();
+    };
+    for (int i = 0; i < warmup; ++i) sessions[i % n]->session->LaunchGraph(slot);
+    idle();
+    const auto t0 = std::chrono::steady_clock::now();
+    for (int i = 0; i < iters; ++i) sessions[i % n]->session->LaunchGraph(slot);
+    idle();
+    const auto t1 = std::chrono::steady_clock::now();
+    if (total_ms) *total_ms = std::chrono::duration<float, std::milli>(t1 - t0).count();
     return 0;
   });
 }

@@ -19,6 +19,7 @@ SYMBOLS = [
     "ogle_rt_load_file", "ogle_rt_load_bytes", "ogle_rt_run", "ogle_rt_compute",
     "ogle_rt_compute_graph", "ogle_rt_sync", "ogle_rt_time_compute", "ogle_rt_profile",
     "ogle_rt_profile_entry", "ogle_rt_tensor_shape", "ogle_rt_tensor_device_ptr",
+    "ogle_rt_time_pipelined",
     "ogle_rt_stream", "ogle_rt_get_output", "ogle_rt_num_kernels",
     "ogle_rt_registered_kernel_count", "ogle_rt_registered_kernel_name", "ogle_rt_detect",
     "ogle_rt_reserialize", "ogle_rt_model_debug_string", "ogle_rt_tensor_dformat",
@@ -63,6 +64,8 @@ def lib():
         l.ogle_rt_time_compute.argtypes = [vp, i32, i32, i32, i32, i32,
                                            ctypes.POINTER(ctypes.c_float),
                                            ctypes.POINTER(ctypes.c_float)]
+        l.ogle_rt_time_pipelined.argtypes = [ctypes.POINTER(vp), i32, i32, i32, i32,
+                                             ctypes.POINTER(ctypes.c_float)]
         l.ogle_rt_profile.argtypes = [vp]
         l.ogle_rt_profile_entry.argtypes = [vp, i32, ctypes.POINTER(cp), ctypes.POINTER(cp),
                                             ctypes.POINTER(ctypes.c_float)]
@@ -182,6 +185,17 @@ class Session:
                                           1 if with_detect else 0, 1 if sync_each else 0, each,
                                           ctypes.byref(total)))
         return np.array(each[:], np.float64), float(total.value)
+
+    @staticmethod
+    def time_pipelined(sessions, warmup, iters, with_detect=True):
+        """`iters` passes dealt round-robin over `sessions` (same graph, inputs resident), each
+        replaying its hipGraph on its own stream.  Returns the total ms from a common idle
+        start until every stream is idle again."""
+        handles = (ctypes.c_void_p * len(sessions))(*[s._h for s in sessions])
+        total = ctypes.c_float(0)
+        _check(lib().ogle_rt_time_pipelined(handles, len(sessions), warmup, iters,
+                                            1 if with_detect else 0, ctypes.byref(total)))
+        return float(total.value)
 
     def profile(self):
         """One pass with per-node events: list of (label, type, ms)."""

@@ -406,3 +406,31 @@ def test_detector_inside_graph_equals_eager(device_nms):
         sess.time_compute(1, 3, graph=use_graph, with_detect=True)
         got = sess.detect_results(batch)
         assert got == eager
+
+
+def test_pipelined_sessions_keep_their_own_results():
+    """ogle_rt_time_pipelined deals passes round-robin over several sessions, each replaying its
+    hipGraph on its own stream.  Every session must end with exactly what it computes alone:
+    outputs bit-identical to its own eager pass, detections equal to Detector::Detect on its own
+    input, whatever ran next to it."""
+    batch = 2
+    sessions, inputs, eager_out, eager_det = [], [], [], []
+    for i in range(3):
+        g, info = models.mobilenet_v1_ssd(batch, seed=41, head_std=0.05)
+        x = rng(500 + i).uniform(-1, 1, (batch, 300, 300, 3)).astype(np.float32)
+        s = session.Session()
+        s.load_graph(g)
+        eager_det.append(s.detect(x, 300, 300, 0.3, 0.45, 100))
+        eager_out.append([s.get_output(n, "ANY") for n in ("box_preds", "cls_logits")])
+        sessions.append(s)
+        inputs.append(x)
+    assert eager_det[0] != eager_det[1]          # different inputs, different detections
+    total = session.Session.time_pipelined(sessions, 3, 10, with_detect=True)
+    assert total > 0
+    for i, s in enumerate(sessions):
+        for name, ref in zip(("box_preds", "cls_logits"), eager_out[i]):
+            np.testing.assert_array_equal(s.get_output(name, "ANY"), ref)
+        assert s.detect_results(batch) == eager_det[i]
+    # a single session is accepted too, and so is the pass without the detector's work
+    assert session.Session.time_pipelined(sessions[:1], 0, 2, with_detect=False) > 0
+    np.testing.assert_array_equal(sessions[0].get_output("box_preds", "ANY"), eager_out[0][0])
