@@ -72,9 +72,20 @@ int32_t ogle_rt_time_compute(OgleSession* s, int32_t warmup, int32_t iters, int3
  * streams idle) until the last stream is idle again.  The reference executes one
  * graph on one GL context (fbo_session.cc:127-153); this is what a server that keeps
  * several batches in flight does with it.
+ *
+ * host_inputs == NULL: the inputs stay resident.  Otherwise host_inputs[i] is a host
+ * buffer with the bytes of session i's input tensor `input_name` (dense NHWC fp32, as
+ * FBOSession::Run takes it) and every pass starts with its asynchronous copy to the
+ * device on that session's stream, so uploads overlap the other sessions' kernels.
+ * The copies are only asynchronous from page-locked memory (ogle_rt_alloc_pinned).
  */
 int32_t ogle_rt_time_pipelined(OgleSession** sessions, int32_t n, int32_t warmup, int32_t iters,
-                               int32_t with_detect, float* total_ms);
+                               int32_t with_detect, const char* input_name,
+                               const void* const* host_inputs, float* total_ms);
+
+/* Page-locked host memory (hipHostMalloc / hipHostFree); NULL when it cannot be had. */
+void* ogle_rt_alloc_pinned(size_t bytes);
+void ogle_rt_free_pinned(void* p);
 
 /*
  * One pass with an event pair around every node (the reference's per-node TraceMe

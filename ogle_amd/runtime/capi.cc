@@ -178,11 +178,35 @@ int32_t ogle_rt_time_compute(OgleSession* s, int32_t warmup, int32_t iters, int3
   });
 }
 
+void* ogle_rt_alloc_pinned(size_t bytes) {
+  void* p = nullptr;
+  if (bytes == 0 || hipHostMalloc(&p, bytes, hipHostMallocDefault) != hipSuccess) return nullptr;
+  return p;
+}
+
+void ogle_rt_free_pinned(void* p) {
+  if (p != nullptr) (void)hipHostFree(p);
+}
+
 int32_t ogle_rt_time_pipelined(OgleSession** sessions, int32_t n, int32_t warmup, int32_t iters,
-                               int32_t with_detect, float* total_ms) {
+                               int32_t with_detect, const char* input_name,
+                               const void* const* host_inputs, float* total_ms) {
   return (int32_t)Guard([&]() -> int64_t {
     CHECK(sessions != nullptr && n >= 1 && n <= 16) << "1..16 sessions";
     const int slot = with_detect ? 1 : 0;
+    std::vector<void*> dev_input(n, nullptr);
+    std::vector<size_t> input_bytes(n, 0);
+    if (host_inputs != nullptr) {
+      CHECK(input_name != nullptr) << "input_name is required with host_inputs";
+      for (int i = 0; i < n; ++i) {
+        CHECK(sessions[i] != nullptr && host_inputs[i] != nullptr) << "null session or host input";
+        Tensor* t = sessions[i]->session->FindTensorByName(input_name);
+        CHECK(t != nullptr && t->device_ptr() != nullptr)
+            << "input '" << input_name << "' is not resident: Run the session once first";
+        dev_input[i] = t->device_ptr();
+        input_bytes[i] = t->num_elements() * sizeof(float);
+      }
+    }
     for (int i = 0; i < n; ++i) {
       OgleSession* s = sessions[i];
       CHECK(s != nullptr && s->session != nullptr) << "null session";
@@ -203,10 +227,20 @@ int32_t ogle_rt_time_pipelined(OgleSession** sessions, int32_t n, int32_t warmup
     auto idle = [&]() {
       for (int i = 0; i < n; ++i) sessions[i]->context->Finish();
     };
-    for (int i = 0; i < warmup; ++i) sessions[i % n]->session->LaunchGraph(slot);
+    auto step = [&](int i) {
+      OgleSession* s = sessions[i % n];
+      if (host_inputs != nullptr) {
+        const hipError_t e =
+            hipMemcpyAsync(dev_input[i % n], host_inputs[i % n], input_bytes[i % n],
+                           hipMemcpyHostToDevice, static_cast<hipStream_t>(s->context->stream()));
+        if (e != hipSuccess) LOG(FATAL) << "input upload: " << hipGetErrorString(e);
+      }
+      s->session->LaunchGraph(slot);
+    };
+    for (int i = 0; i < warmup; ++i) step(i);
     idle();
     const auto t0 = std::chrono::steady_clock::now();
-    for (int i = 0; i < iters; ++i) sessions[i % n]->session->LaunchGraph(slot);
+    for (int i = 0; i < iters; ++i) step(i);
     idle();
     const auto t1 = std::chrono::steady_clock::now();
     if (total_ms) *total_ms = std::chrono::duration<float, std::milli>(t1 - t0).count();

@@ -19,7 +19,7 @@ SYMBOLS = [
     "ogle_rt_load_file", "ogle_rt_load_bytes", "ogle_rt_run", "ogle_rt_compute",
     "ogle_rt_compute_graph", "ogle_rt_sync", "ogle_rt_time_compute", "ogle_rt_profile",
     "ogle_rt_profile_entry", "ogle_rt_tensor_shape", "ogle_rt_tensor_device_ptr",
-    "ogle_rt_time_pipelined",
+    "ogle_rt_time_pipelined", "ogle_rt_alloc_pinned", "ogle_rt_free_pinned",
     "ogle_rt_stream", "ogle_rt_get_output", "ogle_rt_num_kernels",
     "ogle_rt_registered_kernel_count", "ogle_rt_registered_kernel_name", "ogle_rt_detect",
     "ogle_rt_reserialize", "ogle_rt_model_debug_string", "ogle_rt_tensor_dformat",
@@ -64,8 +64,12 @@ def lib():
         l.ogle_rt_time_compute.argtypes = [vp, i32, i32, i32, i32, i32,
                                            ctypes.POINTER(ctypes.c_float),
                                            ctypes.POINTER(ctypes.c_float)]
-        l.ogle_rt_time_pipelined.argtypes = [ctypes.POINTER(vp), i32, i32, i32, i32,
-                                             ctypes.POINTER(ctypes.c_float)]
+        l.ogle_rt_time_pipelined.argtypes = [ctypes.POINTER(vp), i32, i32, i32, i32, cp,
+                                             ctypes.POINTER(vp), ctypes.POINTER(ctypes.c_float)]
+        l.ogle_rt_alloc_pinned.argtypes = [ctypes.c_size_t]
+        l.ogle_rt_alloc_pinned.restype = vp
+        l.ogle_rt_free_pinned.argtypes = [vp]
+        l.ogle_rt_free_pinned.restype = None
         l.ogle_rt_profile.argtypes = [vp]
         l.ogle_rt_profile_entry.argtypes = [vp, i32, ctypes.POINTER(cp), ctypes.POINTER(cp),
                                             ctypes.POINTER(ctypes.c_float)]
@@ -124,6 +128,27 @@ def registered_kernels():
     l = lib()
     return [l.ogle_rt_registered_kernel_name(i).decode()
             for i in range(l.ogle_rt_registered_kernel_count())]
+
+
+class PinnedBuffer:
+    """Page-locked host memory (ogle_rt_alloc_pinned) viewed as a numpy array."""
+
+    def __init__(self, shape, dtype=np.float32):
+        self.nbytes = int(np.prod(shape)) * np.dtype(dtype).itemsize
+        self.ptr = lib().ogle_rt_alloc_pinned(self.nbytes)
+        if not self.ptr:
+            raise MemoryError("ogle_rt_alloc_pinned(%d) failed" % self.nbytes)
+        buf = (ctypes.c_char * self.nbytes).from_address(self.ptr)
+        self.array = np.frombuffer(buf, dtype=dtype).reshape(shape)
+
+    def close(self):
+        if self.ptr:
+            self.array = None
+            lib().ogle_rt_free_pinned(self.ptr)
+            self.ptr = None
+
+    def __del__(self):
+        self.close()
 
 
 class Session:
@@ -187,14 +212,22 @@ class Session:
         return np.array(each[:], np.float64), float(total.value)
 
     @staticmethod
-    def time_pipelined(sessions, warmup, iters, with_detect=True):
-        """`iters` passes dealt round-robin over `sessions` (same graph, inputs resident), each
-        replaying its hipGraph on its own stream.  Returns the total ms from a common idle
-        start until every stream is idle again."""
+    def time_pipelined(sessions, warmup, iters, with_detect=True, input_name=None, host_inputs=None):
+        """`iters` passes dealt round-robin over `sessions` (same graph), each replaying its
+        hipGraph on its own stream.  With `host_inputs` (one PinnedBuffer per session holding the
+        bytes of input `input_name`) every pass first copies its input to the device on its
+        stream; otherwise the inputs stay resident.  Returns the total ms from a common idle start
+        until every stream is idle again."""
         handles = (ctypes.c_void_p * len(sessions))(*[s._h for s in sessions])
         total = ctypes.c_float(0)
+        hosts = None
+        if host_inputs is not None:
+            assert input_name is not None and len(host_inputs) == len(sessions)
+            hosts = (ctypes.c_void_p * len(sessions))(*[h.ptr for h in host_inputs])
         _check(lib().ogle_rt_time_pipelined(handles, len(sessions), warmup, iters,
-                                            1 if with_detect else 0, ctypes.byref(total)))
+                                            1 if with_detect else 0,
+                                            input_name.encode() if input_name else None, hosts,
+                                            ctypes.byref(total)))
         return float(total.value)
 
     def profile(self):

@@ -434,3 +434,15 @@ def test_pipelined_sessions_keep_their_own_results():
     # a single session is accepted too, and so is the pass without the detector's work
     assert session.Session.time_pipelined(sessions[:1], 0, 2, with_detect=False) > 0
     np.testing.assert_array_equal(sessions[0].get_output("box_preds", "ANY"), eager_out[0][0])
+    # with uploads from page-locked memory: the sessions swap inputs, and their results follow
+    pinned = [session.PinnedBuffer((batch, 300, 300, 3)) for _ in sessions]
+    order = [1, 2, 0]
+    for pb, j in zip(pinned, order):
+        pb.array[...] = inputs[j]
+    session.Session.time_pipelined(sessions, 1, 5, True, "input", pinned)
+    for s, j in zip(sessions, order):
+        for name, ref in zip(("box_preds", "cls_logits"), eager_out[j]):
+            np.testing.assert_array_equal(s.get_output(name, "ANY"), ref)
+        assert s.detect_results(batch) == eager_det[j]
+    for pb in pinned:
+        pb.close()
