@@ -446,3 +446,23 @@ def test_pipelined_sessions_keep_their_own_results():
         assert s.detect_results(batch) == eager_det[j]
     for pb in pinned:
         pb.close()
+
+
+def test_batch16_images_match_their_batch1_passes():
+    """The headline configuration (batch 16) takes other tile shapes, K splits and issue order than
+    batch 1.  Every image is independent through every kernel, so image i of a batch-16 pass must
+    equal a batch-1 pass over that image, up to the summation order (1e-4 of the output scale)."""
+    sess16, info, x = _run_ssd(16)
+    loc16 = sess16.get_output("box_preds", "ANY")
+    conf16 = sess16.get_output("cls_logits", "ANY")
+    feat16 = sess16.get_output("block13.pw", "NHWC")
+    assert loc16.shape == (16, 1917, 4) and conf16.shape == (16, 1917, 21)
+    g1, _ = models.mobilenet_v1_ssd(1, seed=20240005)
+    sess1 = session.Session()
+    sess1.load_graph(g1)
+    for i in (0, 7, 15):
+        sess1.run({"input": x[i:i + 1]})
+        for name, ref in (("box_preds", loc16), ("cls_logits", conf16), ("block13.pw", feat16)):
+            got = sess1.get_output(name, "ANY" if name != "block13.pw" else "NHWC")
+            scale = float(np.abs(ref[i]).max())
+            assert np.abs(got[0] - ref[i]).max() <= 1e-4 * scale, (name, i)
