@@ -470,6 +470,9 @@ def test_decode_matches_oracle():
 POOL_CASES = [
     (1, 112, 112, 64, 3, 2, 1), (2, 11, 9, 5, 2, 2, 0), (1, 8, 8, 7, 3, 1, 1), (3, 13, 13, 16, 5, 3, 2),
     (1, 4, 4, 4, 2, 2, 2),       # corner windows with no in-image tap
+    (4, 112, 112, 64, 3, 2, 1),  # 3x3 stride 2 on a large map: the 2x2-patch kernel
+    (3, 75, 61, 32, 3, 2, 0),    # the same with odd output sizes (the last patch row / column is half empty)
+    (2, 90, 90, 16, 3, 2, 2),    # and with padding 2: whole windows outside the image
 ]
 
 
