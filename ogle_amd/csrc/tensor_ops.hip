@@ -102,7 +102,9 @@ __global__ __launch_bounds__(256) void pool_small_kernel(
     PoolDiv div_cv, PoolDiv div_ow, PoolDiv div_oh) {
   typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
   constexpr unsigned kOut = 0x80000000u;
-  const unsigned idx = blockIdx.x * 256u + threadIdx.x;
+  // consecutive workgroups (neighbouring output rows, whose windows share input rows)
+  // are kept on one XCD so that the re-read rows hit that XCD's L2
+  const unsigned idx = (unsigned)xcd_swizzle((int)blockIdx.x, (int)gridDim.x) * 256u + threadIdx.x;
   if (idx >= total) return;
   const unsigned t1 = pool_div(idx, div_cv);
   const unsigned cg = idx - t1 * div_cv.d;
@@ -304,7 +306,7 @@ int32_t run_pool(const OglePoolArgs& a, hipStream_t s) {
     const long x_bytes = (long)a.n * a.in_h * a.in_w * a.c * 4, y_bytes = total4 * 16;
     if (a.c % 4 == 0 && (a.kernel_size == 2 || a.kernel_size == 3) && total4 < 0x7fffffffL &&
         x_bytes < 0x7fffffffL && y_bytes < 0x7fffffffL && total4 > 0) {
-      const dim3 grid((unsigned)((total4 + 255) / 256));
+      const dim3 grid((unsigned)(((total4 + 255) / 256 + 7) / 8 * 8));  // whole XCD rounds
 #define OGLE_POOL_SMALL(K)                                                                        \
   hipLaunchKernelGGL((pool_small_kernel<K>), grid, dim3(256), 0, s, x, y, a.in_h, a.in_w, a.c,    \
                      a.out_h, a.out_w, a.stride, a.padding, a.pool_type, (unsigned)total4,        \
