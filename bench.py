@@ -251,6 +251,11 @@ def kernel_table(iters=50, warm=5):
         gg.workspace_dev, gg.workspace_bytes = gws.data_ptr(), need
     row("gemm classifier head (M=16 K=1024 N=1000)", timed(lambda: H.check(L.ogle_hip_gemm(ctypes.byref(gg), st))),
         2.0 * 16 * 1000 * 1024, 4.0 * (16 * 1024 + 1000 * 1024 + 1000 + 16 * 1000), "hbm")
+    # what a launch costs when there is nothing to do: the floor under every small row above
+    # (calls in a row on one stream, as all rows are timed)
+    tiny = H.UnaryArgs(xe.data_ptr(), oe.data_ptr(), 4, H.UNARY_CLIP, 0.0, 6.0, H.F32)
+    row("launch floor: clip on 4 elements", timed(lambda: H.check(L.ogle_hip_unary(ctypes.byref(tiny), st))),
+        0.0, 32.0, "hbm")
     return rows
 
 
