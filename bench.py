@@ -168,6 +168,13 @@ def kernel_table(iters=50, warm=5):
                  b, 38, 38, 256, 256, 3, 1, 1, g=256, act=H.ACT_CLIP, maxv=6.0)
         conv_row("pointwise @C2 b%d (M=%d K=256 N=512)" % (b, b * 1444), "ogle_hip_pwconv_gemm", "mfma",
                  b, 38, 38, 256, 512, 1, 1, 0, act=H.ACT_CLIP, maxv=6.0)
+    # the depthwise layers of the headline pass (C5 at batch 16) with the largest maps
+    conv_row("depthwise 3x3 @C5 b16 block1 (150x150x32)", "ogle_hip_dwconv2d", "hbm",
+             16, 150, 150, 32, 32, 3, 1, 1, g=32, act=H.ACT_CLIP, maxv=6.0)
+    conv_row("depthwise 3x3 s2 @C5 b16 block2 (150x150x64)", "ogle_hip_dwconv2d", "hbm",
+             16, 150, 150, 64, 64, 3, 2, 1, g=64, act=H.ACT_CLIP, maxv=6.0)
+    conv_row("depthwise 3x3 @C5 b16 block3 (75x75x128)", "ogle_hip_dwconv2d", "hbm",
+             16, 75, 75, 128, 128, 3, 1, 1, g=128, act=H.ACT_CLIP, maxv=6.0)
     conv_row("pointwise GEMM @C3 fp32 (M=11552 K=512 N=1024)", "ogle_hip_pwconv_gemm", "mfma",
              32, 19, 19, 512, 1024, 1, 1, 0)
     conv_row("pointwise GEMM @C3 fp16 storage, fp32 accumulate", "ogle_hip_pwconv_gemm", "mfma",
