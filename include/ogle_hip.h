@@ -169,6 +169,26 @@ int32_t ogle_hip_conv2d(const OgleConvArgs* args, ogle_stream_t stream);
  */
 int32_t ogle_hip_conv2d_batch(const OgleConvArgs* args, int32_t count, ogle_stream_t stream);
 
+/*
+ * ogle_hip_conv2d for callers that cannot allocate device memory: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
+ * counterpart in the reference.  Same kernels, same plans and bit-identical results
+ * as ogle_hip_conv2d called with the workspace ogle_hip_conv_workspace_bytes asks
+ * for, but the split-K partial sums go to a fixed array of
+ * OGLE_CONV_NOALLOC_SCRATCH_BYTES inside the library's device image (every GPU the
+ * library runs on holds it until the process ends) instead of a caller buffer.
+ *  - args->workspace_dev must be NULL and workspace_bytes 0.
+ *  - A convolution whose split-K plan needs more than the array holds is refused
+ *    with OGLE_ERR_INVALID_ARG and a message naming both sizes; nothing is launched.
+ *  - The call allocates and frees nothing and does not synchronise.  The array's
+ *    address is looked up at the first call on each device (a symbol lookup, not an
+ *    allocation); make that first call outside a stream capture.
+ *  - All calls on one GPU share the one array: calls that may overlap in time on one
+ *    GPU (different streams, different threads) race.  Calls on one stream are safe.
+ */
+#define OGLE_CONV_NOALLOC_SCRATCH_BYTES (16u << 20)
+int32_t ogle_hip_conv2d_noalloc(const OgleConvArgs* args, ogle_stream_t stream);
+
 /* Depthwise KxK (group == in_c == out_c): conv2d_dw.glsl:38-96,
  * conv2d_dw_any4.glsl:38-98.  Filter layout HWC. */
 int32_t ogle_hip_dwconv2d(const OgleConvArgs* args, ogle_stream_t stream);

@@ -218,6 +218,19 @@ int32_t ogle_hip_conv2d(const OgleConvArgs* a, ogle_stream_t stream) {
   return launch_conv_direct(*a, as_stream(stream));
 }
 
+int32_t ogle_hip_conv2d_noalloc(const OgleConvArgs* a, ogle_stream_t stream) {
+  int32_t st = validate_conv(a, "conv2d_noalloc");
+  if (st != OGLE_OK) return st;
+  if (a->workspace_dev != nullptr || a->workspace_bytes != 0)
+    return fail(OGLE_ERR_INVALID_ARG,
+                "conv2d_noalloc: workspace_dev must be NULL (the scratch is built in)");
+  if (a->group == 1) {
+    st = launch_conv_igemm_static_scratch(*a, as_stream(stream));
+    if (st != OGLE_ERR_UNSUPPORTED) return st;
+  }
+  return launch_conv_direct(*a, as_stream(stream));
+}
+
 int32_t ogle_hip_conv2d_batch(const OgleConvArgs* args, int32_t count, ogle_stream_t stream) {
   if (count < 0 || (count > 0 && args == nullptr))
     return fail(OGLE_ERR_INVALID_ARG, "conv2d_batch: null args or negative count");

@@ -81,6 +81,7 @@ __device__ __forceinline__ int xcd_swizzle(int pid, int grid) {
 // Launchers implemented in the .hip files (host side).
 int32_t launch_conv_igemm(const OgleConvArgs& a, hipStream_t s);   // returns OGLE_ERR_UNSUPPORTED if shape not eligible
 size_t conv_igemm_workspace_bytes(const OgleConvArgs& a);
+int32_t launch_conv_igemm_static_scratch(const OgleConvArgs& a, hipStream_t s);
 int32_t launch_conv_batch(const OgleConvArgs* args, int count, hipStream_t s,
                           int32_t (*fallback)(const OgleConvArgs&, hipStream_t));
 int32_t launch_conv_direct(const OgleConvArgs& a, hipStream_t s);

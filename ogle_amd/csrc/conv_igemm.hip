@@ -26,6 +26,7 @@
 // Result layout of a 32x32 block: register r of lane l holds
 // row 8*(r/4) + 4*(l/32) + r%4, column l%32, so a store instruction writes two
 // 128-byte runs of one output pixel's channels.
+#include <mutex>
 #include <vector>
 
 #include "common.h"
@@ -1169,6 +1170,72 @@ int32_t launch_conv_batch(const OgleConvArgs* args, int count, hipStream_t s,
     if (st != OGLE_OK) return st;
   }
   return OGLE_OK;
+}
+
+// ---------------------------------------------------------------------------
+// Split-K scratch that lives in the library's device image, for callers that may
+// not allocate.  Every GPU the library runs on holds its own copy of the array
+// until the process ends.  In host code the array's name is only a stand-in for the
+// symbol, not a device address: the address on the current device comes from
+// hipGetSymbolAddress, once per device, and only that pointer is handed to kernels.
+static __device__ __align__(256) unsigned char scratch[OGLE_CONV_NOALLOC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+// Address of `scratch` on the current device (resolved at the first call on it).
+int32_t static_scratch(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) {
+    set_error("conv2d_noalloc: hipGetDevice: %s", hipGetErrorString(e));
+    return OGLE_ERR_NO_DEVICE;
+  }
+  if (dev < 0 || dev >= kMaxDevices) {
+    set_error("conv2d_noalloc: device ordinal %d outside 0..%d", dev, kMaxDevices - 1);
+    return OGLE_ERR_UNSUPPORTED;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr) {
+      set_error("conv2d_noalloc: hipGetSymbolAddress(scratch) on device %d: %s", dev,
+                hipGetErrorString(e));
+      return OGLE_ERR_NO_DEVICE;
+    }
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return OGLE_OK;
+}
+}  // namespace
+
+// launch_conv_igemm with the split-K partial sums in the static array.  The split-K
+// kernels write every partial they later read, so nothing has to start at zero.
+int32_t launch_conv_igemm_static_scratch(const OgleConvArgs& a, hipStream_t s) {
+  long m = 0;
+  if (!igemm_eligible(a, &m)) return OGLE_ERR_UNSUPPORTED;  // the other kernels use no scratch
+  const size_t need = plan_igemm(a, m, true).workspace_bytes;
+  if (need > (size_t)OGLE_CONV_NOALLOC_SCRATCH_BYTES) {
+    set_error("conv2d_noalloc: this convolution's split-K plan needs %zu bytes of scratch, the "
+              "built-in buffer holds %zu; use ogle_hip_conv2d with a caller workspace",
+              need, (size_t)OGLE_CONV_NOALLOC_SCRATCH_BYTES);
+    return OGLE_ERR_INVALID_ARG;
+  }
+  OgleConvArgs q = a;
+  q.workspace_dev = nullptr;
+  q.workspace_bytes = 0;
+  if (need > 0) {
+    void* ptr = nullptr;
+    const int32_t st = static_scratch(&ptr);
+    if (st != OGLE_OK) return st;
+    q.workspace_dev = ptr;
+    q.workspace_bytes = (size_t)OGLE_CONV_NOALLOC_SCRATCH_BYTES;
+  }
+  return launch_conv_igemm(q, s);
 }
 
 }  // namespace ogle

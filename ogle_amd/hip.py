@@ -28,7 +28,9 @@ SYMBOLS = [
     "ogle_hip_expf", "ogle_hip_transpose", "ogle_hip_conv_workspace_bytes",
     "ogle_hip_conv2d_batch", "ogle_hip_ssd_topk_nms", "ogle_hip_unary", "ogle_hip_add",
     "ogle_hip_batchnorm", "ogle_hip_gemm", "ogle_hip_gemm_workspace_bytes",
+    "ogle_hip_conv2d_noalloc",
 ]
+CONV_NOALLOC_SCRATCH_BYTES = 16 << 20
 UNARY_RELU, UNARY_CLIP = 0, 1
 
 
@@ -167,6 +169,7 @@ def lib():
         l.ogle_hip_convert.argtypes = [ctypes.c_void_p, ctypes.c_int32, ctypes.c_void_p,
                                        ctypes.c_int32, ctypes.c_int64, ctypes.c_void_p]
         for name, typ in (("ogle_hip_conv2d", ConvArgs), ("ogle_hip_dwconv2d", ConvArgs),
+                          ("ogle_hip_conv2d_noalloc", ConvArgs),
                           ("ogle_hip_pwconv_gemm", ConvArgs), ("ogle_hip_pool2d", PoolArgs),
                           ("ogle_hip_concat", ConcatArgs), ("ogle_hip_ssd_decode", DecodeArgs),
                           ("ogle_hip_ssd_detect", DetectArgs),
