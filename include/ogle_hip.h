@@ -56,7 +56,8 @@ typedef enum OgleAct { OGLE_ACT_NONE = 0, OGLE_ACT_CLIP = 1, OGLE_ACT_RELU = 2 }
 /* How a shader variant reads min/max for the fused activation.
  * NHWC4: conv2d.glsl:82-90 (clamp(x,min,max); relu max(0,x)).
  * PW:    conv2d_pw.glsl:85 (clamp(x,0,max): min ignored).
- * ANY4:  conv2d_any4.glsl:89-94 (relu is max(min,x)). */
+ * ANY4:  conv2d_any4.glsl:89-94, conv2d_dw_any4.glsl:90-97, conv2d_pw_any4.glsl:80-87
+ *        and conv2d_grp.glsl:115-121 (clip (min,max); relu is max(min,x)). */
 typedef enum OgleActVariant {
   OGLE_VARIANT_NHWC4 = 0,
   OGLE_VARIANT_PW = 1,

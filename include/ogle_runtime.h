@@ -17,6 +17,8 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#include "ogle_hip.h"
+
 #ifdef __cplusplus
 extern "C" {
 #endif
@@ -48,6 +50,23 @@ int32_t ogle_rt_compute(OgleSession* s);
 /* The same pass as one captured hipGraph (captured on the first call). */
 int32_t ogle_rt_compute_graph(OgleSession* s);
 int32_t ogle_rt_sync(OgleSession* s);
+/* 1 if graph slot `slot` (0 or 1) holds a recorded pass, 0 if not.  Loading a graph
+ * into a session drops every recorded pass of the previous one. */
+int32_t ogle_rt_graph_captured(OgleSession* s, int32_t slot);
+
+/*
+ * The executor's dependency rule on plain data (touches no device): 1 if a launch that
+ * reads the byte ranges [read_ptrs[i], +read_bytes[i]) and writes [write_ptrs[i],
+ * +write_bytes[i]) must wait for one of the `n_pending` deferred convolutions, i.e. a
+ * read overlaps something one of them writes (output, workspace) or a write overlaps
+ * anything one of them reads or writes; 0 otherwise.  The reference needs no such rule
+ * (one draw per node, in order, fbo_session.cc:140-153); here convolutions are held
+ * back to share grids, and this is what decides when they must go out.
+ */
+int32_t ogle_rt_hazard_conflicts(const OgleConvArgs* pending, int32_t n_pending,
+                                 const void* const* read_ptrs, const size_t* read_bytes,
+                                 int32_t n_reads, const void* const* write_ptrs,
+                                 const size_t* write_bytes, int32_t n_writes);
 
 /*
  * Times `iters` passes (after `warmup` untimed ones) with HIP events recorded on

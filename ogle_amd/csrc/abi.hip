@@ -69,6 +69,20 @@ constexpr int kRegistrySize = sizeof(kRegistry) / sizeof(kRegistry[0]);
 
 bool positive(int v) { return v > 0; }
 
+// Byte extents of a convolution's tensors, and interval overlap of two device ranges.
+size_t elem_bytes(const OgleConvArgs& a) { return a.dtype == OGLE_F16 ? 2 : 4; }
+size_t input_bytes(const OgleConvArgs& a) {
+  return (size_t)a.n * a.in_h * a.in_w * a.in_c * elem_bytes(a);
+}
+size_t output_bytes(const OgleConvArgs& a) {
+  return (size_t)a.n * a.out_h * a.out_w * a.out_c * elem_bytes(a);
+}
+bool overlap(const void* a, size_t a_bytes, const void* b, size_t b_bytes) {
+  if (a == nullptr || b == nullptr || a_bytes == 0 || b_bytes == 0) return false;
+  const uintptr_t a0 = reinterpret_cast<uintptr_t>(a), b0 = reinterpret_cast<uintptr_t>(b);
+  return a0 < b0 + b_bytes && b0 < a0 + a_bytes;
+}
+
 int32_t validate_conv(const OgleConvArgs* a, const char* who) {
   if (a == nullptr) return fail(OGLE_ERR_INVALID_ARG, "null args");
   if (!a->input_dev || !a->filter_dev || !a->output_dev) {
@@ -238,11 +252,19 @@ int32_t ogle_hip_conv2d_batch(const OgleConvArgs* args, int32_t count, ogle_stre
     const int32_t st = validate_conv(&args[i], "conv2d_batch");
     if (st != OGLE_OK) return st;
     for (int j = 0; j < i; ++j) {
-      if (args[i].input_dev == args[j].output_dev || args[j].input_dev == args[i].output_dev ||
-          args[i].output_dev == args[j].output_dev)
+      const OgleConvArgs &p = args[i], &q = args[j];
+      if (overlap(p.input_dev, input_bytes(p), q.output_dev, output_bytes(q)) ||
+          overlap(q.input_dev, input_bytes(q), p.output_dev, output_bytes(p)) ||
+          overlap(p.output_dev, output_bytes(p), q.output_dev, output_bytes(q)))
         return fail(OGLE_ERR_INVALID_ARG, "conv2d_batch: the convolutions depend on each other");
-      if (args[i].workspace_dev != nullptr && args[i].workspace_dev == args[j].workspace_dev)
+      if (overlap(p.workspace_dev, p.workspace_bytes, q.workspace_dev, q.workspace_bytes))
         return fail(OGLE_ERR_INVALID_ARG, "conv2d_batch: two convolutions share one workspace");
+      if (overlap(p.workspace_dev, p.workspace_bytes, q.output_dev, output_bytes(q)) ||
+          overlap(q.workspace_dev, q.workspace_bytes, p.output_dev, output_bytes(p)) ||
+          overlap(p.workspace_dev, p.workspace_bytes, q.input_dev, input_bytes(q)) ||
+          overlap(q.workspace_dev, q.workspace_bytes, p.input_dev, input_bytes(p)))
+        return fail(OGLE_ERR_INVALID_ARG,
+                    "conv2d_batch: a workspace overlaps another convolution's tensor");
     }
   }
   return launch_conv_batch(args, count, as_stream(stream), launch_conv_direct);

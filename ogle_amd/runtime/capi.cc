@@ -73,6 +73,7 @@ void ogle_rt_session_destroy(OgleSession* s) {
 int32_t ogle_rt_load_file(OgleSession* s, const char* path) {
   return (int32_t)Guard([&]() -> int64_t {
     s->session->LoadGraph(std::string(path));
+    s->detector.reset();
     return 0;
   });
 }
@@ -85,8 +86,28 @@ int32_t ogle_rt_load_bytes(OgleSession* s, const void* data, size_t size) {
       return -1;
     }
     s->session->LoadGraph(model);
+    s->detector.reset();  // its device lists belonged to the previous graph's passes
     return 0;
   });
+}
+
+int32_t ogle_rt_graph_captured(OgleSession* s, int32_t slot) {
+  if (s == nullptr || slot < 0 || slot >= FBOSession::kGraphSlots) return -1;
+  return s->session->graph_captured(slot) ? 1 : 0;
+}
+
+int32_t ogle_rt_hazard_conflicts(const OgleConvArgs* pending, int32_t n_pending,
+                                 const void* const* read_ptrs, const size_t* read_bytes,
+                                 int32_t n_reads, const void* const* write_ptrs,
+                                 const size_t* write_bytes, int32_t n_writes) {
+  if (n_pending < 0 || n_reads < 0 || n_writes < 0) return -1;
+  std::vector<opengl::MemRange> reads, writes;
+  for (int i = 0; i < n_reads; ++i) reads.push_back({read_ptrs[i], read_bytes[i]});
+  for (int i = 0; i < n_writes; ++i) writes.push_back({write_ptrs[i], write_bytes[i]});
+  return opengl::Context::Conflicts(pending, n_pending, reads.data(), n_reads, writes.data(),
+                                    n_writes)
+             ? 1
+             : 0;
 }
 
 int32_t ogle_rt_run(OgleSession* s, int32_t n_inputs, const char* const* names,
@@ -316,7 +337,7 @@ int64_t ogle_rt_get_output(OgleSession* s, const char* name, const char* dformat
     opengl::TensorList outs;
     s->session->GetOutputs({name}, {dformat}, &outs);
     std::unique_ptr<Tensor> host(outs[0]);
-    const int64_t n = (int64_t)host->num_elements();
+    const int64_t n = (int64_t)host->AllocatedElements();  // padded for the stride-4 tags
     if (n > capacity) {
       g_error = "output buffer too small";
       return -1;

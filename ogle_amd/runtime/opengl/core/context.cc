@@ -2,6 +2,7 @@
 
 #include <hip/hip_runtime_api.h>
 
+#include <cstring>
 #include <vector>
 
 namespace opengl {
@@ -58,41 +59,58 @@ void* Context::Workspace(size_t bytes) {
 
 namespace {
 size_t ElemBytes(const OgleConvArgs& a) { return a.dtype == OGLE_F16 ? 2 : 4; }
-bool Inside(const void* p, const void* base, size_t bytes) {
-  const char* q = static_cast<const char*>(p);
-  const char* b = static_cast<const char*>(base);
-  return q >= b && q < b + bytes;
+bool Overlap(const MemRange& a, const MemRange& b) {
+  if (a.ptr == nullptr || b.ptr == nullptr || a.bytes == 0 || b.bytes == 0) return false;
+  const uintptr_t a0 = reinterpret_cast<uintptr_t>(a.ptr), b0 = reinterpret_cast<uintptr_t>(b.ptr);
+  return a0 < b0 + b.bytes && b0 < a0 + a.bytes;
 }
 }  // namespace
 
-bool Context::TouchesPending(const void* p, bool written_only) const {
-  if (p == nullptr) return false;
-  for (const OgleConvArgs& c : pending_) {
-    const size_t esz = ElemBytes(c);
-    if (Inside(p, c.output_dev, static_cast<size_t>(c.n) * c.out_h * c.out_w * c.out_c * esz))
-      return true;
-    if (written_only) continue;
-    if (Inside(p, c.input_dev, static_cast<size_t>(c.n) * c.in_h * c.in_w * c.in_c * esz)) return true;
-    if (p == c.filter_dev || p == c.bias_dev) return true;
+void Context::ConvRanges(const OgleConvArgs& c, MemRange reads[3], MemRange writes[2]) {
+  const size_t esz = ElemBytes(c);
+  const int group = c.group > 0 ? c.group : 1;
+  reads[0] = {c.input_dev, static_cast<size_t>(c.n) * c.in_h * c.in_w * c.in_c * esz};
+  reads[1] = {c.filter_dev, static_cast<size_t>(c.out_c) * c.kernel_size * c.kernel_size *
+                                (c.in_c / group) * esz};
+  reads[2] = {c.bias_dev, c.bias_dev != nullptr ? static_cast<size_t>(c.out_c) * sizeof(float) : 0};
+  writes[0] = {c.output_dev, static_cast<size_t>(c.n) * c.out_h * c.out_w * c.out_c * esz};
+  writes[1] = {c.workspace_dev, c.workspace_dev != nullptr ? c.workspace_bytes : 0};
+}
+
+bool Context::Conflicts(const OgleConvArgs* pending, int n_pending, const MemRange* reads,
+                        int n_reads, const MemRange* writes, int n_writes) {
+  for (int p = 0; p < n_pending; ++p) {
+    MemRange pr[3], pw[2];
+    ConvRanges(pending[p], pr, pw);
+    // read after write
+    for (int i = 0; i < n_reads; ++i)
+      for (const MemRange& w : pw)
+        if (Overlap(reads[i], w)) return true;
+    // write after read, write after write
+    for (int i = 0; i < n_writes; ++i) {
+      for (const MemRange& w : pw)
+        if (Overlap(writes[i], w)) return true;
+      for (const MemRange& r : pr)
+        if (Overlap(writes[i], r)) return true;
+    }
   }
   return false;
 }
 
-void Context::BeforeConv(const void* input, const void* filter, const void* bias,
-                         const void* output) {
-  // reads of something a deferred convolution writes; a write into anything one touches
-  if (pending_.size() >= 16 || TouchesPending(input, true) || TouchesPending(filter, true) ||
-      TouchesPending(bias, true) || TouchesPending(output, false))
+void Context::BeforeConv(const OgleConvArgs& args) {
+  if (pending_.empty()) return;
+  MemRange reads[3], writes[2];
+  ConvRanges(args, reads, writes);
+  if (pending_.size() >= 16 ||
+      Conflicts(pending_.data(), static_cast<int>(pending_.size()), reads, 3, writes, 2))
     Flush();
 }
 
-void Context::BeforeLaunch(const void* const* reads, int n_reads, const void* const* writes,
+void Context::BeforeLaunch(const MemRange* reads, int n_reads, const MemRange* writes,
                            int n_writes) {
   if (pending_.empty()) return;
-  bool flush = false;
-  for (int i = 0; i < n_reads && !flush; ++i) flush = TouchesPending(reads[i], true);
-  for (int i = 0; i < n_writes && !flush; ++i) flush = TouchesPending(writes[i], false);
-  if (flush) Flush();
+  if (Conflicts(pending_.data(), static_cast<int>(pending_.size()), reads, n_reads, writes, n_writes))
+    Flush();
 }
 
 void Context::EnqueueConv(const OgleConvArgs& args) {
@@ -149,6 +167,42 @@ void Permute4(const float* src, float* dst, const IntList& nhwc, bool to_nhwc = 
 bool IsImageTag(DataFormat f) {
   return f == dlxnet::TensorProto::NHWC4 || f == dlxnet::TensorProto::NHWC;
 }
+bool IsPaddedTag(DataFormat f) {
+  return f == dlxnet::TensorProto::NHWC4 || f == dlxnet::TensorProto::ANY4 ||
+         f == dlxnet::TensorProto::HWN4C4;
+}
+
+// Dense row-major `dense` (logical shape order) <-> the reference's padded host layout
+// for tag `f` (ogl_runtime/opengl/core/tensor_format.cc:272-343,
+// core/cpu_functor.cc:10-127): NHWC4 and ANY4 pad the last dimension to a multiple
+// of 4 (for NHWC4 that is the texel row (w*C4 + c/4, n*H + h), lane c%4, read row by
+// row); HWN4C4 places OIHW element (o, i, ky, kx) at texel x = i,
+// y = (ky*kw + kx)*ceil(O/4) + o/4, lane o%4, rows ceil(I/4)*4 texels wide.
+void PaddedIndexWalk(const IntList& shape, DataFormat f, float* dense, float* padded, bool to_padded) {
+  size_t n = 1;
+  for (int d : shape) n *= static_cast<size_t>(d);
+  if (f == dlxnet::TensorProto::HWN4C4) {
+    CHECK_EQ(shape.size(), 4u);
+    const size_t O = shape[0], I = shape[1], kh = shape[2], kw = shape[3];
+    const size_t o4 = (O + 3) / 4, width = (I + 3) / 4 * 4;
+    for (size_t o = 0; o < O; ++o)
+      for (size_t i = 0; i < I; ++i)
+        for (size_t t = 0; t < kh * kw; ++t) {
+          const size_t di = ((t * o4 + o / 4) * width + i) * 4 + o % 4;
+          const size_t si = (o * I + i) * kh * kw + t;
+          if (to_padded) padded[di] = dense[si];
+          else dense[si] = padded[di];
+        }
+    return;
+  }
+  if (shape.empty() || shape.back() == 0) return;
+  const size_t last = static_cast<size_t>(shape.back()), last4 = (last + 3) / 4 * 4;
+  for (size_t i = 0; i < n; ++i) {
+    const size_t di = i / last * last4 + i % last;
+    if (to_padded) padded[di] = dense[i];
+    else dense[i] = padded[di];
+  }
+}
 }  // namespace
 
 void Context::CopyCPUTensorToDevice(const Tensor* cpu, Tensor* dev) {
@@ -159,6 +213,15 @@ void Context::CopyCPUTensorToDevice(const Tensor* cpu, Tensor* dev) {
   if (bytes == 0) return;
   Flush();
   hipStream_t s = static_cast<hipStream_t>(stream());
+  if (IsPaddedTag(cpu->dformat()) && cpu->AllocatedSize() != bytes) {
+    // a host tensor in one of the reference's padded layouts: strip the padding
+    std::vector<float> dense(cpu->num_elements());
+    PaddedIndexWalk(cpu->shape(), cpu->dformat(), dense.data(), cpu->host<float>(), false);
+    OGLE_HIP_CALL(hipMemcpyAsync(dev->device_ptr(), dense.data(), bytes, hipMemcpyHostToDevice, s));
+    OGLE_HIP_CALL(hipStreamSynchronize(s));
+    dev->set_initialized(true);
+    return;
+  }
   // The host tensor's element order is the device's: NHWC images, ANY tensors and
   // filters in the file's OIHW order are all dense row-major over shape().
   OGLE_HIP_CALL(hipMemcpyAsync(dev->device_ptr(), cpu->host(), bytes, hipMemcpyHostToDevice, s));
@@ -177,7 +240,20 @@ void Context::CopyDeviceTensorToCPU(const Tensor* dev, Tensor* cpu) {
     OGLE_HIP_CALL(hipStreamSynchronize(s));
     return;
   }
-  if (cpu->dformat() == dlxnet::TensorProto::NCHW && IsImageTag(dev->dformat())) {
+  if (IsPaddedTag(cpu->dformat())) {
+    // "NHWC4" / "ANY4" / "HWN4C4": the caller gets the reference's padded layout,
+    // padding lanes zero (the texture upload shaders write zeros there,
+    // any_to_nhwc4.glsl:44-52).  HWN4C4 is only meaningful for an OIHW filter, NHWC4
+    // for a rank-4 tensor; HostElements checked the rank when `cpu` was made.
+    if (cpu->dformat() == dlxnet::TensorProto::HWN4C4)
+      CHECK(dev->dformat() == dlxnet::TensorProto::HWN4C4)
+          << "HWN4C4 readback of a tensor that is not a filter (" << FormatToStr(dev->dformat()) << ")";
+    std::vector<float> dense(dev->num_elements());
+    OGLE_HIP_CALL(hipMemcpyAsync(dense.data(), dev->device_ptr(), bytes, hipMemcpyDeviceToHost, s));
+    OGLE_HIP_CALL(hipStreamSynchronize(s));
+    std::memset(cpu->host(), 0, cpu->AllocatedSize());
+    PaddedIndexWalk(dev->shape(), cpu->dformat(), dense.data(), cpu->host<float>(), true);
+  } else if (cpu->dformat() == dlxnet::TensorProto::NCHW && IsImageTag(dev->dformat())) {
     CHECK_EQ(dev->dims_size(), 4);
     std::vector<float> tmp(dev->num_elements());
     OGLE_HIP_CALL(hipMemcpyAsync(tmp.data(), dev->device_ptr(), bytes, hipMemcpyDeviceToHost, s));
@@ -209,61 +285,86 @@ void Program::Check(int32_t status, const char* what) const {
 }
 void Program::RunConv2d(const OgleConvArgs& a) const { context_->EnqueueConv(a); }
 void Program::RunDepthwise(const OgleConvArgs& a) const {
-  const void* reads[] = {a.input_dev, a.filter_dev, a.bias_dev};
-  const void* writes[] = {a.output_dev};
-  context_->BeforeLaunch(reads, 3, writes, 1);
+  MemRange reads[3], writes[2];
+  Context::ConvRanges(a, reads, writes);
+  context_->BeforeLaunch(reads, 3, writes, 2);
   Check(ogle_hip_dwconv2d(&a, context_->stream()), "ogle_hip_dwconv2d");
 }
 void Program::RunPointwise(const OgleConvArgs& a) const {
   // the pointwise attribute rules (conv2d.cc:37) were checked by SelectKernel
   context_->EnqueueConv(a);
 }
+namespace {
+size_t DtypeBytes(int32_t dtype) { return dtype == OGLE_F16 ? 2 : 4; }
+}  // namespace
 void Program::RunPool(const OglePoolArgs& a) const {
-  const void* reads[] = {a.input_dev};
-  const void* writes[] = {a.output_dev};
+  const size_t esz = DtypeBytes(a.dtype);
+  const MemRange reads[] = {{a.input_dev, static_cast<size_t>(a.n) * a.in_h * a.in_w * a.c * esz}};
+  const MemRange writes[] = {{a.output_dev, static_cast<size_t>(a.n) * a.out_h * a.out_w * a.c * esz}};
   context_->BeforeLaunch(reads, 1, writes, 1);
   Check(ogle_hip_pool2d(&a, context_->stream()), "ogle_hip_pool2d");
 }
 void Program::RunConcat(const OgleConcatArgs& a) const {
-  const void* writes[] = {a.output_dev};
-  context_->BeforeLaunch(a.inputs_dev, a.n_inputs, writes, 1);
+  const size_t esz = DtypeBytes(a.dtype);
+  MemRange reads[OGLE_CONCAT_MAX_INPUTS];
+  int64_t total = 0;
+  for (int i = 0; i < a.n_inputs; ++i) {
+    reads[i] = {a.inputs_dev[i], static_cast<size_t>(a.outer * a.axis_len[i] * a.inner) * esz};
+    total += a.axis_len[i];
+  }
+  const MemRange writes[] = {{a.output_dev, static_cast<size_t>(a.outer * total * a.inner) * esz}};
+  context_->BeforeLaunch(reads, a.n_inputs, writes, 1);
   Check(ogle_hip_concat(&a, context_->stream()), "ogle_hip_concat");
 }
 void Program::RunDecode(const OgleDecodeArgs& a) const {
-  const void* reads[] = {a.prediction_dev, a.anchors_dev};
-  const void* writes[] = {a.boxes_dev};
+  const size_t boxes = static_cast<size_t>(a.batch) * a.priors * 4 * sizeof(float);
+  const size_t anchors = a.anchors_batch_stride != 0 ? boxes : static_cast<size_t>(a.priors) * 4 * sizeof(float);
+  const MemRange reads[] = {{a.prediction_dev, boxes}, {a.anchors_dev, anchors}};
+  const MemRange writes[] = {{a.boxes_dev, boxes}};
   context_->BeforeLaunch(reads, 2, writes, 1);
   Check(ogle_hip_ssd_decode(&a, context_->stream()), "ogle_hip_ssd_decode");
 }
 void Program::RunTranspose(const OgleTransposeArgs& a) const {
-  const void* reads[] = {a.input_dev};
-  const void* writes[] = {a.output_dev};
+  size_t bytes = DtypeBytes(a.dtype);
+  for (int d = 0; d < 4; ++d) bytes *= static_cast<size_t>(a.in_shape[d]);
+  const MemRange reads[] = {{a.input_dev, bytes}};
+  const MemRange writes[] = {{a.output_dev, bytes}};
   context_->BeforeLaunch(reads, 1, writes, 1);
   Check(ogle_hip_transpose(&a, context_->stream()), "ogle_hip_transpose");
 }
 
 void Program::RunUnary(const OgleUnaryArgs& a) const {
-  const void* reads[] = {a.input_dev};
-  const void* writes[] = {a.output_dev};
+  const size_t bytes = static_cast<size_t>(a.count) * DtypeBytes(a.dtype);
+  const MemRange reads[] = {{a.input_dev, bytes}};
+  const MemRange writes[] = {{a.output_dev, bytes}};
   context_->BeforeLaunch(reads, 1, writes, 1);
   Check(ogle_hip_unary(&a, context_->stream()), "ogle_hip_unary");
 }
 void Program::RunAdd(const OgleBinaryArgs& a) const {
-  const void* reads[] = {a.a_dev, a.b_dev};
-  const void* writes[] = {a.output_dev};
+  const size_t bytes = static_cast<size_t>(a.count) * DtypeBytes(a.dtype);
+  const MemRange reads[] = {{a.a_dev, bytes}, {a.b_dev, bytes}};
+  const MemRange writes[] = {{a.output_dev, bytes}};
   context_->BeforeLaunch(reads, 2, writes, 1);
   Check(ogle_hip_add(&a, context_->stream()), "ogle_hip_add");
 }
 void Program::RunBatchNorm(const OgleBatchNormArgs& a) const {
-  const void* reads[] = {a.input_dev, a.gamma_dev, a.beta_dev, a.mean_dev, a.var_dev};
-  const void* writes[] = {a.output_dev};
+  const size_t bytes = static_cast<size_t>(a.outer) * a.channels * DtypeBytes(a.dtype);
+  const size_t vec = static_cast<size_t>(a.channels) * sizeof(float);
+  const MemRange reads[] = {{a.input_dev, bytes}, {a.gamma_dev, vec}, {a.beta_dev, vec},
+                            {a.mean_dev, vec}, {a.var_dev, vec}};
+  const MemRange writes[] = {{a.output_dev, bytes}};
   context_->BeforeLaunch(reads, 5, writes, 1);
   Check(ogle_hip_batchnorm(&a, context_->stream()), "ogle_hip_batchnorm");
 }
 void Program::RunGemm(const OgleGemmArgs& a) const {
-  const void* reads[] = {a.a_dev, a.b_dev, a.c_dev};
-  const void* writes[] = {a.y_dev};
-  context_->BeforeLaunch(reads, 3, writes, 1);
+  const size_t f = sizeof(float);
+  const size_t c_bytes = a.c_dev == nullptr ? 0 : (a.c_rank == 2 ? static_cast<size_t>(a.m) * a.n : static_cast<size_t>(a.n)) * f;
+  const MemRange reads[] = {{a.a_dev, static_cast<size_t>(a.m) * a.k * f},
+                            {a.b_dev, static_cast<size_t>(a.k) * a.n * f},
+                            {a.c_dev, c_bytes}};
+  const MemRange writes[] = {{a.y_dev, static_cast<size_t>(a.m) * a.n * f},
+                             {a.workspace_dev, a.workspace_dev != nullptr ? a.workspace_bytes : 0}};
+  context_->BeforeLaunch(reads, 3, writes, 2);
   Check(ogle_hip_gemm(&a, context_->stream()), "ogle_hip_gemm");
 }
 

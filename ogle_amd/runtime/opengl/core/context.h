@@ -14,6 +14,12 @@
 
 namespace opengl {
 
+// A byte range of device memory, [ptr, ptr + bytes).
+struct MemRange {
+  const void* ptr;
+  size_t bytes;
+};
+
 class Context {
  public:
   Context();
@@ -46,12 +52,23 @@ class Context {
   // Deferred convolutions.  Dense and pointwise Conv nodes are not launched one by
   // one: they are collected and go out through ogle_hip_conv2d_batch, so that
   // mutually independent convolutions (the SSD heads next to the feature-extractor
-  // chain) share a grid.  A batch is launched as soon as anything depends on it:
-  // BeforeConv flushes if the coming convolution touches a deferred one's buffers (or
-  // the batch is full), BeforeLaunch does the same for any other kernel given the
-  // buffers it reads and writes; copies and waits always flush.
-  void BeforeConv(const void* input, const void* filter, const void* bias, const void* output);
-  void BeforeLaunch(const void* const* reads, int n_reads, const void* const* writes, int n_writes);
+  // chain) share a grid.  A batch is launched as soon as anything depends on it.
+  // Dependencies are found by byte-range overlap: every launch names the [ptr, ptr +
+  // bytes) ranges it reads and writes, and a range that overlaps what a deferred
+  // convolution writes (or, for a write, anything it reads or writes: input, filter,
+  // bias, output, workspace) launches the batch first.  A buffer that merely encloses a
+  // deferred convolution's output (a concat output whose slices the convolutions write
+  // in place) is therefore seen, wherever it starts.  BeforeConv does this for the
+  // coming convolution (and also launches a full batch), BeforeLaunch for any other
+  // kernel; copies and waits always flush.
+  void BeforeConv(const OgleConvArgs& args);
+  void BeforeLaunch(const MemRange* reads, int n_reads, const MemRange* writes, int n_writes);
+  // The overlap rule itself, on plain data (no device needed): true if a launch with
+  // these reads and writes must wait for one of `pending`.
+  static bool Conflicts(const OgleConvArgs* pending, int n_pending, const MemRange* reads,
+                        int n_reads, const MemRange* writes, int n_writes);
+  // The ranges a convolution reads (input, filter, bias) and writes (output, workspace).
+  static void ConvRanges(const OgleConvArgs& a, MemRange reads[3], MemRange writes[2]);
   void EnqueueConv(const OgleConvArgs& args);
   void Flush();
   void set_batching(bool on) {
@@ -68,9 +85,6 @@ class Context {
   void* workspace_ = nullptr;
   size_t workspace_bytes_ = 0;
   size_t workspace_used_ = 0;
-  // True if `p` lies inside a buffer a deferred convolution writes (`written`) or
-  // reads or writes (`!written`).
-  bool TouchesPending(const void* p, bool written_only) const;
   std::vector<OgleConvArgs> pending_;
   bool batching_ = true;
   std::map<std::string, std::unique_ptr<Program>> programs_;

@@ -51,6 +51,17 @@ void FBOSession::LoadGraph(std::string model_path) {
 }
 
 void FBOSession::LoadGraph(const ::dlxnet::ModelProto& model_proto) {
+  // A session that has already run holds device state that refers to the old graph's
+  // tensors: deferred convolutions, recorded hipGraphs (their kernel arguments are the
+  // old buffers' addresses) and the issue order's Kernel pointers.  All of it goes
+  // before the tensors are released.
+  if (finalized_) context_->Finish();
+  for (int slot = 0; slot < kGraphSlots; ++slot) DropGraph(slot);
+  order_.clear();
+  ready_.clear();
+  finalized_ = false;
+  graph_created_ = false;
+  computed_once_ = false;
   model_ = model_proto;
   kernels_.clear();
   total_tensors_.clear();
@@ -162,6 +173,30 @@ void FBOSession::PlaceInputsInOutputs() {
   for (auto& k : kernels_)
     for (size_t j = 0; j < k->output_tensor_indexes_.size(); ++j)
       producer[k->output_tensor_indexes_[j]] = {k.get(), static_cast<int>(j)};
+  // The allocation a tensor's memory belongs to: the tensor itself, or, for the output of
+  // a node that only re-interprets memory, the root of the input it aliases.
+  auto root_of = [&](int idx) {
+    for (;;) {
+      auto it = producer.find(idx);
+      if (it == producer.end()) return idx;
+      const int alias = it->second.first->OutputAliasesInput(it->second.second);
+      if (alias < 0) return idx;
+      idx = it->second.first->input_tensor_indexes_[alias];
+    }
+  };
+  // True if a node other than `self` computes on the memory of allocation `root`.
+  auto has_other_reader = [&](int root, const Kernel* self) {
+    for (auto& other : kernels_) {
+      if (other.get() == self) continue;
+      bool view = !other->output_tensor_indexes_.empty();
+      for (size_t j = 0; j < other->output_tensor_indexes_.size(); ++j)
+        if (other->OutputAliasesInput(static_cast<int>(j)) < 0) view = false;
+      if (view) continue;  // only passes the memory on; its consumers are looked at themselves
+      for (int in : other->input_tensor_indexes_)
+        if (root_of(in) == root) return true;
+    }
+    return false;
+  };
   std::set<int> placed;
   for (auto& kp : kernels_) {
     Kernel* k = kp.get();
@@ -186,7 +221,11 @@ void FBOSession::PlaceInputsInOutputs() {
       if (!ok) break;
       Tensor* root = total_tensors_[idx].get();
       const uintptr_t place = reinterpret_cast<uintptr_t>(out->device_ptr()) + offsets[i];
-      const bool by_element = pk->kernel_type() == "Conv" && root->shape().back() % 4 != 0;
+      // A place that is only 4-byte aligned suits a convolution that stores element by
+      // element, but every other kernel reads 16-byte vectors from the tensor's start:
+      // the exception holds only if this node is the allocation's sole reader.
+      const bool by_element = pk->kernel_type() == "Conv" && root->shape().back() % 4 != 0 &&
+                              !has_other_reader(idx, k);
       ok = !CheckKernelReady(pk) && root->owns_device_buffer() && placed.count(idx) == 0 &&
            std::find(roots.begin(), roots.end(), idx) == roots.end() &&
            root->num_elements() == k->input_tensors_[i]->num_elements() &&
@@ -366,6 +405,7 @@ void FBOSession::Compute() {
   CHECK(finalized_) << "Please Setup Session First";
   for (Kernel* kernel : order_) kernel->Compute();
   context_->Flush();  // convolutions still deferred at the end of the pass
+  computed_once_ = true;
 }
 
 void FBOSession::Run(const NamedTensorList& inputs_cpu) {
@@ -386,6 +426,7 @@ void FBOSession::RunProfiled(std::vector<NodeTiming>* timings) {
     OGLE_HIP_CALL(hipEventRecord(ev[i + 1], s));
   }
   OGLE_HIP_CALL(hipStreamSynchronize(s));
+  computed_once_ = true;
   timings->clear();
   for (size_t i = 0; i < live.size(); ++i) {
     float ms = 0.f;
@@ -401,6 +442,11 @@ void FBOSession::CaptureGraph(int slot, const std::function<void()>& after_pass)
   CHECK(slot >= 0 && slot < kGraphSlots) << "graph slot";
   if (graph_exec_[slot] != nullptr) return;
   hipStream_t s = static_cast<hipStream_t>(context_->stream());
+  if (!computed_once_) {
+    // The first pass packs filters and may grow the workspace (allocations), which
+    // must not happen inside a capture: make that pass eagerly.
+    Compute();
+  }
   OGLE_HIP_CALL(hipStreamSynchronize(s));
   hipGraph_t graph = nullptr;
   OGLE_HIP_CALL(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal));

@@ -91,6 +91,7 @@ class FBOSession {
   OwnedTensorList total_tensors_;
   bool finalized_ = false;
   bool graph_created_ = false;
+  bool computed_once_ = false;  // a full eager pass has run since the graph was loaded
   NamedIndex tensor_name_index_;
   std::vector<bool> ready_;
   bool allow_resized_ = false;

@@ -35,6 +35,9 @@ Tensor::Tensor(DataType dtype, IntList shape, MemoryType mem_type, DataFormat df
   }
   requested_size_ = num_elements() * ElementSize(dtype_);
   allocated_size_ = requested_size_;
+  // Host tensors with a stride-4 tag hold the reference's padded layout (what
+  // GetOutputs hands back for "NHWC4" / "ANY4" / "HWN4C4"); device tensors are dense.
+  if (mem_type_ == HOST_MEMORY) allocated_size_ = HostElements(shape_, dformat_) * ElementSize(dtype_);
   const size_t bytes = allocated_size_ > 0 ? allocated_size_ : 16;
   if (mem_type_ == HOST_MEMORY) {
     host_ = std::malloc(bytes);
@@ -107,6 +110,7 @@ Tensor* Tensor::Empty(DataType dtype, IntList shape, DataFormat dformat) {
 Tensor* Tensor::Random(DataType dtype, IntList shape, DataFormat dformat) {
   Tensor* t = Empty(dtype, shape, dformat);
   CHECK_EQ(dtype, DT_FLOAT);
+  CHECK_EQ(t->AllocatedSize(), t->RequestedSize()) << "Random fills dense host tensors only";
   float* p = t->host<float>();
   // Uniform in [0, 1) from libc random(), as tensor.cc:105-114 of the reference.
   for (size_t i = 0; i < t->num_elements(); ++i)
@@ -118,6 +122,7 @@ Tensor* Tensor::Random(DataType dtype, IntList shape, DataFormat dformat) {
 Tensor* Tensor::Ones(DataType dtype, IntList shape, DataFormat dformat) {
   Tensor* t = Empty(dtype, shape, dformat);
   CHECK_EQ(dtype, DT_FLOAT);
+  CHECK_EQ(t->AllocatedSize(), t->RequestedSize()) << "Ones fills dense host tensors only";
   float* p = t->host<float>();
   for (size_t i = 0; i < t->num_elements(); ++i) p[i] = 1.0f;
   t->initialized_ = true;
@@ -183,6 +188,27 @@ std::string Tensor::DebugString() const {
     if (n < num_elements()) ss << " ...";
   }
   return ss.str();
+}
+
+size_t HostElements(const IntList& shape, DataFormat dformat) {
+  size_t n = 1;
+  for (int d : shape) n *= static_cast<size_t>(d);
+  const auto up4 = [](size_t v) { return (v + 3) / 4 * 4; };
+  switch (dformat) {
+    case dlxnet::TensorProto::ANY4: {
+      if (shape.empty() || shape.back() == 0) return n;
+      const size_t last = static_cast<size_t>(shape.back());
+      return n / last * up4(last);
+    }
+    case dlxnet::TensorProto::NHWC4:
+      CHECK_EQ(shape.size(), 4u) << "NHWC4 needs a rank-4 shape";
+      return static_cast<size_t>(shape[0]) * shape[1] * shape[2] * up4(shape[3]);
+    case dlxnet::TensorProto::HWN4C4:
+      CHECK_EQ(shape.size(), 4u) << "HWN4C4 needs an OIHW shape";
+      return static_cast<size_t>(shape[2]) * shape[3] * ((shape[0] + 3) / 4) * up4(shape[1]) * 4;
+    default:
+      return n;
+  }
 }
 
 DataFormat StrToFormat(const std::string& s) {

@@ -38,7 +38,7 @@ class Tensor {
   Tensor(DataType dtype, IntList shape, const T* data,
          DataFormat dformat = dlxnet::TensorProto::NHWC)
       : Tensor(dtype, shape, HOST_MEMORY, dformat) {
-    std::memcpy(host_, data, num_elements() * sizeof(T));
+    std::memcpy(host_, data, allocated_size_);  // `data` is in `dformat`'s host layout
     initialized_ = true;
   }
   // Host tensor from a model constant (float_data, int32_data or int64_data are all
@@ -108,6 +108,15 @@ class Tensor {
   IntList shape_;
   DataFormat dformat_;
 };
+
+// Elements (floats) a HOST tensor of this shape and tag occupies.  Dense for NHWC, NCHW
+// and ANY; for the stride-4 tags the reference's padded texture layouts
+// (ogl_runtime/opengl/core/tensor_format.cc:251-298): NHWC4 pads the channels of every
+// pixel to a multiple of 4, ANY4 the last dimension, HWN4C4 (OIHW filters) is
+// kh*kw*ceil(O/4) rows of ceil(I/4)*4 texels of 4 output channels.  The reference
+// further rounds sizes above GL_MAX_TEXTURE_SIZE*4 elements up to whole texture rows;
+// there is no texture here, so that rounding is not applied.
+size_t HostElements(const IntList& shape, DataFormat dformat);
 
 // "NHWC", "NCHW", "ANY", "NHWC4", "HWN4C4", "ANY4" <-> DataFormat
 // (ogl_runtime/opengl/core/tensor_format.cc:136-152).

@@ -63,7 +63,11 @@ void Conv2DKernel::SelectKernel(const TensorList& inputs) {
     variant_ = kDense;
     kernel_fname_ = any4 ? "conv2d_any4" : "conv2d";
   }
-  act_variant_ = any4 ? OGLE_VARIANT_ANY4 : (variant_ == kPointwise ? OGLE_VARIANT_PW : OGLE_VARIANT_NHWC4);
+  // How the fused activation reads min / max differs per shader: conv2d_pw.glsl:85 clamps
+  // to (0, max); the *_any4 shaders and conv2d_grp.glsl:115-121 use max(min, x) for Relu
+  // and (min, max) for Clip; conv2d.glsl / conv2d_dw.glsl use max(0, x) and (min, max).
+  if (any4 || variant_ == kGrouped) act_variant_ = OGLE_VARIANT_ANY4;
+  else act_variant_ = variant_ == kPointwise ? OGLE_VARIANT_PW : OGLE_VARIANT_NHWC4;
 
   if (input_tensor_indexes_.size() == 3) build_options_ += "#define USE_BIAS\n";
   if (activation_type_ == "Clip") {
@@ -156,8 +160,7 @@ void Conv2DKernel::Compute(TensorList& inputs, TensorList& outputs) {
   a.filter_dev = packed_filter_->device_ptr();
   a.bias_dev = inputs.size() > 2 ? static_cast<const float*>(inputs[2]->device_ptr()) : nullptr;
   a.output_dev = outputs[0]->device_ptr();
-  if (variant_ != kDepthwise)
-    context_->BeforeConv(a.input_dev, a.filter_dev, a.bias_dev, a.output_dev);
+  if (variant_ != kDepthwise) context_->BeforeConv(a);
   if (workspace_need_ < 0) workspace_need_ = static_cast<long>(ogle_hip_conv_workspace_bytes(&a));
   if (workspace_need_ > 0) {
     a.workspace_dev = context_->Workspace(static_cast<size_t>(workspace_need_));

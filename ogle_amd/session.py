@@ -24,7 +24,7 @@ SYMBOLS = [
     "ogle_rt_registered_kernel_count", "ogle_rt_registered_kernel_name", "ogle_rt_detect",
     "ogle_rt_reserialize", "ogle_rt_model_debug_string", "ogle_rt_tensor_dformat",
     "ogle_rt_set_reorder", "ogle_rt_issue_order_name", "ogle_rt_set_device_nms",
-    "ogle_rt_detect_results",
+    "ogle_rt_detect_results", "ogle_rt_graph_captured", "ogle_rt_hazard_conflicts",
 ]
 
 
@@ -61,6 +61,10 @@ def lib():
         l.ogle_rt_compute.argtypes = [vp]
         l.ogle_rt_compute_graph.argtypes = [vp]
         l.ogle_rt_sync.argtypes = [vp]
+        l.ogle_rt_graph_captured.argtypes = [vp, i32]
+        l.ogle_rt_hazard_conflicts.argtypes = [
+            ctypes.POINTER(_hip.ConvArgs), i32, ctypes.POINTER(vp), ctypes.POINTER(ctypes.c_size_t),
+            i32, ctypes.POINTER(vp), ctypes.POINTER(ctypes.c_size_t), i32]
         l.ogle_rt_time_compute.argtypes = [vp, i32, i32, i32, i32, i32,
                                            ctypes.POINTER(ctypes.c_float),
                                            ctypes.POINTER(ctypes.c_float)]
@@ -124,6 +128,23 @@ def model_debug_string(model_bytes):
     return dst.value.decode()
 
 
+def hazard_conflicts(pending, reads, writes):
+    """The executor's dependency rule on plain numbers (no device): `pending` is a list of
+    hip.ConvArgs (deferred convolutions), `reads` / `writes` lists of (address, bytes).
+    True if the launch must wait for one of them."""
+    arr = (_hip.ConvArgs * max(1, len(pending)))(*pending)
+
+    def split(ranges):
+        n = max(1, len(ranges))
+        ptrs = (ctypes.c_void_p * n)(*[r[0] for r in ranges])
+        sizes = (ctypes.c_size_t * n)(*[r[1] for r in ranges])
+        return ptrs, sizes
+    rp, rb = split(reads)
+    wp, wb = split(writes)
+    return bool(_check(lib().ogle_rt_hazard_conflicts(arr, len(pending), rp, rb, len(reads), wp, wb,
+                                                      len(writes))))
+
+
 def registered_kernels():
     l = lib()
     return [l.ogle_rt_registered_kernel_name(i).decode()
@@ -178,24 +199,29 @@ class Session:
         else:
             _check(lib().ogle_rt_load_file(self._h, str(model).encode()))
 
-    def run(self, inputs, dformats=None):
+    def run(self, inputs, dformats=None, shapes=None):
         """inputs: {name: float32 ndarray}; dformats: {name: "NHWC"|"NCHW"|"ANY"} (default NHWC
-        for rank 4, ANY otherwise)."""
+        for rank 4, ANY otherwise).  An input in one of the padded layouts ("NHWC4", "ANY4")
+        also needs its logical shape in `shapes`."""
         names = list(inputs)
         arrs = [np.ascontiguousarray(inputs[n], dtype=np.float32) for n in names]
         n = len(names)
         c_names = (ctypes.c_char_p * n)(*[s.encode() for s in names])
         c_data = (ctypes.c_void_p * n)(*[a.ctypes.data for a in arrs])
-        dims = [(ctypes.c_int32 * a.ndim)(*a.shape) for a in arrs]
+        logical = [tuple((shapes or {}).get(nm, a.shape)) for nm, a in zip(names, arrs)]
+        dims = [(ctypes.c_int32 * len(sh))(*sh) for sh in logical]
         c_dims = (ctypes.POINTER(ctypes.c_int32) * n)(
             *[ctypes.cast(d, ctypes.POINTER(ctypes.c_int32)) for d in dims])
-        c_ranks = (ctypes.c_int32 * n)(*[a.ndim for a in arrs])
+        c_ranks = (ctypes.c_int32 * n)(*[len(sh) for sh in logical])
         fm = [(dformats or {}).get(nm, "NHWC" if a.ndim == 4 else "ANY") for nm, a in zip(names, arrs)]
         c_fm = (ctypes.c_char_p * n)(*[f.encode() for f in fm])
         _check(lib().ogle_rt_run(self._h, n, c_names, c_data, c_dims, c_ranks, c_fm))
 
     def compute(self, graph=False):
         _check(lib().ogle_rt_compute_graph(self._h) if graph else lib().ogle_rt_compute(self._h))
+
+    def graph_captured(self, slot=0):
+        return bool(_check(lib().ogle_rt_graph_captured(self._h, slot)))
 
     def sync(self):
         _check(lib().ogle_rt_sync(self._h))
@@ -283,6 +309,13 @@ class Session:
     def get_output(self, name, dformat="ANY"):
         shape = self.tensor_shape(name)
         out = np.empty(shape, np.float32)
+        up4 = lambda v: (v + 3) // 4 * 4
+        if dformat in ("NHWC4", "ANY4") and len(shape) > 0:
+            # the reference's padded host layouts: last dimension padded to a multiple of 4
+            out = np.empty(tuple(shape[:-1]) + (up4(shape[-1]),), np.float32)
+        elif dformat == "HWN4C4" and len(shape) == 4:
+            o, i, kh, kw = shape  # an OIHW filter: (kh*kw*ceil(O/4), ceil(I/4)*4, 4) texels
+            out = np.empty((kh * kw * ((o + 3) // 4), up4(i), 4), np.float32)
         if dformat == "NCHW" and len(shape) == 4 and self.tensor_dformat(name) in ("NHWC", "NHWC4"):
             out = np.empty((shape[0], shape[3], shape[1], shape[2]), np.float32)
         n = _check(lib().ogle_rt_get_output(self._h, name.encode(), dformat.encode(),

@@ -46,9 +46,10 @@
 /* Shader variants differ only in how the fused activation reads min/max
  * (RT/nn/glsl/conv2d.glsl:82-90, conv2d_pw.glsl:82-90,
  * conv2d_any4.glsl:89-94). */
-#define ORACLE_VARIANT_NHWC4 0 /* conv2d.glsl, conv2d_dw.glsl, conv2d_grp.glsl */
+#define ORACLE_VARIANT_NHWC4 0 /* conv2d.glsl, conv2d_dw.glsl                  */
 #define ORACLE_VARIANT_PW 1    /* conv2d_pw.glsl: clamp(x, 0, max)            */
-#define ORACLE_VARIANT_ANY4 2  /* *_any4.glsl: relu is max(min_value, x)      */
+#define ORACLE_VARIANT_ANY4 2  /* *_any4.glsl and conv2d_grp.glsl:115-121:
+                                  relu is max(min_value, x)                   */
 
 static inline float oracle_activation(float v, int act, float minv, float maxv,
                                       int variant) {

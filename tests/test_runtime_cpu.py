@@ -214,3 +214,62 @@ def test_fold_batchnorm_is_the_bn_of_the_conv():
     wo, bo = O.fold_bn(w, None, gamma, beta, mean, var, 1e-5)
     np.testing.assert_allclose(wf, wo, rtol=2e-7, atol=0)
     np.testing.assert_allclose(bf, bo, rtol=0, atol=1e-7)
+
+
+# ---- dependency rule of the deferred-convolution queue (no device) --------------------
+
+def _fake_conv(inp, out, n=1, h=4, w=4, c=8, o=16, k=1, ws=0, ws_bytes=0, filt=0x10000, bias=0x20000):
+    from ogle_amd import hip as H
+    a = H.conv_args(inp, filt, bias, out, n, h, w, c, o, k)
+    a.workspace_dev, a.workspace_bytes = (ws or None), ws_bytes
+    return a
+
+
+def test_hazard_rule_is_interval_overlap():
+    """Two deferred convolutions write slices at non-zero offsets inside one larger buffer
+    (what placing concat inputs in the concat output produces).  Readers and writers are
+    given as byte ranges; the rule must see every overlap, wherever the range starts."""
+    big = 0x1000000                      # the enclosing buffer (a concat output), 4 KiB
+    out_bytes = 4 * 4 * 16 * 4           # 1 KiB per convolution output
+    pend = [_fake_conv(0x5000000, big + 1024), _fake_conv(0x6000000, big + 2048, ws=0x7000000, ws_bytes=512)]
+    C = session.hazard_conflicts
+    # a reader of the whole enclosing buffer starts BEFORE both pending outputs
+    assert C(pend, [(big, 4096)], [])
+    # a reader that straddles the start of a pending output
+    assert C(pend, [(big + 512, 600)], [])
+    # the in-place concat slice itself, and a range that ends exactly where an output begins
+    assert C(pend, [(big + 2048, out_bytes)], [])
+    assert not C(pend, [(big, 1024)], [])
+    assert not C(pend, [(big + 3072, 1024)], [])
+    # reading what a pending convolution only reads is no hazard; writing it is
+    assert not C(pend, [(0x5000000, 512)], [])
+    assert C(pend, [], [(0x5000000 + 500, 8)])
+    assert C(pend, [], [(0x10000 + 4, 4)])          # inside a pending filter
+    assert C(pend, [], [(0x20000, 4)])              # a pending bias
+    # workspace of a pending convolution: reads and writes both conflict
+    assert C(pend, [(0x7000000 + 100, 4)], [])
+    assert C(pend, [], [(0x7000000 + 511, 1)])
+    assert not C(pend, [], [(0x7000000 + 512, 64)])
+    # write-after-write into the enclosing buffer
+    assert C(pend, [], [(big, 4096)])
+    # empty ranges and null pointers never conflict; nothing pending never conflicts
+    assert not C(pend, [(big + 1024, 0), (0, 100)], [(0, 8)])
+    assert not C([], [(big, 4096)], [(big, 4096)])
+
+
+def test_reloading_a_graph_resets_the_session():
+    """LoadGraph on a session that already holds a graph starts from scratch: kernel count
+    follows the new graph and no recorded pass survives (checked on the device as well)."""
+    g1, _ = models.separable_block(1, size=8, cin=8, cout=16)
+    sess = session.Session()
+    sess.load_graph(g1)
+    n1 = sess.num_kernels
+    gb = dlx.GraphBuilder()
+    x = gb.add_input("input", [1, 4, 6, 6])
+    gb.add_pool("output", x, "MaxPool", 2, 2, 0)
+    sess.load_graph(gb)
+    assert sess.num_kernels == 1 and n1 > 1
+    assert not sess.graph_captured(0) and not sess.graph_captured(1)
+    assert sess.issue_order() == []
+    sess.load_graph(g1)
+    assert sess.num_kernels == n1

@@ -466,3 +466,159 @@ def test_batch16_images_match_their_batch1_passes():
             got = sess1.get_output(name, "ANY" if name != "block13.pw" else "NHWC")
             scale = float(np.abs(ref[i]).max())
             assert np.abs(got[0] - ref[i]).max() <= 1e-4 * scale, (name, i)
+
+
+# ---- ANY / ANY4 inputs, activation rules, padded readback, reload -----------------------
+
+ANY_INPUT_CASES = [
+    # n, h, w, c, o, k, s, p, g, bias, act, minv, maxv
+    (1, 2, 2, 1, 1, 3, 1, 1, 1, False, "", 0.0, 0.0),         # conv2d_test.cc:220-234 as written
+    (2, 9, 9, 8, 12, 3, 1, 1, 1, True, "Relu", -0.5, 0.0),    # conv2d_any4: relu is max(min, x)
+    (1, 7, 7, 16, 16, 3, 1, 1, 16, True, "Clip", 0.25, 2.0),  # conv2d_dw_any4: clip (min, max)
+    (2, 5, 5, 32, 24, 1, 1, 0, 1, True, "Clip", 0.25, 2.0),   # conv2d_pw_any4: min is NOT ignored
+    (2, 5, 5, 32, 24, 1, 1, 0, 1, True, "Relu", -0.5, 0.0),
+]
+
+
+@pytest.mark.parametrize("case", ANY_INPUT_CASES)
+def test_conv_on_any_input_selects_the_any4_variant(case):
+    """An ANY host input becomes an ANY4 device tensor and Conv then takes the *_any4 shader
+    (conv2d.cc:44-61), whose fused activation reads min / max differently
+    (conv2d_any4.glsl:89-94); the output keeps the input's tag (conv2d.cc:64)."""
+    n, h, w, c, o, k, s, p, g, use_bias, act, minv, maxv = case
+    r = rng(7700 + ANY_INPUT_CASES.index(case))
+    x = r.uniform(-1, 1, (n, h, w, c)).astype(np.float32)
+    wt = r.normal(0, 0.5, (o, c // g, k, k)).astype(np.float32)
+    b = r.uniform(-0.1, 0.1, o).astype(np.float32) if use_bias else None
+    sess = session.Session()
+    sess.load_graph(conv_graph(x.shape, wt, b, k, s, p, 1, g, act, minv, maxv))
+    sess.run({"input": x}, dformats={"input": "ANY"})
+    assert sess.tensor_dformat("input") == "ANY4" and sess.tensor_dformat("output") == "ANY4"
+    got = sess.get_output("output", "ANY")
+    oact = {"": O.ACT_NONE, "Relu": O.ACT_RELU, "Clip": O.ACT_CLIP}[act]
+    ref = O.conv2d(x, wt, b, s, p, 1, g, oact, minv, maxv, O.VARIANT_ANY4)
+    assert_conv_close(got, ref, O.conv2d_abs(x, wt, b, s, p, 1, g), 1e-5, str(case))
+    if act:
+        assert got.min() >= minv and (ref != O.conv2d(x, wt, b, s, p, 1, g, oact, 0.0, maxv,
+                                                       O.VARIANT_PW)).any()
+
+
+def test_grouped_conv_activation_reads_min_like_the_any4_shaders():
+    """conv2d_grp.glsl:115-121: Relu is max(min_value, x), Clip is (min, max)."""
+    r = rng(7750)
+    x = r.uniform(-1, 1, (2, 8, 8, 8)).astype(np.float32)
+    wt = r.normal(0, 0.5, (12, 2, 3, 3)).astype(np.float32)
+    b = r.uniform(-0.1, 0.1, 12).astype(np.float32)
+    for act, oact, minv, maxv in (("Relu", O.ACT_RELU, -0.25, 0.0), ("Clip", O.ACT_CLIP, -0.5, 0.75)):
+        sess = session.Session()
+        sess.load_graph(conv_graph(x.shape, wt, b, 3, 1, 1, 1, 4, act, minv, maxv))
+        sess.run({"input": x})
+        ref = O.conv2d(x, wt, b, 1, 1, 1, 4, oact, minv, maxv, O.VARIANT_ANY4)
+        got = sess.get_output("output", "NHWC")
+        assert_conv_close(got, ref, O.conv2d_abs(x, wt, b, 1, 1, 1, 4), 1e-5, act)
+        assert got.min() == np.float32(minv)
+
+
+def test_get_outputs_in_the_padded_host_layouts():
+    """GetOutputs with "NHWC4" / "ANY4" / "HWN4C4" returns the reference's stride-4 layouts
+    (tensor_format.cc:272-343, cpu_functor.cc:10-127), padding lanes zero; an input handed
+    over in a padded layout is unpadded on upload."""
+    r = rng(7800)
+    x = r.uniform(-1, 1, (2, 5, 4, 6)).astype(np.float32)
+    wt = r.normal(0, 0.5, (7, 6, 3, 3)).astype(np.float32)
+    b = r.uniform(-0.1, 0.1, 7).astype(np.float32)
+    sess = session.Session()
+    sess.load_graph(conv_graph(x.shape, wt, b, 3, 1, 1))
+    sess.run({"input": x})
+    dense = sess.get_output("output", "NHWC")
+    pad = sess.get_output("output", "NHWC4")
+    assert pad.shape == (2, 5, 4, 8)
+    np.testing.assert_array_equal(pad[..., :7], dense)
+    assert (pad[..., 7:] == 0).all()
+    np.testing.assert_array_equal(sess.get_output("output", "ANY4"), pad)
+    bias4 = sess.get_output("conv2d1.bias", "ANY4")
+    assert bias4.shape == (8,) and (bias4[:7] == b).all() and bias4[7] == 0
+    np.testing.assert_array_equal(sess.get_output("conv2d1.weight", "HWN4C4").ravel(),
+                                  O.nchw_to_hwn4c4(wt).ravel())
+    with pytest.raises(RuntimeError, match="HWN4C4"):
+        sess.get_output("output", "HWN4C4")
+    # upload from the padded layout: same device contents, same result
+    xp = np.zeros((2, 5, 4, 8), np.float32)
+    xp[..., :6] = x
+    sess2 = session.Session()
+    sess2.load_graph(conv_graph(x.shape, wt, b, 3, 1, 1))
+    sess2.run({"input": xp}, dformats={"input": "NHWC4"}, shapes={"input": x.shape})
+    np.testing.assert_array_equal(sess2.get_output("input", "NHWC4"), xp)
+    np.testing.assert_array_equal(sess2.get_output("output", "NHWC"), dense)
+
+
+def test_reload_after_a_captured_pass():
+    """LoadGraph on a session that has run and recorded its pass: the recorded hipGraph (whose
+    kernel arguments are the old tensors' addresses) must be gone, and the new graph runs and
+    records on its own."""
+    g1, w1 = models.separable_block(1, size=19, cin=64, cout=128)
+    r = rng(7900)
+    x1 = r.uniform(0, 6, (1, 19, 19, 64)).astype(np.float32)
+    sess = session.Session()
+    sess.load_graph(g1)
+    sess.run({"input": x1})
+    sess.compute(graph=True)
+    first = sess.get_output("pw", "NHWC")
+    assert sess.graph_captured(0)
+    g2, w2 = models.separable_block(2, seed=5, size=10, cin=32, cout=48)
+    x2 = r.uniform(0, 6, (2, 10, 10, 32)).astype(np.float32)
+    sess.load_graph(g2)
+    assert not sess.graph_captured(0) and sess.issue_order() == []
+    sess.run({"input": x2})
+    dw = O.conv2d(x2, w2["wd"], w2["bd"], 1, 1, 1, 32, O.ACT_CLIP, 0.0, 6.0)
+    ref = O.conv2d(dw, w2["wp"], w2["bp"], act=O.ACT_CLIP, maxv=6.0, variant=O.VARIANT_PW)
+    got = sess.get_output("pw", "NHWC")
+    assert_conv_close(got, ref, O.conv2d_abs(dw, w2["wp"], w2["bp"]), 1e-5, "after reload")
+    sess.compute(graph=True)
+    assert sess.graph_captured(0)
+    np.testing.assert_array_equal(sess.get_output("pw", "NHWC"), got)
+    # and back to the first graph: same answer as before
+    sess.load_graph(g1)
+    sess.run({"input": x1})
+    np.testing.assert_array_equal(sess.get_output("pw", "NHWC"), first)
+
+
+@pytest.mark.parametrize("second_reader", [False, True])
+def test_unaligned_head_also_read_by_another_node_keeps_its_own_buffer(second_reader):
+    """At batch 1 head outputs are produced inside the concat output; a 63-channel head lands
+    at a 4-byte-aligned place, which only a convolution's element-wise stores tolerate.  If the
+    head also feeds a Relu node (16-byte vector loads from the tensor start), it must not be
+    moved there."""
+    r = rng(7990)
+    x = r.uniform(-1, 1, (1, 3, 3, 16)).astype(np.float32)
+    wa = r.normal(0, 0.3, (63, 16, 3, 3)).astype(np.float32)
+    wb = r.normal(0, 0.3, (63, 16, 3, 3)).astype(np.float32)
+    gb = dlx.GraphBuilder()
+    xi = gb.add_input("input", [1, 16, 3, 3])
+    outs = []
+    for name, wt in (("a", wa), ("b", wb)):
+        y = gb.add_conv(name, xi, gb.add_filter(name + ".weight", wt), None, 3, 1, 1)
+        t = gb.add_transpose(name + ".permute", y, [0, 2, 3, 1])
+        shp = gb.add_const(name + ".shape", np.array([1, -1, 21], np.float32))
+        outs.append(gb.add_reshape(name + ".view", t, shp))
+        if name == "b" and second_reader:
+            gb.add_relu("b.relu", y)
+    gb.add_concat("cat", outs, 1)
+    sess = session.Session()
+    sess.load_graph(gb)
+    sess.run({"input": x})
+    ra, rb = O.conv2d(x, wa, None, 1, 1), O.conv2d(x, wb, None, 1, 1)
+    cat = sess.get_output("cat", "ANY")
+    ref = np.concatenate([ra.reshape(1, -1, 21), rb.reshape(1, -1, 21)], 1)
+    np.testing.assert_allclose(cat, ref, rtol=0, atol=1e-4)
+    base = sess.tensor_device_ptr("cat")
+    if second_reader:
+        np.testing.assert_array_equal(sess.get_output("b.relu", "NHWC"),
+                                      np.maximum(sess.get_output("b", "NHWC"), 0))
+        # head b would start at byte 9*63*4 = 2268 of the concat output, which is not 16-byte
+        # aligned, and it has a second reader: nothing is placed, the concat copies
+        assert sess.tensor_device_ptr("a") != base
+        assert sess.tensor_device_ptr("b") != base + 2268
+    else:
+        assert sess.tensor_device_ptr("a") == base
+        assert sess.tensor_device_ptr("b") == base + 2268
