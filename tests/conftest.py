@@ -28,3 +28,27 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+def pytest_sessionfinish(session, exitstatus):
+    """After a GPU session: the achieved parity figures (worst |err| / sum|x||w| and worst
+    relative error per comparison label), so that they can be quoted next to the tolerances."""
+    try:
+        import json
+        import util
+        if not util.PARITY_LOG:
+            return
+        out = os.path.join(ROOT, "gpurun_out")
+        os.makedirs(out, exist_ok=True)
+        rows = {k: dict(normwise=v[0], relative=v[1], rtol=v[2]) for k, v in util.PARITY_LOG.items()}
+        fp32 = [v for v in util.PARITY_LOG.values() if v[2] <= 1e-4]
+        fp16 = [v for v in util.PARITY_LOG.values() if v[2] > 1e-4]
+        summary = dict(
+            fp32_worst_normwise=max([v[0] for v in fp32], default=0.0),
+            fp32_worst_relative=max([v[1] for v in fp32], default=0.0),
+            fp16_worst_normwise=max([v[0] for v in fp16], default=0.0),
+            fp16_worst_relative=max([v[1] for v in fp16], default=0.0), comparisons=len(rows))
+        with open(os.path.join(out, "parity_achieved.json"), "w") as f:
+            json.dump(dict(summary=summary, rows=rows), f, indent=1, sort_keys=True)
+    except Exception:
+        pass

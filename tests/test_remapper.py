@@ -91,7 +91,7 @@ def test_remap_leaves_shared_or_activated_patterns_alone():
 @pytest.mark.gpu
 def test_unfused_and_folded_graphs_on_the_device():
     from ogle_amd import session
-    from util import assert_conv_close
+    from util import FP32_RTOL, assert_conv_close
     r = rng(30002)
     batch, size, c = 2, 12, 16
     gb, weights = residual_graph(r, batch, size, c)
@@ -130,7 +130,7 @@ def test_unfused_and_folded_graphs_on_the_device():
     # the folded first stage against the oracle with the oracle's folded parameters
     wf, bf = O.fold_bn(w1, b1, *p1, 1e-5)
     ref1 = O.conv2d(x, wf, bf, 1, 1, 1, 1, O.ACT_CLIP, 0.0, 6.0)
-    assert_conv_close(folded.get_output("c1.act", "NHWC"), ref1, O.conv2d_abs(x, wf, bf, 1, 1), 1e-4, "c1")
+    assert_conv_close(folded.get_output("c1.act", "NHWC"), ref1, O.conv2d_abs(x, wf, bf, 1, 1), FP32_RTOL, "c1")
     assert len(folded.issue_order()) == 5 and len(unfused.issue_order()) == 9
 
 

@@ -54,7 +54,7 @@ def test_noalloc_matches_workspace_entry_two_calls_in_a_row():
         needs.append(need)
         assert np.array_equal(got, ref), (n, h, w, c, o, k)
         ora = O.conv2d(x, wt, b, s, p, 1, 1, O.ACT_RELU)
-        U.assert_conv_close(got, ora, O.conv2d_abs(x, wt, b, s, p, 1, 1), 1e-5, "noalloc")
+        U.assert_conv_close(got, ora, O.conv2d_abs(x, wt, b, s, p, 1, 1), U.FP32_RTOL, "noalloc")
     assert needs[0] > needs[1] > 0 and needs[0] <= H.CONV_NOALLOC_SCRATCH_BYTES, needs
 
 

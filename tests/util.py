@@ -200,20 +200,48 @@ def gpu_topk_nms(counts, prior, cls, score, rect, topk, threshold, box=None):
     return out
 
 
-def assert_conv_close(got, ref, scale, rtol, what=""):
-    """The fp32 / fp16 parity rule for contractions.
+# Parity rule for contractions (BASELINE: fp32 max relative error 1e-4, fp16 5e-3).
+# Two tests per output tensor:
+#  (1) normwise: |got - ref| <= RTOL * (sum|x||w| + |b|) for EVERY output.  This is the bound
+#      fp32 summation can be held to: it stays meaningful where cancellation or the activation
+#      leaves an output at or near zero, where no relative bound can hold.
+#  (2) BASELINE's literal wording on every output that is not dominated by cancellation,
+#      |ref| >= REL_FLOOR * (sum|x||w| + |b|): |got - ref| <= REL * |ref|.  With fp16 storage
+#      the operands themselves are rounded (2^-11 each), an error proportional to sum|x||w|, not
+#      to the output, so the literal bound can only be asked of outputs that keep at least
+#      FP16_REL_FLOOR of that magnitude.
+FP32_RTOL = 1e-5
+FP16_RTOL = 5e-3
+FP32_REL = 1e-4
+FP16_REL = 5e-3
+REL_FLOOR = 1e-2
+FP16_REL_FLOOR = 5e-2
 
-    `scale` is sum |x||w| + |b| per output (oracle.conv2d_abs): the magnitude the
-    rounding error of a dot product is proportional to.  The rule is
-    |got - ref| <= rtol * scale elementwise: "relative error" measured against the
-    accumulated magnitude, which stays meaningful where cancellation or the
-    activation leaves an output at or near zero.
-    """
+# what -> (worst normwise ratio err/scale, worst relative error where test (2) applies):
+# the achieved figures, written to gpurun_out/parity_achieved.json at the end of a GPU session.
+PARITY_LOG = {}
+
+
+def assert_conv_close(got, ref, scale, rtol, what="", rel=None):
+    """Both parity tests above.  `scale` is sum|x||w| + |b| per output (oracle.conv2d_abs, or
+    the same contraction of absolute values in float64).  rtol FP32_RTOL or FP16_RTOL selects
+    the matching relative bound unless `rel` is given.  Returns the worst err / scale."""
     assert got.shape == ref.shape, (got.shape, ref.shape)
     assert np.all(np.isfinite(got)), "non-finite output " + what
-    err = np.abs(got.astype(np.float64) - ref.astype(np.float64))
-    bound = rtol * scale.astype(np.float64) + 1e-30
-    worst = float(np.max(err / bound))
-    assert worst <= 1.0, "%s: error is %.3g x the allowed %g * sum|x||w| (max abs err %.3g)" % (
-        what, worst, rtol, float(err.max()))
-    return worst * rtol
+    if rel is None:
+        rel = FP32_REL if rtol <= FP32_REL else FP16_REL
+    floor = REL_FLOOR if rtol <= FP32_REL else FP16_REL_FLOOR
+    g64, r64, s64 = got.astype(np.float64), ref.astype(np.float64), scale.astype(np.float64)
+    err = np.abs(g64 - r64)
+    norm = float(np.max(err / (s64 + 1e-30))) if err.size else 0.0
+    assert norm <= rtol, "%s: error is %.3g of sum|x||w|, allowed %g (max abs err %.3g)" % (
+        what, norm, rtol, float(err.max()))
+    big = np.abs(r64) >= floor * s64
+    big &= np.abs(r64) > 0
+    worst_rel = float(np.max(err[big] / np.abs(r64[big]))) if big.any() else 0.0
+    assert worst_rel <= rel, "%s: max relative error %.3g over outputs with |ref| >= %g*scale, " \
+        "allowed %g" % (what, worst_rel, floor, rel)
+    key = what or "conv"
+    old = PARITY_LOG.get(key, (0.0, 0.0, rtol))
+    PARITY_LOG[key] = (max(old[0], norm), max(old[1], worst_rel), rtol)
+    return norm
