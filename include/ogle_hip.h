@@ -149,6 +149,18 @@ typedef struct OgleConvArgs {
    * that needs none.  Launches on one stream may share one workspace. */
   void* workspace_dev;
   size_t workspace_bytes;
+  /* Optional second destination (NULL: none).  With output2_dev set, 0 < out_c_split <
+   * out_c and the convolution's output channels are divided between two dense NHWC
+   * tensors: channels [0, out_c_split) of every pixel go to output_dev (out_c_split
+   * channels per pixel), channels [out_c_split, out_c) to output2_dev (out_c -
+   * out_c_split channels per pixel).  filter_dev and bias_dev cover all out_c channels.
+   * This is how two convolutions that read the same input with the same geometry (the
+   * box and class head of one SSD feature map) run as ONE contraction that fetches the
+   * input once; the reference draws them one after the other (fbo_session.cc:140-153).
+   * Only the MFMA implicit-GEMM path takes it (group 1, in_c % 4 == 0, k*k*in_c >= 32;
+   * fp16 storage: in_c % 8 == 0): otherwise OGLE_ERR_UNSUPPORTED. */
+  void* output2_dev;
+  int32_t out_c_split;
 } OgleConvArgs;
 
 /* Bytes of workspace the fastest plan for `args` would use (0 if it needs none). */

@@ -153,6 +153,14 @@ int32_t ogle_rt_num_kernels(OgleSession* s);
  * the i-th node a pass issues (valid after the first run; NULL past the end).
  */
 int32_t ogle_rt_set_reorder(OgleSession* s, int32_t on);
+/*
+ * Sibling fusion.  Two Conv nodes that read the same tensor with the same attributes (the
+ * box and the class head of an SSD feature map) run as one launch that fetches the input
+ * once and writes each node's channels to its own tensor; the reference draws them one
+ * after the other.  ogle_rt_set_fuse_siblings(s, 0) before the first run keeps one launch
+ * per node.  Results agree to summation order.
+ */
+int32_t ogle_rt_set_fuse_siblings(OgleSession* s, int32_t on);
 const char* ogle_rt_issue_order_name(OgleSession* s, int32_t i);
 int32_t ogle_rt_registered_kernel_count(void);
 const char* ogle_rt_registered_kernel_name(int32_t i);

@@ -69,13 +69,28 @@ constexpr int kRegistrySize = sizeof(kRegistry) / sizeof(kRegistry[0]);
 
 bool positive(int v) { return v > 0; }
 
+const char kSplitNeedsMfma[] =
+    "a second destination (output2_dev) is only supported by the MFMA implicit-GEMM kernels: "
+    "group 1, in_c % 4 == 0 (fp16: % 8), kernel_size^2 * in_c >= 32";
+
+// launch_conv_direct for the batch entry point: it cannot divide the output.
+int32_t direct_no_split(const OgleConvArgs& a, hipStream_t s) {
+  if (a.output2_dev != nullptr) return fail(OGLE_ERR_UNSUPPORTED, kSplitNeedsMfma);
+  return launch_conv_direct(a, s);
+}
+
 // Byte extents of a convolution's tensors, and interval overlap of two device ranges.
 size_t elem_bytes(const OgleConvArgs& a) { return a.dtype == OGLE_F16 ? 2 : 4; }
 size_t input_bytes(const OgleConvArgs& a) {
   return (size_t)a.n * a.in_h * a.in_w * a.in_c * elem_bytes(a);
 }
 size_t output_bytes(const OgleConvArgs& a) {
-  return (size_t)a.n * a.out_h * a.out_w * a.out_c * elem_bytes(a);
+  const int c = a.output2_dev != nullptr ? a.out_c_split : a.out_c;
+  return (size_t)a.n * a.out_h * a.out_w * c * elem_bytes(a);
+}
+size_t output2_bytes(const OgleConvArgs& a) {
+  if (a.output2_dev == nullptr) return 0;
+  return (size_t)a.n * a.out_h * a.out_w * (a.out_c - a.out_c_split) * elem_bytes(a);
 }
 bool overlap(const void* a, size_t a_bytes, const void* b, size_t b_bytes) {
   if (a == nullptr || b == nullptr || a_bytes == 0 || b_bytes == 0) return false;
@@ -115,6 +130,11 @@ int32_t validate_conv(const OgleConvArgs* a, const char* who) {
     set_error("%s: output %dx%d does not follow from input %dx%d k%d s%d p%d d%d (expect %dx%d)",
               who, a->out_h, a->out_w, a->in_h, a->in_w, a->kernel_size, a->stride, a->padding,
               a->dilation, oh, ow);
+    return OGLE_ERR_INVALID_ARG;
+  }
+  if (a->output2_dev != nullptr && (a->out_c_split <= 0 || a->out_c_split >= a->out_c)) {
+    set_error("%s: out_c_split %d must lie strictly between 0 and out_c %d", who, a->out_c_split,
+              a->out_c);
     return OGLE_ERR_INVALID_ARG;
   }
   if (a->in_c % a->group != 0 || a->out_c % a->group != 0) {
@@ -229,6 +249,7 @@ int32_t ogle_hip_conv2d(const OgleConvArgs* a, ogle_stream_t stream) {
     st = launch_conv_igemm(*a, as_stream(stream));
     if (st != OGLE_ERR_UNSUPPORTED) return st;
   }
+  if (a->output2_dev != nullptr) return fail(OGLE_ERR_UNSUPPORTED, kSplitNeedsMfma);
   return launch_conv_direct(*a, as_stream(stream));
 }
 
@@ -242,6 +263,7 @@ int32_t ogle_hip_conv2d_noalloc(const OgleConvArgs* a, ogle_stream_t stream) {
     st = launch_conv_igemm_static_scratch(*a, as_stream(stream));
     if (st != OGLE_ERR_UNSUPPORTED) return st;
   }
+  if (a->output2_dev != nullptr) return fail(OGLE_ERR_UNSUPPORTED, kSplitNeedsMfma);
   return launch_conv_direct(*a, as_stream(stream));
 }
 
@@ -257,6 +279,12 @@ int32_t ogle_hip_conv2d_batch(const OgleConvArgs* args, int32_t count, ogle_stre
           overlap(q.input_dev, input_bytes(q), p.output_dev, output_bytes(p)) ||
           overlap(p.output_dev, output_bytes(p), q.output_dev, output_bytes(q)))
         return fail(OGLE_ERR_INVALID_ARG, "conv2d_batch: the convolutions depend on each other");
+      if (overlap(p.output2_dev, output2_bytes(p), q.input_dev, input_bytes(q)) ||
+          overlap(q.output2_dev, output2_bytes(q), p.input_dev, input_bytes(p)) ||
+          overlap(p.output2_dev, output2_bytes(p), q.output_dev, output_bytes(q)) ||
+          overlap(q.output2_dev, output2_bytes(q), p.output_dev, output_bytes(p)) ||
+          overlap(p.output2_dev, output2_bytes(p), q.output2_dev, output2_bytes(q)))
+        return fail(OGLE_ERR_INVALID_ARG, "conv2d_batch: the convolutions depend on each other");
       if (overlap(p.workspace_dev, p.workspace_bytes, q.workspace_dev, q.workspace_bytes))
         return fail(OGLE_ERR_INVALID_ARG, "conv2d_batch: two convolutions share one workspace");
       if (overlap(p.workspace_dev, p.workspace_bytes, q.output_dev, output_bytes(q)) ||
@@ -267,7 +295,7 @@ int32_t ogle_hip_conv2d_batch(const OgleConvArgs* args, int32_t count, ogle_stre
                     "conv2d_batch: a workspace overlaps another convolution's tensor");
     }
   }
-  return launch_conv_batch(args, count, as_stream(stream), launch_conv_direct);
+  return launch_conv_batch(args, count, as_stream(stream), direct_no_split);
 }
 
 int32_t ogle_hip_dwconv2d(const OgleConvArgs* a, ogle_stream_t stream) {
@@ -278,6 +306,7 @@ int32_t ogle_hip_dwconv2d(const OgleConvArgs* a, ogle_stream_t stream) {
     set_error("dwconv2d: group %d must equal in_c %d and out_c %d", a->group, a->in_c, a->out_c);
     return OGLE_ERR_INVALID_ARG;
   }
+  if (a->output2_dev != nullptr) return fail(OGLE_ERR_UNSUPPORTED, kSplitNeedsMfma);
   return launch_conv_dw(*a, as_stream(stream));
 }
 
@@ -292,6 +321,7 @@ int32_t ogle_hip_pwconv_gemm(const OgleConvArgs* a, ogle_stream_t stream) {
   }
   st = launch_conv_igemm(*a, as_stream(stream));
   if (st != OGLE_ERR_UNSUPPORTED) return st;
+  if (a->output2_dev != nullptr) return fail(OGLE_ERR_UNSUPPORTED, kSplitNeedsMfma);
   return launch_conv_direct(*a, as_stream(stream));
 }
 

@@ -4,13 +4,11 @@
 //
 // Thread mapping: consecutive threads take consecutive 16-byte channel vectors
 // of consecutive pixel columns of one image row, so a wave's loads and stores
-// are contiguous runs of NHWC memory.  Each thread owns a small patch of output
-// pixels (R rows x Q columns) and requests every input vector the patch needs
-// with branch-free buffer loads before it starts to accumulate, so all of a
-// wave's loads are in flight at once; neighbouring patches' halo vectors are the
-// same bytes other lanes and the adjacent wave load at the same time and are
-// served by the vector L1 / the XCD's L2 (the block order keeps neighbours on one
-// XCD).
+// are contiguous runs of NHWC memory.  A thread walks down a segment of output rows
+// with the input rows it needs in a ring of registers and the next rows already
+// requested (see dwconv3x3_rows); neighbouring threads' halo columns are the same
+// bytes other lanes and the adjacent wave load at the same time and are served by
+// the vector L1 / the XCD's L2 (the block order keeps neighbours on one XCD).
 //
 // Semantics follow conv2d_dw.glsl:38-96: accumulator starts at the bias, taps
 // outside the image are skipped, order ky then kx, then the fused activation.
@@ -93,126 +91,122 @@ __device__ __forceinline__ unsigned fast_div(unsigned n, const FastDiv& f) {
   return (__umulhi(n, f.mul) + n) >> f.shift;
 }
 
-// 3x3, dilation 1, stride S, channel count a multiple of the vector width.
-// A thread owns a patch of R output rows x Q output columns of one channel vector.
-// Index arithmetic is kept off the vector ALU as far as possible (the kernel issues
-// about as many address instructions as FMAs otherwise): the thread index is split
-// with multiply-high divisions, input offsets are a row term plus a column term, and
-// a tap outside the image just gets the out-of-range bit set in its offset.
-template <typename T, int S, int R, int Q>
-__global__ __launch_bounds__(256) void dwconv3x3_strip(
+// 3x3, dilation 1, stride S, channel count a multiple of the vector width.  A thread owns Q output columns of one
+// channel vector and walks DOWN a segment of output rows, holding the input rows it needs
+// in a ring of registers: moving one output row down re-uses 3 - S of the 3 input rows and
+// loads S new ones, so an input vector is requested once per thread that needs it (2
+// requests per output at stride 1 with Q = 2, against 4 for a 2x2 patch and 9 naively),
+// and the rows PF steps ahead are requested before the current row is accumulated: the
+// loads of a wave never stop while it computes and stores.  Rows above / below the image
+// and columns left / right of it come back as zeros (out-of-range buffer offsets), rows
+// past the end of the segment are not requested at all.
+template <typename T, int S, int Q, int PF>
+__global__ __launch_bounds__(256) void dwconv3x3_rows(
     const T* __restrict__ x, const T* __restrict__ w, const float* __restrict__ bias,
     T* __restrict__ y, int h, int wd, int c, int oh, int ow, int pad, Epilogue ep,
     unsigned x_bytes, unsigned y_bytes, unsigned total, FastDiv div_cv, FastDiv div_cols,
-    FastDiv div_strips) {
+    FastDiv div_segs, int seg_rows) {
   constexpr int V = Vec<T>::N;
-  constexpr int IN_ROWS = (R - 1) * S + 3;
   constexpr int IN_COLS = (Q - 1) * S + 3;
+  constexpr int NB = 3 + S * PF;  // ring of input rows: three in use, S * PF on their way
   constexpr unsigned ESZ = sizeof(T);
-  constexpr unsigned kOut = 0x80000000u;  // offsets at or above this are outside every operand
-  // Consecutive logical blocks (neighbouring pixels and strips, which share halo
-  // rows) are kept on one XCD so that the re-read rows hit that XCD's L2.
+  constexpr unsigned kOut = 0x80000000u;
   const unsigned idx = (unsigned)xcd_swizzle(blockIdx.x, gridDim.x) * 256u + threadIdx.x;
   if (idx >= total) return;
   const unsigned t1 = fast_div(idx, div_cv);
   const int cg = (int)(idx - t1 * div_cv.d);
   const unsigned t2 = fast_div(t1, div_cols);
   const int oxg = (int)(t1 - t2 * div_cols.d);
-  const unsigned b = fast_div(t2, div_strips);
-  const int strip = (int)(t2 - b * div_strips.d);
+  const unsigned b = fast_div(t2, div_segs);
+  const int seg = (int)(t2 - b * div_segs.d);
   const int ch = cg * V;
-  const int oy0 = strip * R;
+  const int oy0 = seg * seg_rows;
+  const int rows = min(seg_rows, oh - oy0);  // output rows of this segment (>= 1)
   const int ox0 = oxg * Q;
 
   float wt[9][V];
 #pragma unroll
   for (int tap = 0; tap < 9; ++tap) Vec<T>::load(w + tap * c + ch, wt[tap]);
-
-  float acc[R][Q][V];
-  {
-    float bv[V];
+  float bv[V];
 #pragma unroll
-    for (int v = 0; v < V; ++v) bv[v] = 0.f;
-    if (bias != nullptr) {
+  for (int v = 0; v < V; ++v) bv[v] = 0.f;
+  if (bias != nullptr) {
 #pragma unroll
-      for (int v = 0; v < V; v += 4) {
-        const float4 t = *reinterpret_cast<const float4*>(bias + ch + v);  // ch % 4 == 0
-        bv[v] = t.x; bv[v + 1] = t.y; bv[v + 2] = t.z; bv[v + 3] = t.w;
-      }
+    for (int v = 0; v < V; v += 4) {
+      const float4 t = *reinterpret_cast<const float4*>(bias + ch + v);
+      bv[v] = t.x; bv[v + 1] = t.y; bv[v + 2] = t.z; bv[v + 3] = t.w;
     }
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-#pragma unroll
-      for (int q = 0; q < Q; ++q)
-#pragma unroll
-        for (int v = 0; v < V; ++v) acc[r][q][v] = bv[v];
   }
 
-  // Every input vector the patch needs is requested up front with buffer loads;
-  // taps outside the image get an out-of-range offset and come back as zeros, so
-  // there is no branch between the loads and they are all in flight together.
-  const int iy0 = oy0 * S - pad;
-  const int ix0 = ox0 * S - pad;
   const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<T*>(x), 0, (int)x_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t ry = __builtin_amdgcn_make_buffer_rsrc(y, 0, (int)y_bytes, 0x00020000);
   const unsigned row_bytes = (unsigned)(wd * c) * ESZ;
   const unsigned img = (b * (unsigned)h) * row_bytes + (unsigned)ch * ESZ;
-  unsigned row_off[IN_ROWS], col_off[IN_COLS];
-#pragma unroll
-  for (int j = 0; j < IN_ROWS; ++j) {
-    const int iy = iy0 + j;
-    row_off[j] = (unsigned)iy < (unsigned)h ? img + (unsigned)iy * row_bytes : kOut;
-  }
+  const int iy_base = oy0 * S - pad;           // input row of ring position 0
+  const int in_rows = (rows - 1) * S + 3;      // input rows this segment touches
+  unsigned col_off[IN_COLS];
 #pragma unroll
   for (int s = 0; s < IN_COLS; ++s) {
-    const int ix = ix0 + s;
+    const int ix = ox0 * S - pad + s;
     col_off[s] = (unsigned)ix < (unsigned)wd ? (unsigned)(ix * c) * ESZ : kOut;
   }
-  u32x4 raw[IN_ROWS][IN_COLS];
+  u32x4 raw[NB][IN_COLS];
+  // requests input row `r` (relative to iy_base) into ring slot `slot`
+#define OGLE_DW_LOAD_ROW(slot, r)                                                               \
+  {                                                                                             \
+    const int iy_ = iy_base + (r);                                                              \
+    const unsigned ro_ = ((r) < in_rows && (unsigned)iy_ < (unsigned)h)                         \
+                             ? img + (unsigned)iy_ * row_bytes : kOut;                          \
+    _Pragma("unroll") for (int s = 0; s < IN_COLS; ++s) {                                       \
+      const unsigned off_ = (ro_ + col_off[s]) | ((ro_ | col_off[s]) & kOut);                   \
+      raw[slot][s] = __builtin_amdgcn_raw_buffer_load_b128(rx, (int)off_, 0, 0);                \
+    }                                                                                           \
+  }
 #pragma unroll
-  for (int j = 0; j < IN_ROWS; ++j)
+  for (int j = 0; j < NB - S; ++j) OGLE_DW_LOAD_ROW(j, j);   // rows 0 .. 2 + S*(PF-1)
+  const unsigned out_row_bytes = (unsigned)(ow * c) * ESZ;
+  unsigned out_off = (b * (unsigned)oh + (unsigned)oy0) * out_row_bytes + (unsigned)(ox0 * c + ch) * ESZ;
+  for (int t0 = 0; t0 < rows; t0 += NB) {
 #pragma unroll
-    for (int s = 0; s < IN_COLS; ++s) {
-      // a valid row plus a valid column stays below 2^31; either term being kOut sets
-      // the top bit of the OR, whatever the sum wrapped to
-      const unsigned off = (row_off[j] + col_off[s]) | ((row_off[j] | col_off[s]) & kOut);
-      raw[j][s] = __builtin_amdgcn_raw_buffer_load_b128(rx, (int)off, 0, 0);
-    }
+    for (int u = 0; u < NB; ++u) {
+      const int t = t0 + u;                    // output row of the segment
+      if (t < rows) {
+        // the S rows that output row t + PF will newly need go into the slots of the rows
+        // output row t - 1 was the last to use
 #pragma unroll
-  for (int j = 0; j < IN_ROWS; ++j) {
-    float in[IN_COLS][V];
+        for (int e = 0; e < S; ++e)
+          OGLE_DW_LOAD_ROW((S * u + 3 + S * (PF - 1) + e) % NB, S * t + 3 + S * (PF - 1) + e);
+        float acc[Q][V];
 #pragma unroll
-    for (int s = 0; s < IN_COLS; ++s) Vec<T>::unpack(raw[j][s], in[s]);
+        for (int q = 0; q < Q; ++q)
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      const int ky = j - r * S;  // compile-time after unrolling
-      if (ky < 0 || ky > 2) continue;
+          for (int v = 0; v < V; ++v) acc[q][v] = bv[v];
 #pragma unroll
-      for (int q = 0; q < Q; ++q) {
+        for (int ky = 0; ky < 3; ++ky) {
+          float in[IN_COLS][V];
 #pragma unroll
-        for (int kx = 0; kx < 3; ++kx) {
+          for (int s = 0; s < IN_COLS; ++s) Vec<T>::unpack(raw[(S * u + ky) % NB][s], in[s]);
 #pragma unroll
-          for (int v = 0; v < V; ++v) acc[r][q][v] += wt[ky * 3 + kx][v] * in[q * S + kx][v];
+          for (int q = 0; q < Q; ++q)
+#pragma unroll
+            for (int kx = 0; kx < 3; ++kx)
+#pragma unroll
+              for (int v = 0; v < V; ++v) acc[q][v] += wt[ky * 3 + kx][v] * in[q * S + kx][v];
         }
+#pragma unroll
+        for (int q = 0; q < Q; ++q) {
+          float out[V];
+#pragma unroll
+          for (int v = 0; v < V; ++v) out[v] = apply_epilogue(acc[q][v], ep);
+          const unsigned off = ox0 + q < ow ? out_off + (unsigned)(q * c) * ESZ : kOut;
+          __builtin_amdgcn_raw_buffer_store_b128(Vec<T>::pack(out), ry, (int)off, 0, 0);
+        }
+        out_off += out_row_bytes;
       }
     }
   }
-  const __amdgpu_buffer_rsrc_t ry = __builtin_amdgcn_make_buffer_rsrc(y, 0, (int)y_bytes, 0x00020000);
-  const unsigned out_row_bytes = (unsigned)(ow * c) * ESZ;
-  const unsigned out0 = (b * (unsigned)oh + (unsigned)oy0) * out_row_bytes +
-                        (unsigned)(ox0 * c + ch) * ESZ;
-#pragma unroll
-  for (int r = 0; r < R; ++r) {
-#pragma unroll
-    for (int q = 0; q < Q; ++q) {
-      float out[V];
-#pragma unroll
-      for (int v = 0; v < V; ++v) out[v] = apply_epilogue(acc[r][q][v], ep);
-      const bool ok = oy0 + r < oh && ox0 + q < ow;
-      const unsigned off = ok ? out0 + (unsigned)r * out_row_bytes + (unsigned)(q * c) * ESZ : kOut;
-      __builtin_amdgcn_raw_buffer_store_b128(Vec<T>::pack(out), ry, (int)off, 0, 0);
-    }
-  }
+#undef OGLE_DW_LOAD_ROW
 }
 
 // Any kernel size / dilation / channel count: one thread per output element.
@@ -254,51 +248,49 @@ FastDiv make_fast_div(unsigned d) {
   return f;
 }
 
-template <typename T, int S, int R, int Q = 1>
-int32_t launch_strip(const OgleConvArgs& a, hipStream_t s, const Epilogue& ep) {
+template <typename T, int S, int Q, int PF>
+int32_t launch_rows(const OgleConvArgs& a, hipStream_t s, const Epilogue& ep, int seg_rows) {
   constexpr int V = Vec<T>::N;
-  const int strips = (a.out_h + R - 1) / R, cols = (a.out_w + Q - 1) / Q, cv = a.in_c / V;
-  const long total = (long)a.n * strips * cols * cv;
+  const int segs = (a.out_h + seg_rows - 1) / seg_rows, cols = (a.out_w + Q - 1) / Q, cv = a.in_c / V;
+  const long total = (long)a.n * segs * cols * cv;
   const int blocks = (ceil_div(total, 256) + 7) / 8 * 8;  // whole XCD rounds
-  hipLaunchKernelGGL((dwconv3x3_strip<T, S, R, Q>), dim3(blocks), dim3(256), 0, s,
+  hipLaunchKernelGGL((dwconv3x3_rows<T, S, Q, PF>), dim3(blocks), dim3(256), 0, s,
                      static_cast<const T*>(a.input_dev), static_cast<const T*>(a.filter_dev),
                      a.bias_dev, static_cast<T*>(a.output_dev), a.in_h, a.in_w, a.in_c, a.out_h,
                      a.out_w, a.padding, ep,
                      (unsigned)((long)a.n * a.in_h * a.in_w * a.in_c * sizeof(T)),
                      (unsigned)((long)a.n * a.out_h * a.out_w * a.in_c * sizeof(T)), (unsigned)total,
                      make_fast_div((unsigned)cv), make_fast_div((unsigned)cols),
-                     make_fast_div((unsigned)strips));
-  return check_launch("dwconv3x3_strip");
+                     make_fast_div((unsigned)segs), seg_rows);
+  return check_launch("dwconv3x3_rows");
 }
 
+// Segment length and columns per thread, measured on MI355X over the MobileNet shapes
+// (batch 16; 150x150x32 ... 10x10x1024): two columns per thread at stride 1 (input
+// requests per output: 2), one at stride 2 (two columns would need five input columns in
+// registers); one step of prefetch (two gained nothing); segments of 13 rows on the large
+// maps (halo rows re-read by the next segment: 2 in 15) and of 4 rows on maps of 38 rows
+// and below, where the number of waves, not the re-read rows, decides the time.
 template <typename T, int S>
-int32_t pick_strip(const OgleConvArgs& a, hipStream_t s, const Epilogue& ep) {
-  constexpr int V = Vec<T>::N;
-  // A 2x2 (stride 1) or 2x1 patch per thread shares input rows and columns in
-  // registers; smaller problems fall back to one output per thread so that the
-  // grid still covers the 256 CUs (measured on MI355X: patches beyond 2 rows gain
-  // nothing once all loads of a patch are in flight together).
-  const long per_row_threads = (long)a.n * a.out_w * (a.in_c / V);
-  const long want = 256L * 256 * 4;
-  if (S == 1 && per_row_threads / 2 * ((a.out_h + 1) / 2) >= want / 2)
-    return launch_strip<T, S, 2, 2>(a, s, ep);
-  if (per_row_threads * ((a.out_h + 1) / 2) >= want / 2) return launch_strip<T, S, 2, 1>(a, s, ep);
-  return launch_strip<T, S, 1>(a, s, ep);
+int32_t pick_rows(const OgleConvArgs& a, hipStream_t s, const Epilogue& ep) {
+  const int seg_rows = (S == 1 && a.out_h > 40) ? 13 : 4;
+  if (S == 1 && a.out_w >= 2) return launch_rows<T, S, 2, 1>(a, s, ep, seg_rows);
+  return launch_rows<T, S, 1, 1>(a, s, ep, seg_rows);
 }
 
 template <typename T>
 int32_t run_dw(const OgleConvArgs& a, hipStream_t s) {
   const Epilogue ep = make_epilogue(a.act, a.min_value, a.max_value, a.act_variant);
   constexpr int V = Vec<T>::N;
-  // the strip kernel addresses the input with 32-bit byte offsets (buffer loads)
+  // the 3x3 kernel addresses the input with 32-bit byte offsets (buffer loads)
   // and the bias with 16-byte loads
   const bool fits = (long)a.n * a.in_h * a.in_w * a.in_c * (long)sizeof(T) < 0x7fffffffL &&
                     (long)a.n * a.out_h * a.out_w * a.in_c * (long)sizeof(T) < 0x7fffffffL &&
                     (reinterpret_cast<uintptr_t>(a.bias_dev) & 15u) == 0;
   if (a.kernel_size == 3 && a.dilation == 1 && a.in_c % V == 0 && fits &&
       (a.stride == 1 || a.stride == 2)) {
-    if (a.stride == 1) return pick_strip<T, 1>(a, s, ep);
-    return pick_strip<T, 2>(a, s, ep);
+    if (a.stride == 1) return pick_rows<T, 1>(a, s, ep);
+    return pick_rows<T, 2>(a, s, ep);
   }
   const long total = (long)a.n * a.out_h * a.out_w * a.out_c;
   int blocks = ceil_div(total, 256);

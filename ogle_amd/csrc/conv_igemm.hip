@@ -92,8 +92,9 @@ constexpr int igemm_lds_bytes() {
 template <typename T, int BM, int BN, int WM, int WN, int ROWB, bool PW>
 __device__ __forceinline__ void igemm_tile(
     unsigned char* __restrict__ lds, const ConvGeom& g, const T* __restrict__ x, const T* __restrict__ w,
-    const float* __restrict__ bias, T* __restrict__ y, const Epilogue& ep, int tiles_n,
-    int tiles, float* __restrict__ partial, int slabs_per_split, int splits, int bid) {
+    const float* __restrict__ bias, T* __restrict__ y, T* __restrict__ y2, int o1,
+    const Epilogue& ep, int tiles_n, int tiles, float* __restrict__ partial,
+    int slabs_per_split, int splits, int bid) {
   static_assert(WM * WN == 4, "four waves per workgroup");
   constexpr int WTM = BM / WM, WTN = BN / WN;
   constexpr int TM = WTM / 32, TN = WTN / 32;
@@ -128,14 +129,17 @@ __device__ __forceinline__ void igemm_tile(
       const int r = (j / tiles_n) * 8 + xcd;
       pid = r * tiles_n + j % tiles_n;
       split = 0;
-    } else if (splits >= 8) {
-      const int zs = splits >> 3;  // splits is a multiple of 8
+    } else if (splits >= 8 && (splits & 7) == 0) {
+      const int zs = splits >> 3;
       pid = j / zs;
       split = xcd + 8 * (j - pid * zs);
-    } else {                       // splits is 2 or 4
+    } else if (splits == 2 || splits == 4) {
       const int xpz = 8 / splits;
       split = xcd % splits;
       pid = j * xpz + xcd / splits;
+    } else {                       // any other count: the splits of a tile are neighbours
+      pid = bid / splits;
+      split = bid - pid * splits;
     }
     if (pid >= tiles) return;
   }
@@ -303,69 +307,36 @@ __device__ __forceinline__ void igemm_tile(
 #undef OGLE_LOAD_SLAB
 #undef OGLE_STORE_SLAB
 
-  // Epilogue.  When the row pitch allows 16-byte stores (out_c % 4 == 0) the
-  // accumulators go through a wave-private LDS region to be transposed from the MFMA
-  // layout (a lane holds one column) into rows, so that a wave writes whole
-  // contiguous row segments with 16-byte stores; bias and activation are applied
-  // on the way out.  Otherwise each lane stores its elements one by one.
-  float* const pdst = partial != nullptr ? partial + (long)split * g.m_total * g.o : nullptr;
+  // Epilogue.  Destinations: split-K partial sums go to `partial` (rows of opitch floats,
+  // the channel count rounded up to 4 so that rows stay 16-byte aligned); finished outputs
+  // go to y, or, with a second destination, channels [0, o1) to y (o1 per pixel) and
+  // channels [o1, o) to y2 (o - o1 per pixel).  When the row pitches allow 16-byte stores
+  // the accumulators go through a wave-private LDS region to be transposed from the MFMA
+  // layout (a lane holds one column) into rows, so that a wave writes whole contiguous row
+  // segments with 16-byte stores; bias and activation are applied on the way out.
+  // Otherwise each lane stores its elements one by one (32 lanes cover 128 contiguous
+  // bytes of a row).
+  const int opitch = (g.o + 3) & ~3;
+  const int o2 = g.o - o1;
+  float* const pdst = partial != nullptr ? partial + (long)split * g.m_total * opitch : nullptr;
   constexpr int SROW = WTN + 4;            // floats per staged row (padded)
-  static_assert(4 * 32 * SROW * 4 <= 2 * STAGE, "epilogue staging exceeds the K-loop LDS");
+  constexpr bool STAGED = 4 * 32 * SROW * 4 <= 2 * STAGE;  // staging fits the K-loop LDS
   float* const smw = reinterpret_cast<float*>(lds) + wave * 32 * SROW;
-  if ((g.o & 3) == 0 && (sizeof(T) == 4 || pdst != nullptr)) {
-    constexpr int LPR = WTN / 4;             // lanes covering one staged row
-    constexpr int RPI = 64 / LPR;            // rows one store instruction covers
-    const int cv = lane % LPR;
-    const int rsub = lane / LPR;
-    const int col = n0 + wave_n * WTN + cv * 4;
-    float4 bias4 = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (pdst == nullptr && bias != nullptr && col < g.o)
-      bias4 = *reinterpret_cast<const float4*>(bias + col);
-#pragma unroll
-    for (int i = 0; i < TM; ++i) {
-#pragma unroll
-      for (int j = 0; j < TN; ++j)
-#pragma unroll
-        for (int r = 0; r < 16; ++r)
-          smw[((r >> 2) * 8 + lh * 4 + (r & 3)) * SROW + j * 32 + l32] = acc[i][j][r];
-#pragma unroll
-      for (int it = 0; it < 32 / RPI; ++it) {
-        const int row = it * RPI + rsub;
-        float4 v = *reinterpret_cast<const float4*>(smw + row * SROW + cv * 4);
-        const int grow = m0 + wave_m * WTM + i * 32 + row;
-        if (grow < g.m_total && col < g.o) {
-          if (pdst != nullptr) {
-            *reinterpret_cast<float4*>(pdst + (long)grow * g.o + col) = v;
-          } else {
-            v.x = apply_epilogue(v.x + bias4.x, ep);
-            v.y = apply_epilogue(v.y + bias4.y, ep);
-            v.z = apply_epilogue(v.z + bias4.z, ep);
-            v.w = apply_epilogue(v.w + bias4.w, ep);
-            *reinterpret_cast<float4*>(reinterpret_cast<float*>(y) + (long)grow * g.o + col) = v;
-          }
-        }
-      }
-    }
-    return;
-  }
-  if constexpr (sizeof(T) == 2) {
-    if ((g.o & 7) == 0) {
-      // fp16 output: the same staging, a lane then takes eight consecutive channels
-      // of a row and stores them as one 16-byte vector of halves
-      constexpr int LPR = WTN / 8;
-      constexpr int RPI = 64 / LPR;
+  if constexpr (STAGED) {
+    if (pdst != nullptr || (sizeof(T) == 4 && (o1 & 3) == 0 && (o2 & 3) == 0)) {
+      constexpr int LPR = WTN / 4;             // lanes covering one staged row
+      constexpr int RPI = 64 / LPR;            // rows one store instruction covers
       const int cv = lane % LPR;
       const int rsub = lane / LPR;
-      const int col = n0 + wave_n * WTN + cv * 8;
-      float bias8[8];
-#pragma unroll
-      for (int q = 0; q < 8; ++q) bias8[q] = 0.f;
-      if (bias != nullptr && col < g.o) {
-        const float4 b0 = *reinterpret_cast<const float4*>(bias + col);
-        const float4 b1 = *reinterpret_cast<const float4*>(bias + col + 4);
-        bias8[0] = b0.x; bias8[1] = b0.y; bias8[2] = b0.z; bias8[3] = b0.w;
-        bias8[4] = b1.x; bias8[5] = b1.y; bias8[6] = b1.z; bias8[7] = b1.w;
-      }
+      const int col = n0 + wave_n * WTN + cv * 4;
+      float4 bias4 = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (pdst == nullptr && bias != nullptr && col < g.o)
+        bias4 = *reinterpret_cast<const float4*>(bias + col);
+      // row pitch and first column of the destination this lane's four channels lie in
+      const bool second = pdst == nullptr && col >= o1;
+      const int dpitch = pdst != nullptr ? opitch : (second ? o2 : o1);
+      const int dcol = second ? col - o1 : col;
+      float* const dbase = pdst != nullptr ? pdst : reinterpret_cast<float*>(second ? y2 : y);
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
 #pragma unroll
@@ -376,22 +347,66 @@ __device__ __forceinline__ void igemm_tile(
 #pragma unroll
         for (int it = 0; it < 32 / RPI; ++it) {
           const int row = it * RPI + rsub;
-          const float4 v0 = *reinterpret_cast<const float4*>(smw + row * SROW + cv * 8);
-          const float4 v1 = *reinterpret_cast<const float4*>(smw + row * SROW + cv * 8 + 4);
+          float4 v = *reinterpret_cast<const float4*>(smw + row * SROW + cv * 4);
           const int grow = m0 + wave_m * WTM + i * 32 + row;
           if (grow < g.m_total && col < g.o) {
-            const float f[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
-            uint4 packed;
-            __half2* h = reinterpret_cast<__half2*>(&packed);
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
-              h[q] = __floats2half2_rn(apply_epilogue(f[2 * q] + bias8[2 * q], ep),
-                                       apply_epilogue(f[2 * q + 1] + bias8[2 * q + 1], ep));
-            *reinterpret_cast<uint4*>(reinterpret_cast<__half*>(y) + (long)grow * g.o + col) = packed;
+            if (pdst == nullptr) {
+              v.x = apply_epilogue(v.x + bias4.x, ep);
+              v.y = apply_epilogue(v.y + bias4.y, ep);
+              v.z = apply_epilogue(v.z + bias4.z, ep);
+              v.w = apply_epilogue(v.w + bias4.w, ep);
+            }
+            *reinterpret_cast<float4*>(dbase + (long)grow * dpitch + dcol) = v;
           }
         }
       }
       return;
+    }
+    if constexpr (sizeof(T) == 2) {
+      if ((g.o & 7) == 0 && y2 == nullptr) {
+        // fp16 output: the same staging, a lane then takes eight consecutive channels
+        // of a row and stores them as one 16-byte vector of halves
+        constexpr int LPR = WTN / 8;
+        constexpr int RPI = 64 / LPR;
+        const int cv = lane % LPR;
+        const int rsub = lane / LPR;
+        const int col = n0 + wave_n * WTN + cv * 8;
+        float bias8[8];
+#pragma unroll
+        for (int q = 0; q < 8; ++q) bias8[q] = 0.f;
+        if (bias != nullptr && col < g.o) {
+          const float4 b0 = *reinterpret_cast<const float4*>(bias + col);
+          const float4 b1 = *reinterpret_cast<const float4*>(bias + col + 4);
+          bias8[0] = b0.x; bias8[1] = b0.y; bias8[2] = b0.z; bias8[3] = b0.w;
+          bias8[4] = b1.x; bias8[5] = b1.y; bias8[6] = b1.z; bias8[7] = b1.w;
+        }
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+              smw[((r >> 2) * 8 + lh * 4 + (r & 3)) * SROW + j * 32 + l32] = acc[i][j][r];
+#pragma unroll
+          for (int it = 0; it < 32 / RPI; ++it) {
+            const int row = it * RPI + rsub;
+            const float4 v0 = *reinterpret_cast<const float4*>(smw + row * SROW + cv * 8);
+            const float4 v1 = *reinterpret_cast<const float4*>(smw + row * SROW + cv * 8 + 4);
+            const int grow = m0 + wave_m * WTM + i * 32 + row;
+            if (grow < g.m_total && col < g.o) {
+              const float f[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+              uint4 packed;
+              __half2* h = reinterpret_cast<__half2*>(&packed);
+#pragma unroll
+              for (int q = 0; q < 4; ++q)
+                h[q] = __floats2half2_rn(apply_epilogue(f[2 * q] + bias8[2 * q], ep),
+                                         apply_epilogue(f[2 * q + 1] + bias8[2 * q + 1], ep));
+              *reinterpret_cast<uint4*>(reinterpret_cast<__half*>(y) + (long)grow * g.o + col) = packed;
+            }
+          }
+        }
+        return;
+      }
     }
   }
 #pragma unroll
@@ -399,6 +414,9 @@ __device__ __forceinline__ void igemm_tile(
     const int col = n0 + wave_n * WTN + j * 32 + l32;
     if (col >= g.o) continue;
     const float bv = (pdst == nullptr && bias != nullptr) ? bias[col] : 0.f;
+    const bool second = col >= o1;
+    T* const dst = second ? y2 + (col - o1) : y + col;
+    const int dpitch = second ? o2 : o1;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
       const int rbase = m0 + wave_m * WTM + i * 32 + lh * 4;
@@ -407,9 +425,9 @@ __device__ __forceinline__ void igemm_tile(
         const int row = rbase + (r >> 2) * 8 + (r & 3);
         if (row >= g.m_total) continue;
         if (pdst != nullptr) {
-          pdst[(long)row * g.o + col] = acc[i][j][r];
+          pdst[(long)row * opitch + col] = acc[i][j][r];
         } else {
-          y[(long)row * g.o + col] = from_f32<T>(apply_epilogue(acc[i][j][r] + bv, ep));
+          dst[(long)row * dpitch] = from_f32<T>(apply_epilogue(acc[i][j][r] + bv, ep));
         }
       }
     }
@@ -423,6 +441,8 @@ struct IgemmProblem {
   const void* w;
   const float* bias;
   void* y;
+  void* y2;  // second destination for channels [o1, o), or nullptr
+  int o1;    // channels that go to y (== g.o without a second destination)
   Epilogue ep;
   int tiles_n, tiles;
   float* partial;
@@ -435,8 +455,9 @@ __global__ __launch_bounds__(256) void conv_igemm_kernel(IgemmProblem p) {
   __shared__ __attribute__((aligned(16))) unsigned char lds[igemm_lds_bytes<BM, BN, ROWB>()];
   igemm_tile<T, BM, BN, WM, WN, ROWB, PW>(lds, p.g, static_cast<const T*>(p.x),
                                           static_cast<const T*>(p.w), p.bias,
-                                          static_cast<T*>(p.y), p.ep, p.tiles_n, p.tiles, p.partial,
-                                          p.slabs_per_split, p.splits, (int)blockIdx.x);
+                                          static_cast<T*>(p.y), static_cast<T*>(p.y2), p.o1, p.ep,
+                                          p.tiles_n, p.tiles, p.partial, p.slabs_per_split, p.splits,
+                                          (int)blockIdx.x);
 }
 
 // Several independent convolutions in one grid: blocks [first[i], first[i+1]) work
@@ -457,15 +478,16 @@ __global__ __launch_bounds__(256) void conv_igemm_group_kernel(IgemmGroup grp) {
   const IgemmProblem& p = grp.p[i];
   igemm_tile<T, BM, BN, WM, WN, ROWB, PW>(lds, p.g, static_cast<const T*>(p.x),
                                           static_cast<const T*>(p.w), p.bias,
-                                          static_cast<T*>(p.y), p.ep, p.tiles_n, p.tiles, p.partial,
-                                          p.slabs_per_split, p.splits,
+                                          static_cast<T*>(p.y), static_cast<T*>(p.y2), p.o1, p.ep,
+                                          p.tiles_n, p.tiles, p.partial, p.slabs_per_split, p.splits,
                                           (int)blockIdx.x - grp.first[i]);
 }
 
 template <typename T, bool PW, int TS, int U>
 __device__ __forceinline__ void igemm_wave_tile(
     float* __restrict__ red, const ConvGeom& g, const T* __restrict__ x, const T* __restrict__ w,
-    const float* __restrict__ bias, T* __restrict__ y, const Epilogue& ep, int tiles_n, int bid);
+    const float* __restrict__ bias, T* __restrict__ y, T* __restrict__ y2, int o1, const Epilogue& ep,
+    int tiles_n, int bid);
 
 // A group whose members differ in tile shape (64x64 or 128x32) or in being
 // pointwise: each workgroup takes the code path of its own problem.  The branch is
@@ -485,7 +507,8 @@ __global__ __launch_bounds__(256) void conv_igemm_mixed_kernel(IgemmGroup grp) {
   case V:                                                                                       \
     igemm_tile<T, BM, BN, WM, WN, ROWB, PW>(lds, p.g, static_cast<const T*>(p.x),               \
                                             static_cast<const T*>(p.w), p.bias,                 \
-                                            static_cast<T*>(p.y), p.ep, p.tiles_n, p.tiles,     \
+                                            static_cast<T*>(p.y), static_cast<T*>(p.y2), p.o1,  \
+                                            p.ep, p.tiles_n, p.tiles,                           \
                                             p.partial, p.slabs_per_split, p.splits, bid);       \
     break;
   switch (p.variant) {
@@ -497,8 +520,8 @@ __global__ __launch_bounds__(256) void conv_igemm_mixed_kernel(IgemmGroup grp) {
   case V:                                                                                       \
     /* two steps in flight only: the group kernel's register budget is the 64x64 tile's */      \
     igemm_wave_tile<T, PW, TS, 2>(reinterpret_cast<float*>(lds), p.g, static_cast<const T*>(p.x), \
-                               static_cast<const T*>(p.w), p.bias, static_cast<T*>(p.y), p.ep,   \
-                               p.tiles_n, bid);                                                 \
+                               static_cast<const T*>(p.w), p.bias, static_cast<T*>(p.y),         \
+                               static_cast<T*>(p.y2), p.o1, p.ep, p.tiles_n, bid);               \
     break;
     OGLE_MIXED_WAVE(4, false, 32)
     OGLE_MIXED_WAVE(5, true, 32)
@@ -577,7 +600,8 @@ constexpr int kWaveRedBytes = 4 * 32 * 36 * 4;  // four staged 32x32 partial til
 template <typename T, bool PW, int TS, int U>
 __device__ __forceinline__ void igemm_wave_tile(
     float* __restrict__ red, const ConvGeom& g, const T* __restrict__ x, const T* __restrict__ w,
-    const float* __restrict__ bias, T* __restrict__ y, const Epilogue& ep, int tiles_n, int bid) {
+    const float* __restrict__ bias, T* __restrict__ y, T* __restrict__ y2, int o1, const Epilogue& ep,
+    int tiles_n, int bid) {
   typedef WaveMma<T, TS> M;
   constexpr int ESZ = (int)sizeof(T);
   constexpr int VE = 16 / ESZ;          // elements per 16-byte load
@@ -718,6 +742,18 @@ __device__ __forceinline__ void igemm_wave_tile(
   for (int q = 0; q < 4; ++q) {
     if (gcol + q < g.o) v[q] = apply_epilogue(v[q] + (bias != nullptr ? bias[gcol + q] : 0.f), ep);
   }
+  if (y2 != nullptr) {
+    // two destinations: element by element, each channel to its own tensor
+    const int o2 = g.o - o1;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int c = gcol + q;
+      if (c >= g.o) continue;
+      if (c < o1) y[(long)grow * o1 + c] = from_f32<T>(v[q]);
+      else y2[(long)grow * o2 + (c - o1)] = from_f32<T>(v[q]);
+    }
+    return;
+  }
   T* dst = y + (long)grow * g.o + gcol;
   if ((g.o & 3) == 0) {
     if constexpr (sizeof(T) == 4) {
@@ -740,15 +776,17 @@ template <typename T, bool PW, int TS>
 __global__ __launch_bounds__(256) void conv_igemm_wave_kernel(IgemmProblem p) {
   __shared__ __attribute__((aligned(16))) float red[kWaveRedBytes / 4];
   igemm_wave_tile<T, PW, TS, 4>(red, p.g, static_cast<const T*>(p.x), static_cast<const T*>(p.w),
-                             p.bias, static_cast<T*>(p.y), p.ep, p.tiles_n, (int)blockIdx.x);
+                             p.bias, static_cast<T*>(p.y), static_cast<T*>(p.y2), p.o1, p.ep, p.tiles_n,
+                             (int)blockIdx.x);
 }
 
 struct ReduceProblem {
-  const float* partial;
+  const float* partial;  // [splits][m][opitch]
   const float* bias;
   void* y;
-  long mn;
-  int o, splits;
+  void* y2;   // second destination for channels [o1, o), or nullptr
+  long mn;    // m * o output elements
+  int o, o1, opitch, splits;
   Epilogue ep;
   int lanes;  // lanes per output element (1, 2, 4 or 8)
 };
@@ -769,15 +807,21 @@ __device__ __forceinline__ void splitk_reduce_block(const ReduceProblem& r, int 
   const long idx = (long)bid * (blockDim.x / LANES) + threadIdx.x / LANES;
   const bool live = idx < r.mn;  // dead lanes still take part in the shuffles
   float acc = 0.f;
+  const long row = idx / r.o;
+  const int col = (int)(idx - row * r.o);
   if (live) {
+    const long src = row * r.opitch + col;
+    const long zstride = (r.mn / r.o) * r.opitch;
 #pragma unroll 4
-    for (int z = q; z < r.splits; z += LANES) acc += r.partial[(long)z * r.mn + idx];
+    for (int z = q; z < r.splits; z += LANES) acc += r.partial[(long)z * zstride + src];
   }
 #pragma unroll
   for (int d = 1; d < LANES; d <<= 1) acc += __shfl_xor(acc, d, 64);
   if (live && q == 0) {
-    if (r.bias != nullptr) acc += r.bias[idx % r.o];
-    static_cast<T*>(r.y)[idx] = from_f32<T>(apply_epilogue(acc, r.ep));
+    if (r.bias != nullptr) acc += r.bias[col];
+    const T out = from_f32<T>(apply_epilogue(acc, r.ep));
+    if (col < r.o1) static_cast<T*>(r.y)[row * r.o1 + col] = out;
+    else static_cast<T*>(r.y2)[row * (r.o - r.o1) + (col - r.o1)] = out;
   }
 }
 
@@ -804,10 +848,11 @@ __global__ __launch_bounds__(256) void splitk_reduce_group_kernel(ReduceGroup gr
 
 // Tile configurations (BM, BN, waves along M, waves along N).
 enum TileCfg {
-  CFG_128x128 = 0, CFG_128x64 = 1, CFG_64x64 = 2, CFG_128x32 = 3, CFG_WAVE32 = 4, CFG_WAVE16 = 5
+  CFG_128x128 = 0, CFG_128x64 = 1, CFG_64x64 = 2, CFG_128x32 = 3, CFG_WAVE32 = 4, CFG_WAVE16 = 5,
+  CFG_128x96 = 6, CFG_128x160 = 7  // all output channels of a narrow, long-K problem in one tile
 };
-constexpr int kCfgBM[] = {128, 128, 64, 128, 32, 16};
-constexpr int kCfgBN[] = {128, 64, 64, 32, 32, 16};
+constexpr int kCfgBM[] = {128, 128, 64, 128, 32, 16, 128, 128};
+constexpr int kCfgBN[] = {128, 64, 64, 32, 32, 16, 96, 160};
 
 struct IgemmPlan {
   int cfg;
@@ -822,6 +867,7 @@ constexpr long kComputeUnits = 256;
 constexpr int kRowBytesF32 = 64;   // bytes of K per tile row per slab, fp32
 
 bool is_pointwise(const OgleConvArgs& a);
+bool is_wave(int cfg);
 
 // Picks the output tile and the K split.  Problems with few output
 // tiles but a long contraction (the SSD heads, the small feature maps) are split
@@ -844,7 +890,15 @@ IgemmPlan plan_igemm(const OgleConvArgs& a, long m, bool allow_split) {
   // 64x64 tile is bound by LDS traffic and instruction issue; 128x128 pays off as soon
   // as its tiles cover the compute units.
   const long big_tiles_wanted = a.dtype == OGLE_F16 ? kComputeUnits : 4 * kComputeUnits;
-  if (a.out_c <= 32) {
+  // Narrow outputs with a long contraction (the SSD heads, box and class head of a feature
+  // map fused: 75 or 150 channels, K = 2304 ... 9216): one tile column holds every output
+  // channel, so the input is gathered once instead of once per 64-channel tile column, and
+  // 96 / 160 columns waste far less of the MFMA work than two or three 64-wide tiles.
+  const bool narrow_long = a.dtype == OGLE_F32 && p.ktiles >= 32 &&
+                           ((a.out_c > 64 && a.out_c <= 96) || (a.out_c > 128 && a.out_c <= 160));
+  if (narrow_long) {
+    p.cfg = a.out_c <= 96 ? CFG_128x96 : CFG_128x160;
+  } else if (a.out_c <= 32) {
     p.cfg = CFG_128x32;
   } else if (a.out_c > 64 && tiles(CFG_128x128) >= big_tiles_wanted) {
     p.cfg = CFG_128x128;
@@ -854,7 +908,24 @@ IgemmPlan plan_igemm(const OgleConvArgs& a, long m, bool allow_split) {
   p.splits = 1;
   const long t = tiles(p.cfg);
   long sp = 1;
-  if (allow_split && 2 * t <= kComputeUnits && p.ktiles >= 8) {
+  bool exact_split = false;  // sp was chosen by the search below: any count is fine
+  if (allow_split && narrow_long && t < 2 * kComputeUnits) {
+    // One tile column, few tile rows, a long K: the K split decides how evenly the chip is
+    // filled.  Workgroups are (tile, K range) pairs dealt to 256 compute units, each doing
+    // ceil(ktiles / s) slabs plus a fixed cost (first loads, epilogue: about `fixed` slabs);
+    // take the s with the shortest estimated time, partial-sum traffic as the tie break.
+    const double fixed = p.cfg == CFG_128x96 ? 6.0 : 4.0;
+    double best = 1e30;
+    for (long s = 1; s <= 64 && p.ktiles / s >= 8; ++s) {
+      const long rounds = (t * s + kComputeUnits - 1) / kComputeUnits;
+      const double cost = (double)rounds * ((double)((p.ktiles + s - 1) / s) + fixed) + 0.25 * (double)s;
+      if (cost < best - 1e-9) {
+        best = cost;
+        sp = s;
+      }
+    }
+    exact_split = true;
+  } else if (allow_split && 2 * t <= kComputeUnits && p.ktiles >= 8) {
     // too few tiles to occupy every compute unit: about three workgroups per unit,
     // at least four slabs per split
     const long want = (3 * kComputeUnits + t - 1) / t;
@@ -870,7 +941,8 @@ IgemmPlan plan_igemm(const OgleConvArgs& a, long m, bool allow_split) {
   }
   if (sp > 64) sp = 64;
   // the kernel's XCD-aware work layout wants a divisor or a multiple of 8
-  if (sp >= 8) sp -= sp % 8;
+  if (exact_split) {}
+  else if (sp >= 8) sp -= sp % 8;
   else if (sp >= 4) sp = 4;
   else if (sp >= 2) sp = 2;
   if (sp >= 2) p.splits = (int)sp;
@@ -890,7 +962,9 @@ IgemmPlan plan_igemm(const OgleConvArgs& a, long m, bool allow_split) {
     const long t32 = tiles(CFG_WAVE32), t16 = tiles(CFG_WAVE16);
     const bool small16 = (pw && k_total <= 1024 && t16 <= 2 * kComputeUnits) ||
                          (k_total <= 1536 && t16 <= kComputeUnits / 2);
-    if (would_split && !small16 && k_total <= (pw ? 1024 : 512) && t32 >= kComputeUnits / 2 &&
+    if (narrow_long) {
+      // stays on the wide tile
+    } else if (would_split && !small16 && k_total <= (pw ? 1024 : 512) && t32 >= kComputeUnits / 2 &&
         t32 <= 4 * kComputeUnits) {
       p.cfg = CFG_WAVE32;
       p.splits = 1;
@@ -899,11 +973,14 @@ IgemmPlan plan_igemm(const OgleConvArgs& a, long m, bool allow_split) {
       p.splits = 1;
     }
   }
+  if (const char* e = getenv("OGLE_DEBUG_SPLITS")) { if (allow_split && !is_wave(p.cfg)) p.splits = atoi(e); }  // TEMP
   p.slabs_per_split = (p.ktiles + p.splits - 1) / p.splits;
   if (p.splits > 1) p.slabs_per_split += p.slabs_per_split & 1;  // the K loop runs slab pairs
   // (a split past the end of K would only add zeros; rounding splits down keeps the
   // divisor-or-multiple-of-8 shape, so empty splits are simply avoided by the cap above)
-  p.workspace_bytes = p.splits > 1 ? (size_t)p.splits * (size_t)m * a.out_c * sizeof(float) : 0;
+  // partial sums are kept in rows of the channel count rounded up to four
+  p.workspace_bytes =
+      p.splits > 1 ? (size_t)p.splits * (size_t)m * ((a.out_c + 3) & ~3) * sizeof(float) : 0;
   return p;
 }
 
@@ -915,7 +992,7 @@ int tile_bn(int cfg) { return kCfgBN[cfg]; }
 unsigned grid_blocks(const IgemmPlan& p, int tiles_m, int tiles_n) {
   const int tiles = tiles_m * tiles_n;
   if (p.splits == 1) return 8u * (unsigned)((tiles_m + 7) / 8) * (unsigned)tiles_n;
-  if (p.splits >= 8) return (unsigned)tiles * (unsigned)p.splits;
+  if (p.splits != 2 && p.splits != 4) return (unsigned)tiles * (unsigned)p.splits;
   const int xpz = 8 / p.splits;
   return 8u * (unsigned)((tiles + xpz - 1) / xpz);
 }
@@ -973,6 +1050,8 @@ Prepared prepare(const OgleConvArgs& a, long m, const IgemmPlan& p) {
   out.prob.w = a.filter_dev;
   out.prob.bias = a.bias_dev;
   out.prob.y = a.output_dev;
+  out.prob.y2 = a.output2_dev;
+  out.prob.o1 = a.output2_dev != nullptr ? a.out_c_split : a.out_c;
   out.prob.ep = make_epilogue(a.act, a.min_value, a.max_value, a.act_variant);
   out.prob.tiles_n = tiles_n;
   out.prob.tiles = tiles_m * tiles_n;
@@ -991,8 +1070,8 @@ Prepared prepare(const OgleConvArgs& a, long m, const IgemmPlan& p) {
     // enough lanes per output that the grid still has about a thousand waves
     int lanes = 1;
     while (lanes < 8 && lanes * 2 <= p.splits && mn * lanes < 64L * 1024) lanes *= 2;
-    out.red = ReduceProblem{out.prob.partial, a.bias_dev, a.output_dev, mn, g.o, p.splits,
-                            out.prob.ep, lanes};
+    out.red = ReduceProblem{out.prob.partial, a.bias_dev, a.output_dev, a.output2_dev, mn, g.o,
+                            out.prob.o1, (g.o + 3) & ~3, p.splits, out.prob.ep, lanes};
     out.reduce_lanes = lanes;
     out.reduce_grid = (unsigned)((mn * lanes + 255) / 256);
   }
@@ -1026,6 +1105,12 @@ Prepared prepare(const OgleConvArgs& a, long m, const IgemmPlan& p) {
       break;                                                                                 \
     case CFG_64x64:                                                                          \
       hipLaunchKernelGGL((K<T, 64, 64, 2, 2, ROWB, PW>), dim3(grid), dim3(256), 0, s, arg);   \
+      break;                                                                                 \
+    case CFG_128x96:                                                                         \
+      hipLaunchKernelGGL((K<T, 128, 96, 4, 1, ROWB, PW>), dim3(grid), dim3(256), 0, s, arg);  \
+      break;                                                                                 \
+    case CFG_128x160:                                                                        \
+      hipLaunchKernelGGL((K<T, 128, 160, 4, 1, ROWB, PW>), dim3(grid), dim3(256), 0, s, arg); \
       break;                                                                                 \
     default:                                                                                 \
       hipLaunchKernelGGL((K<T, 128, 32, 4, 1, ROWB, PW>), dim3(grid), dim3(256), 0, s, arg);  \

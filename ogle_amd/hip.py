@@ -52,6 +52,7 @@ class ConvArgs(ctypes.Structure):
         ("act", ctypes.c_int32), ("min_value", ctypes.c_float), ("max_value", ctypes.c_float),
         ("act_variant", ctypes.c_int32), ("dtype", ctypes.c_int32),
         ("workspace_dev", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
+        ("output2_dev", ctypes.c_void_p), ("out_c_split", ctypes.c_int32),
     ]
 
 
@@ -221,4 +222,4 @@ def conv_args(x_ptr, w_ptr, b_ptr, y_ptr, n, h, w, c, o, k, stride=1, pad=0, dil
               act=ACT_NONE, minv=0.0, maxv=0.0, variant=VARIANT_NHWC4, dtype=F32):
     return ConvArgs(x_ptr, w_ptr, b_ptr, y_ptr, n, h, w, c,
                     out_size(h, k, stride, pad, dilation), out_size(w, k, stride, pad, dilation), o,
-                    k, stride, pad, dilation, group, act, minv, maxv, variant, dtype, None, 0)
+                    k, stride, pad, dilation, group, act, minv, maxv, variant, dtype, None, 0, None, 0)

@@ -91,6 +91,13 @@ int32_t ogle_rt_load_bytes(OgleSession* s, const void* data, size_t size) {
   });
 }
 
+int32_t ogle_rt_set_fuse_siblings(OgleSession* s, int32_t on) {
+  return (int32_t)Guard([&]() -> int64_t {
+    s->session->set_fuse_siblings(on != 0);
+    return 0;
+  });
+}
+
 int32_t ogle_rt_graph_captured(OgleSession* s, int32_t slot) {
   if (s == nullptr || slot < 0 || slot >= FBOSession::kGraphSlots) return -1;
   return s->session->graph_captured(slot) ? 1 : 0;

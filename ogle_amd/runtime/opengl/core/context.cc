@@ -66,21 +66,24 @@ bool Overlap(const MemRange& a, const MemRange& b) {
 }
 }  // namespace
 
-void Context::ConvRanges(const OgleConvArgs& c, MemRange reads[3], MemRange writes[2]) {
+void Context::ConvRanges(const OgleConvArgs& c, MemRange reads[3], MemRange writes[3]) {
   const size_t esz = ElemBytes(c);
   const int group = c.group > 0 ? c.group : 1;
   reads[0] = {c.input_dev, static_cast<size_t>(c.n) * c.in_h * c.in_w * c.in_c * esz};
   reads[1] = {c.filter_dev, static_cast<size_t>(c.out_c) * c.kernel_size * c.kernel_size *
                                 (c.in_c / group) * esz};
   reads[2] = {c.bias_dev, c.bias_dev != nullptr ? static_cast<size_t>(c.out_c) * sizeof(float) : 0};
-  writes[0] = {c.output_dev, static_cast<size_t>(c.n) * c.out_h * c.out_w * c.out_c * esz};
+  const size_t pixels = static_cast<size_t>(c.n) * c.out_h * c.out_w;
+  const int first = c.output2_dev != nullptr ? c.out_c_split : c.out_c;
+  writes[0] = {c.output_dev, pixels * first * esz};
   writes[1] = {c.workspace_dev, c.workspace_dev != nullptr ? c.workspace_bytes : 0};
+  writes[2] = {c.output2_dev, c.output2_dev != nullptr ? pixels * (c.out_c - first) * esz : 0};
 }
 
 bool Context::Conflicts(const OgleConvArgs* pending, int n_pending, const MemRange* reads,
                         int n_reads, const MemRange* writes, int n_writes) {
   for (int p = 0; p < n_pending; ++p) {
-    MemRange pr[3], pw[2];
+    MemRange pr[3], pw[3];
     ConvRanges(pending[p], pr, pw);
     // read after write
     for (int i = 0; i < n_reads; ++i)
@@ -99,10 +102,10 @@ bool Context::Conflicts(const OgleConvArgs* pending, int n_pending, const MemRan
 
 void Context::BeforeConv(const OgleConvArgs& args) {
   if (pending_.empty()) return;
-  MemRange reads[3], writes[2];
+  MemRange reads[3], writes[3];
   ConvRanges(args, reads, writes);
   if (pending_.size() >= 16 ||
-      Conflicts(pending_.data(), static_cast<int>(pending_.size()), reads, 3, writes, 2))
+      Conflicts(pending_.data(), static_cast<int>(pending_.size()), reads, 3, writes, 3))
     Flush();
 }
 
@@ -285,9 +288,9 @@ void Program::Check(int32_t status, const char* what) const {
 }
 void Program::RunConv2d(const OgleConvArgs& a) const { context_->EnqueueConv(a); }
 void Program::RunDepthwise(const OgleConvArgs& a) const {
-  MemRange reads[3], writes[2];
+  MemRange reads[3], writes[3];
   Context::ConvRanges(a, reads, writes);
-  context_->BeforeLaunch(reads, 3, writes, 2);
+  context_->BeforeLaunch(reads, 3, writes, 3);
   Check(ogle_hip_dwconv2d(&a, context_->stream()), "ogle_hip_dwconv2d");
 }
 void Program::RunPointwise(const OgleConvArgs& a) const {

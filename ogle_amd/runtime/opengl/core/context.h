@@ -67,8 +67,9 @@ class Context {
   // these reads and writes must wait for one of `pending`.
   static bool Conflicts(const OgleConvArgs* pending, int n_pending, const MemRange* reads,
                         int n_reads, const MemRange* writes, int n_writes);
-  // The ranges a convolution reads (input, filter, bias) and writes (output, workspace).
-  static void ConvRanges(const OgleConvArgs& a, MemRange reads[3], MemRange writes[2]);
+  // The ranges a convolution reads (input, filter, bias) and writes (output, workspace,
+  // second output).
+  static void ConvRanges(const OgleConvArgs& a, MemRange reads[3], MemRange writes[3]);
   void EnqueueConv(const OgleConvArgs& args);
   void Flush();
   void set_batching(bool on) {

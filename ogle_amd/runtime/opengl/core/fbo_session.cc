@@ -26,6 +26,8 @@ FBOSession::FBOSession(Context* context) : context_(context) {
   context_->Reset();
   const char* env = std::getenv("OGLE_FILE_ORDER");
   if (env != nullptr && env[0] != '\0' && env[0] != '0') reorder_ = false;
+  env = std::getenv("OGLE_NO_SIBLING_FUSION");
+  if (env != nullptr && env[0] != '\0' && env[0] != '0') fuse_siblings_ = false;
 }
 
 FBOSession::~FBOSession() {
@@ -154,9 +156,29 @@ void FBOSession::Setup(const NamedTensorList& inputs_cpu) {
       UpdateKernelReady(kernel);
     }
   }
+  FuseSiblings();
   PlaceInputsInOutputs();
   BuildSchedule();
   finalized_ = true;
+}
+
+// Live nodes that read the same tensor are offered to each other (Kernel::TryAbsorb): a
+// pair that agrees runs as one launch from then on.  File order is kept: the absorbing
+// node is the earlier one, so everything that reads either output still comes after the
+// launch that fills it.
+void FBOSession::FuseSiblings() {
+  if (!fuse_siblings_) return;
+  for (size_t i = 0; i < kernels_.size(); ++i) {
+    Kernel* a = kernels_[i].get();
+    if (CheckKernelReady(a) || a->absorbed() || a->input_tensor_indexes_.empty()) continue;
+    for (size_t j = i + 1; j < kernels_.size(); ++j) {
+      Kernel* b = kernels_[j].get();
+      if (CheckKernelReady(b) || b->absorbed() || b->input_tensor_indexes_.empty()) continue;
+      if (a->input_tensor_indexes_[0] != b->input_tensor_indexes_[0]) continue;
+      if (a->kernel_type() != b->kernel_type()) continue;
+      if (a->TryAbsorb(b)) break;
+    }
+  }
 }
 
 // Where a node's output is nothing but its inputs back to back (a Concat with a single
@@ -293,7 +315,11 @@ void FBOSession::BuildSchedule() {
     is_view[i] = view;
     for (size_t j = 0; j < k->output_tensor_indexes_.size(); ++j) {
       int src = i;
-      if (view) {
+      if (k->absorbed()) {
+        // filled by the sibling's launch, which comes earlier in the file
+        for (int q = 0; q < i; ++q)
+          if (live[q] == k->absorbed_by()) src = q;
+      } else if (view) {
         const int in = k->input_tensor_indexes_[k->OutputAliasesInput(static_cast<int>(j))];
         auto it = producer.find(in);
         src = it != producer.end() ? it->second : -1;
@@ -314,7 +340,7 @@ void FBOSession::BuildSchedule() {
       return false;
     };
     for (int i = 0; i < n; ++i) {
-      if (is_view[i]) continue;
+      if (is_view[i] || live[i]->absorbed()) continue;
       const bool defer = live[i]->Deferrable();
       if (!pending.empty() &&
           (depends_on_pending(i) || (defer && static_cast<int>(pending.size()) >= kMaxBatch))) {

@@ -76,11 +76,17 @@ class FBOSession {
   // Takes effect at the first Run.
   void set_reorder(bool on) { reorder_ = on; }
   bool reorder() const { return reorder_; }
+  // Whether Setup may run two Conv nodes that read the same tensor with the same
+  // attributes as one launch (OGLE_NO_SIBLING_FUSION=1 also switches it off).  Takes
+  // effect at the first Run.
+  void set_fuse_siblings(bool on) { fuse_siblings_ = on; }
+  bool fuse_siblings() const { return fuse_siblings_; }
   // Node names in the order Compute() issues them (after the first Run).
   std::vector<std::string> IssueOrder() const;
 
  private:
   bool CheckKernelReady(const Kernel* kernel);
+  void FuseSiblings();
   void PlaceInputsInOutputs();
   void BuildSchedule();
   void UpdateKernelReady(const Kernel* kernel);
@@ -96,6 +102,7 @@ class FBOSession {
   std::vector<bool> ready_;
   bool allow_resized_ = false;
   bool reorder_ = true;
+  bool fuse_siblings_ = true;
   std::vector<Kernel*> order_;  // the per-pass kernels in issue order (not owned)
   IntList default_input_sizes_;
   void* graph_[kGraphSlots] = {nullptr, nullptr};       // hipGraph_t

@@ -70,6 +70,19 @@ class Kernel {
     return -1;
   }
 
+  // Sibling fusion, not in the reference: two nodes that read the same tensor with the
+  // same attributes may run as one launch that fetches the input once (the box and the
+  // class head of an SSD feature map).  TryAbsorb asks this node to take over `other`'s
+  // work as well; on success `other` has been told (Absorbed) and its Compute does
+  // nothing from then on, this node's Compute also fills `other`'s output.  Called by the
+  // executor once all tensors are bound, before the schedule is built.
+  virtual bool TryAbsorb(Kernel* other) {
+    (void)other;
+    return false;
+  }
+  bool absorbed() const { return absorbed_by_ != nullptr; }
+  const Kernel* absorbed_by() const { return absorbed_by_; }
+
   // Scheduling hints, also not in the reference (one draw call per node, in file
   // order).  The launch of a deferrable node may be held back and merged with other
   // deferrable nodes into one grid; WorkEstimate is its device work in multiply-adds
@@ -94,6 +107,7 @@ class Kernel {
   std::string kernel_type_;
   std::string build_options_;
   FBOSession* session_ = nullptr;
+  Kernel* absorbed_by_ = nullptr;  // the sibling that does this node's work, if any
 };
 
 }  // namespace opengl

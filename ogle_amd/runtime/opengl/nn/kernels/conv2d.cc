@@ -105,12 +105,74 @@ void Conv2DKernel::PackFilter(const Tensor* filter) {
   const IntList& fs = filter->shape();
   const int layout = variant_ == kDepthwise ? OGLE_FILTER_HWC : OGLE_FILTER_OHWI;
   if (variant_ == kDepthwise) CHECK_EQ(fs[1], 1) << "depthwise filters have one input channel";
-  packed_filter_.reset(new Tensor(Tensor::DT_FLOAT, fs, Tensor::DEVICE_BUFFER, filter->dformat()));
-  const int32_t st =
+  IntList packed_shape = fs;
+  const Tensor* filter2 = sibling_ != nullptr ? sibling_->input_tensors_[1] : nullptr;
+  if (filter2 != nullptr) packed_shape[0] += filter2->shape()[0];  // OHWI: output channels are rows
+  packed_filter_.reset(new Tensor(Tensor::DT_FLOAT, packed_shape, Tensor::DEVICE_BUFFER, filter->dformat()));
+  int32_t st =
       ogle_hip_pack_filter(static_cast<const float*>(filter->device_ptr()), packed_filter_->device_ptr(),
                            layout, OGLE_F32, fs[0], fs[1], fs[2], fs[3], context_->stream());
+  if (st == OGLE_OK && filter2 != nullptr) {
+    const IntList& f2 = filter2->shape();
+    float* second = static_cast<float*>(packed_filter_->device_ptr()) + filter->num_elements();
+    st = ogle_hip_pack_filter(static_cast<const float*>(filter2->device_ptr()), second, layout, OGLE_F32,
+                              f2[0], f2[1], f2[2], f2[3], context_->stream());
+  }
   if (st != OGLE_OK) LOG(FATAL) << "ogle_hip_pack_filter: " << ogle_hip_last_error();
+  if (sibling_ != nullptr && input_tensors_.size() > 2) {
+    // both bias vectors back to back, this node's first
+    const Tensor* b1 = input_tensors_[2];
+    const Tensor* b2 = sibling_->input_tensors_[2];
+    fused_bias_.reset(new Tensor(Tensor::DT_FLOAT, {static_cast<int>(b1->num_elements() + b2->num_elements())},
+                                 Tensor::DEVICE_BUFFER, dlxnet::TensorProto::ANY4));
+    const int32_t c1 = ogle_hip_convert(b1->device_ptr(), OGLE_F32, fused_bias_->device_ptr(), OGLE_F32,
+                                        static_cast<int64_t>(b1->num_elements()), context_->stream());
+    const int32_t c2 = ogle_hip_convert(b2->device_ptr(), OGLE_F32,
+                                        static_cast<float*>(fused_bias_->device_ptr()) + b1->num_elements(),
+                                        OGLE_F32, static_cast<int64_t>(b2->num_elements()), context_->stream());
+    if (c1 != OGLE_OK || c2 != OGLE_OK) LOG(FATAL) << "ogle_hip_convert: " << ogle_hip_last_error();
+  }
   packed_from_ = filter->device_ptr();
+}
+
+// Two Conv nodes can share one launch when they read the same tensor with the same
+// geometry and fused activation, neither is depthwise or grouped, both or neither have a
+// bias, and their filters are separate constants.  The fused contraction has
+// out_c = O1 + O2 output channels and writes each node's channels to its own tensor
+// (OgleConvArgs.output2_dev).  It is only taken when the library would run it on the MFMA
+// path with all channels in one tile column (out_c <= 160): that is where fetching the
+// input once pays.
+bool Conv2DKernel::TryAbsorb(Kernel* other_kernel) {
+  Conv2DKernel* other = dynamic_cast<Conv2DKernel*>(other_kernel);
+  if (other == nullptr || other == this || sibling_ != nullptr || absorbed() || other->absorbed() ||
+      other->sibling_ != nullptr)
+    return false;
+  if (variant_ != kDense && variant_ != kPointwise) return false;
+  if (other->variant_ != variant_ || other->act_variant_ != act_variant_) return false;
+  if (input_tensors_.empty() || other->input_tensors_.empty() || output_tensors_.empty() ||
+      other->output_tensors_.empty())
+    return false;
+  if (input_tensor_indexes_[0] != other->input_tensor_indexes_[0]) return false;
+  if (input_tensors_.size() != other->input_tensors_.size()) return false;
+  if (kernel_size_ != other->kernel_size_ || stride_ != other->stride_ || padding_ != other->padding_ ||
+      dilation_ != other->dilation_ || group_size_ != 1 || other->group_size_ != 1 ||
+      activation_type_ != other->activation_type_ || min_ != other->min_ || max_ != other->max_)
+    return false;
+  if (input_tensors_[1] == other->input_tensors_[1]) return false;
+  const IntList& f1 = input_tensors_[1]->shape();
+  const IntList& f2 = other->input_tensors_[1]->shape();
+  if (f1[1] != f2[1] || f1[2] != f2[2] || f1[3] != f2[3]) return false;
+  const int in_c = input_tensors_[0]->shape()[3];
+  const long k_total = static_cast<long>(kernel_size_) * kernel_size_ * in_c;
+  const int out_c = f1[0] + f2[0];
+  if (in_c % 4 != 0 || k_total < 512 || out_c <= 64 || out_c > 160 || (out_c > 96 && out_c <= 128))
+    return false;
+  sibling_ = other;
+  other->absorbed_by_ = this;
+  packed_filter_.reset();
+  packed_from_ = nullptr;
+  workspace_need_ = -1;
+  return true;
 }
 
 void Conv2DKernel::FillGeometry(const Tensor* image, const Tensor* output, OgleConvArgs* a) const {
@@ -118,6 +180,10 @@ void Conv2DKernel::FillGeometry(const Tensor* image, const Tensor* output, OgleC
   const IntList& out = output->shape();
   a->n = in[0]; a->in_h = in[1]; a->in_w = in[2]; a->in_c = in[3];
   a->out_h = out[1]; a->out_w = out[2]; a->out_c = out[3];
+  if (sibling_ != nullptr) {
+    a->out_c_split = out[3];
+    a->out_c = out[3] + sibling_->output_tensors_[0]->shape()[3];
+  }
   a->kernel_size = kernel_size_; a->stride = stride_; a->padding = padding_;
   a->dilation = dilation_; a->group = group_size_;
   // "act" uniform: 1 clip, otherwise 2 for any non-empty activation (conv2d.cc:137-147).
@@ -134,21 +200,24 @@ size_t Conv2DKernel::ScratchBytes() const {
     CHECK(!input_tensors_.empty() && !output_tensors_.empty()) << "tensors are not bound yet";
     OgleConvArgs a{};
     FillGeometry(input_tensors_[0], output_tensors_[0], &a);
-    workspace_need_ = static_cast<long>(ogle_hip_conv_workspace_bytes(&a));
+    if (sibling_ != nullptr) a.output2_dev = sibling_->output_tensors_[0]->device_ptr();
+    workspace_need_ = absorbed() ? 0 : static_cast<long>(ogle_hip_conv_workspace_bytes(&a));
   }
   return static_cast<size_t>(workspace_need_);
 }
 
 double Conv2DKernel::WorkEstimate() const {
-  if (input_tensors_.empty() || output_tensors_.empty()) return 0.0;
+  if (input_tensors_.empty() || output_tensors_.empty() || absorbed()) return 0.0;
   const IntList& in = input_tensors_[0]->shape();
   const IntList& out = output_tensors_[0]->shape();
   const double m = static_cast<double>(out[0]) * out[1] * out[2];
-  const double n = 32.0 * ((out[3] + 31) / 32);  // the MFMA tiles are at least 32 channels wide
+  const int out_c = out[3] + (sibling_ != nullptr ? sibling_->output_tensors_[0]->shape()[3] : 0);
+  const double n = 32.0 * ((out_c + 31) / 32);  // the MFMA tiles are at least 32 channels wide
   return m * n * kernel_size_ * kernel_size_ * (in[3] / group_size_);
 }
 
 void Conv2DKernel::Compute(TensorList& inputs, TensorList& outputs) {
+  if (absorbed()) return;  // the sibling's launch fills this node's output
   program_->Activate();
   const Tensor* image = inputs[0];
   const Tensor* filter = inputs[1];
@@ -160,6 +229,10 @@ void Conv2DKernel::Compute(TensorList& inputs, TensorList& outputs) {
   a.filter_dev = packed_filter_->device_ptr();
   a.bias_dev = inputs.size() > 2 ? static_cast<const float*>(inputs[2]->device_ptr()) : nullptr;
   a.output_dev = outputs[0]->device_ptr();
+  if (sibling_ != nullptr) {
+    a.output2_dev = sibling_->output_tensors_[0]->device_ptr();
+    if (fused_bias_) a.bias_dev = static_cast<const float*>(fused_bias_->device_ptr());
+  }
   if (variant_ != kDepthwise) context_->BeforeConv(a);
   if (workspace_need_ < 0) workspace_need_ = static_cast<long>(ogle_hip_conv_workspace_bytes(&a));
   if (workspace_need_ > 0) {

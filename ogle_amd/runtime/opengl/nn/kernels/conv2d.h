@@ -19,7 +19,8 @@ class Conv2DKernel : public Kernel {
   void InferOutputShape(TensorShapeList& inputs, TensorShapeList& outputs) override;
   void SetupAttr(const dlxnet::Attribute& attr) override;
   void SelectKernel(const TensorList& inputs) override;
-  bool Deferrable() const override { return variant_ != kDepthwise; }
+  bool Deferrable() const override { return variant_ != kDepthwise && !absorbed(); }
+  bool TryAbsorb(Kernel* other) override;
   double WorkEstimate() const override;
   size_t ScratchBytes() const override;
 
@@ -43,6 +44,10 @@ class Conv2DKernel : public Kernel {
   // constant the first time the node computes.
   std::unique_ptr<Tensor> packed_filter_;
   const void* packed_from_ = nullptr;
+  // Sibling fusion: this node also computes sibling_'s output.  The packed filter then
+  // holds both filters (this node's output channels first), fused_bias_ both biases.
+  Conv2DKernel* sibling_ = nullptr;
+  std::unique_ptr<Tensor> fused_bias_;
   mutable long workspace_need_ = -1;  // bytes of scratch the launch plan wants; -1 until asked
 };
 

@@ -25,6 +25,7 @@ SYMBOLS = [
     "ogle_rt_reserialize", "ogle_rt_model_debug_string", "ogle_rt_tensor_dformat",
     "ogle_rt_set_reorder", "ogle_rt_issue_order_name", "ogle_rt_set_device_nms",
     "ogle_rt_detect_results", "ogle_rt_graph_captured", "ogle_rt_hazard_conflicts",
+    "ogle_rt_set_fuse_siblings",
 ]
 
 
@@ -87,6 +88,7 @@ def lib():
         l.ogle_rt_get_output.restype = i64
         l.ogle_rt_num_kernels.argtypes = [vp]
         l.ogle_rt_set_reorder.argtypes = [vp, i32]
+        l.ogle_rt_set_fuse_siblings.argtypes = [vp, i32]
         l.ogle_rt_set_device_nms.argtypes = [vp, i32]
         l.ogle_rt_issue_order_name.argtypes = [vp, i32]
         l.ogle_rt_issue_order_name.restype = cp
@@ -295,6 +297,10 @@ class Session:
     def set_reorder(self, on):
         """Before the first run: False keeps the reference's strict file order."""
         _check(lib().ogle_rt_set_reorder(self._h, 1 if on else 0))
+
+    def set_fuse_siblings(self, on):
+        """Before the first run: False keeps one launch per Conv node."""
+        _check(lib().ogle_rt_set_fuse_siblings(self._h, 1 if on else 0))
 
     def issue_order(self):
         """Node names in the order a pass issues them (after the first run)."""
