@@ -28,12 +28,6 @@ MFMA_F32_PEAK_TFLOPS = 157.3   # dense fp32 MFMA
 METRIC = "MobileNet-SSD 300² images/s (b16) + p50 ms (b1); per-kernel % of roofline"
 
 
-def family_of(layer):
-    return {"pw": "pointwise 1x1 (MFMA implicit GEMM)", "dw": "depthwise 3x3",
-            "dense": "dense 3x3 (MFMA implicit GEMM)"}[layer["kind"]] \
-        if not (layer["kind"] == "dense" and layer["cin"] == 3) else "dense 3x3 stem (direct)"
-
-
 def build_session(batch, seed=20240005, input_seed=None):
     from ogle_amd import models, session
     g, info = models.mobilenet_v1_ssd(batch, seed=seed)
@@ -46,35 +40,43 @@ def build_session(batch, seed=20240005, input_seed=None):
     return s, info
 
 
-def per_family_roofline(sess, info, batch, passes):
-    """Per-node HIP-event durations (averaged over `passes` profiled passes), grouped by kernel
-    family, against the algorithmic FLOPs / bytes of each layer."""
-    acc = {}
-    for _ in range(passes):
-        for label, typ, ms in sess.profile():
-            acc[label] = acc.get(label, 0.0) + ms / passes
-    fams = {}
-    for l in info["layers"]:
-        ms = acc[l["name"] + "#Conv#"]
-        f = fams.setdefault(family_of(l), dict(ms=0.0, flops=0.0, bytes=0.0, launches=0))
-        f["ms"] += ms
-        f["flops"] += l["flops_per_image"] * batch
-        f["bytes"] += l["act_bytes_per_image"] * batch + l["weight_bytes"]
-        f["launches"] += 1
+FAMILIES = [
+    # name, bound, which layers, label parts that select the family's nodes
+    ("pointwise 1x1 backbone (MFMA implicit GEMM)", "mfma",
+     lambda l: l["kind"] == "pw" and l["name"].startswith("block"),
+     ["block%d.pw#" % i for i in range(1, 14)]),
+    ("depthwise 3x3", "hbm", lambda l: l["kind"] == "dw", ["block%d.dw#" % i for i in range(1, 14)]),
+    ("SSD heads + extras chain (dense 3x3 and 1x1, MFMA implicit GEMM)", "mfma",
+     lambda l: l["name"].startswith("head") or l["name"].startswith("extra"), ["head", "extra"]),
+    ("dense 3x3 stem (direct MFMA)", "hbm", lambda l: l["name"] == "conv0", ["conv0#"]),
+]
+
+
+def per_family_roofline(sess, info, batch, full_ms, steps, warmup):
+    """What each kernel family costs INSIDE the replayed pass: the pass is recorded again
+    without the family's nodes and timed the same way (HIP events on the session's stream around
+    `steps` graph replays); full minus without is the family's time, launch gaps and tails
+    included, so the rows add up to the pass.  FLOPs / bytes are the layers' algorithmic work."""
+    plan = sess.launch_plan(with_detect=True)
     out = []
-    for name, f in fams.items():
-        sec = f["ms"] * 1e-3
-        tflops = f["flops"] / sec / 1e12
-        gbs = f["bytes"] / sec / 1e9
-        bound = "hbm" if "depthwise" in name or "stem" in name else "mfma"
-        out.append(dict(kernel=name, launches=f["launches"], ms_per_step=round(f["ms"], 4),
-                        avg_launch_us=round(f["ms"] * 1e3 / f["launches"], 2), bound=bound,
+    for name, bound, pick, parts in FAMILIES:
+        layers = [l for l in info["layers"] if pick(l)]
+        names = {l["name"] for l in layers}
+        launches = sum(k for label, k in plan if {p.split("#")[0] for p in label.split("+")} & names)
+        without = sess.time_without(parts, warmup, steps, with_detect=True) / steps
+        ms = max(full_ms - without, 1e-6)
+        flops = float(sum(l["flops_per_image"] for l in layers)) * batch
+        nbytes = float(sum(l["act_bytes_per_image"] * batch + l["weight_bytes"] for l in layers))
+        tflops, gbs = flops / ms / 1e9, nbytes / ms / 1e6
+        out.append(dict(kernel=name, layers=len(layers), launches=launches, ms_per_step=round(ms, 4),
+                        avg_launch_us=round(ms * 1e3 / max(launches, 1), 2), bound=bound,
                         tflops=round(tflops, 2), gbs=round(gbs, 1),
                         frac=round(gbs / HBM_PEAK_GBS if bound == "hbm" else tflops / MFMA_F32_PEAK_TFLOPS, 4),
-                        flops_per_step=f["flops"], bytes_per_step=f["bytes"]))
-    other = sum(ms for label, ms in acc.items() if not label.endswith("#Conv#"))
+                        flops_per_step=flops, bytes_per_step=nbytes))
+    # what is left: transposes / reshapes (views), the two concats, decode + score filter, top-k + NMS
+    rest = full_ms - sum(f["ms_per_step"] for f in out)
     out.sort(key=lambda d: -d["ms_per_step"])
-    return out, other, sum(acc.values())
+    return out, rest, plan
 
 
 def calibration_copy(megabytes=256, launches=3):
@@ -311,6 +313,35 @@ def cpu_baseline(seed=20240005, images=2, repeats=1):
                        % (repeats, images, dt))
 
 
+def profile_layers_run(args):
+    """Replays of the pass and nothing after them, plus the plan file that lets
+    ogle_amd.profile_layers attribute a kernel trace of this run to layers."""
+    import torch
+    sess, info = build_session(args.batch)
+    plan = sess.launch_plan(with_detect=True)
+    sess.time_compute(args.warmup, args.steps, graph=True, with_detect=True)
+    sess.sync()
+    torch.cuda.synchronize()
+    me = "python3 bench.py --profile-layers %s --steps %d --warmup %d --batch %d" % (
+        args.profile_layers, args.steps, args.warmup, args.batch)
+    doc = dict(workload="MobileNet-v1-SSD 300x300 fp32, batch %d, one session, hipGraph replay, "
+                        "network + decode/score filter + top-k/NMS" % args.batch,
+               batch=args.batch, replays=args.steps, dispatches_per_pass=sum(k for _, k in plan),
+               plan=plan,
+               layers={l["name"]: dict(kind=l["kind"], flops_per_image=l["flops_per_image"],
+                                       act_bytes_per_image=l["act_bytes_per_image"],
+                                       weight_bytes=l["weight_bytes"]) for l in info["layers"]},
+               commands=["cd /tmp && export TMPDIR=/tmp && cd $GRAFT_REPO_ROOT",
+                         "rocprofv3 --kernel-trace --output-format csv -d gpurun_out/layers -o b%d -- %s"
+                         % (args.batch, me),
+                         "python3 -m ogle_amd.profile_layers gpurun_out/layers/b%d_kernel_trace.csv %s"
+                         % (args.batch, args.profile_layers)])
+    with open(args.profile_layers, "w") as f:
+        json.dump(doc, f)
+    print(json.dumps(dict(profile_layers=args.profile_layers, dispatches_per_pass=doc["dispatches_per_pass"],
+                          replays=args.steps)))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -326,6 +357,10 @@ def main():
                     help="leave out the per-kernel leg at the single-kernel configurations")
     ap.add_argument("--skip-b1", action="store_true",
                     help="leave out the batch-1 latency leg (keeps a profiler trace to the batch-16 pass)")
+    ap.add_argument("--profile-layers", metavar="PLAN.json",
+                    help="only replay the pass --steps times as a hipGraph (after --warmup) and write the "
+                         "pass's dispatch sequence to PLAN.json: run under `rocprofv3 --kernel-trace` and "
+                         "feed trace + plan to `python -m ogle_amd.profile_layers`")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus %d is not supported (every image is "
@@ -337,6 +372,9 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(2)
 
+    if args.profile_layers:
+        profile_layers_run(args)
+        return
     use_graph = not args.eager
     streams = 1 if args.eager else max(1, min(args.streams, 16))
     # Every session of the pipelined leg is created here, one after the other, before any
@@ -357,6 +395,20 @@ def main():
     single = {"images_per_s": round(args.batch * args.steps / (single_wall_ms * 1e-3), 1),
               "ms_per_step": round(single_wall_ms / args.steps, 4),
               "event_ms_per_step": round(total_ms / args.steps, 4)}
+    # the same, with the final detections (at most 100 per image) read back to the host inside
+    # every step, as the reference's own timing loop does (nn/main.cc:76-111 includes GetOutputs):
+    # the step ends when the host holds the boxes, so steps do not overlap
+    sess.sync()
+    t0 = time.perf_counter()
+    kept = 0
+    for _ in range(args.steps):
+        sess.time_compute(0, 1, graph=use_graph, with_detect=True)
+        kept += sum(len(d) for d in sess.detect_results(args.batch))
+    rb_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    single["with_detection_readback"] = {
+        "images_per_s": round(args.batch / (rb_ms * 1e-3), 1), "ms_per_step": round(rb_ms, 4),
+        "detections_per_step": kept / args.steps,
+        "note": "one pass, then wait and copy the final lists to the host, then the next pass"}
     if streams == 1:
         wall_ms = single_wall_ms
     else:
@@ -411,7 +463,8 @@ def main():
         for pb in pinned:
             pb.close()
 
-    fams, other_ms, node_sum_ms = per_family_roofline(sess, info, args.batch, passes=10)
+    fams, other_ms, plan = per_family_roofline(sess, info, args.batch, total_ms / args.steps,
+                                               min(args.steps, 100), min(args.warmup, 10))
     dom = fams[0]
     roofline = dict(bound=dom["bound"], kernel=dom["kernel"],
                     achieved=dom["gbs"] if dom["bound"] == "hbm" else dom["tflops"],
@@ -419,6 +472,8 @@ def main():
                     unit="GB/s" if dom["bound"] == "hbm" else "TFLOP/s", frac=dom["frac"],
                     traffic=read_traffic_summary(dom["kernel"]), launches_per_step=dom["launches"],
                     avg_launch_us=dom["avg_launch_us"],
+                    measured="HIP events on the session's stream around graph replays of the pass with and "
+                             "without the family's nodes (difference / launches)",
                     algorithmic_per_step=dom["flops_per_step"] if dom["bound"] == "mfma" else dom["bytes_per_step"])
 
     # batch-1 latency: each pass waits for the previous one
@@ -430,7 +485,8 @@ def main():
         lat_eager, _ = s1.time_compute(5, 100, graph=False, with_detect=True, sync_each=True)
 
     result = {
-        "metric": METRIC, "value": round(images_per_s, 1), "unit": "images/s", "n_gpus": 1,
+        "metric": METRIC, "value": round(images_per_s, 1), "unit": "images/s",
+        "single_stream": single, "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
         "data": "synthetic",
@@ -443,13 +499,13 @@ def main():
                                   "stream; the K steps are dealt round-robin" % (streams, args.batch))
                    if streams > 1 else "none: one stream, one pass after the other",
                    "inputs": "resident in HBM", "flops_per_image": 2803531136},
-        "single_stream": single,
         "p50_ms_b1": round(float(np.percentile(lat, 50)), 4),
         "p50_ms_b1_eager": round(float(np.percentile(lat_eager, 50)), 4),
         "network_tflops": round(2803531136 * args.batch / (ms_per_step * 1e-3) / 1e12, 2),
         "roofline": roofline,
         "kernels": fams,
         "non_conv_ms_per_step": round(other_ms, 4),
+        "dispatches_per_step": sum(k for _, k in plan),
         "with_host_upload": upload,
     }
     if not args.skip_kernel_table:

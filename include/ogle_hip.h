@@ -77,6 +77,12 @@ typedef enum OgleFilterLayout {
 /* Version of this ABI (major*100 + minor). */
 int32_t ogle_hip_abi_version(void);
 
+/* Number of device operations (kernels, and the one device-to-device copy an identity
+ * transpose makes) the calling thread has enqueued through this library so far.  The
+ * difference across a call says how many dispatches that call became, which is how a
+ * profiler trace of a replayed pass is lined up with the graph's nodes. */
+int64_t ogle_hip_launch_count(void);
+
 /* Message of the calling thread's most recent failure ("" if none). */
 const char* ogle_hip_last_error(void);
 const char* ogle_hip_status_string(int32_t status);
@@ -181,6 +187,21 @@ int32_t ogle_hip_conv2d(const OgleConvArgs* args, ogle_stream_t stream);
  * Conv nodes into this call.
  */
 int32_t ogle_hip_conv2d_batch(const OgleConvArgs* args, int32_t count, ogle_stream_t stream);
+
+/*
+ * ogle_hip_conv2d_batch in two steps, for convolutions whose results are not needed at
+ * once (the SSD heads, read only by the final concat).  _begin launches the contractions
+ * like ogle_hip_conv2d_batch but leaves the reductions of split-K plans unlaunched:
+ * reduce_pending[i] is set to 1 for every convolution whose partial sums still sit in its
+ * workspace (its output is not valid yet), 0 for the finished ones.  _finish, given those
+ * same arguments (any subset, any order, from one or several _begin calls on the stream),
+ * launches all their reductions as one grid per 16 convolutions.  The workspaces must stay
+ * untouched in between.  One reduction grid at the end of a pass replaces one small
+ * dependent launch per convolution.
+ */
+int32_t ogle_hip_conv2d_batch_begin(const OgleConvArgs* args, int32_t count,
+                                    int32_t* reduce_pending, ogle_stream_t stream);
+int32_t ogle_hip_conv2d_batch_finish(const OgleConvArgs* args, int32_t count, ogle_stream_t stream);
 
 /*
  * ogle_hip_conv2d for callers that cannot allocate device memory: code under HIP

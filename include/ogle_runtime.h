@@ -116,6 +116,31 @@ int32_t ogle_rt_profile(OgleSession* s);
 int32_t ogle_rt_profile_entry(OgleSession* s, int32_t i, const char** label, const char** type,
                               float* ms);
 
+/*
+ * Time of `iters` replays (after `warmup`) of the pass WITHOUT the nodes whose label
+ * "<node>#<type>#" contains one of the n_parts strings in label_parts, recorded as its own
+ * hipGraph and timed with HIP events on the session's stream like ogle_rt_time_compute.
+ * The difference to the full pass is what those nodes cost inside the pass, launch gaps
+ * and all: a per-family time that adds up to the pass.  Outputs are stale afterwards until
+ * the next full pass.
+ */
+int32_t ogle_rt_time_without(OgleSession* s, const char* const* label_parts, int32_t n_parts,
+                             int32_t warmup, int32_t iters, int32_t with_detect, float* total_ms);
+
+/*
+ * Dispatch sequence of a pass.  ogle_rt_launch_plan makes one eager pass (with_detect:
+ * followed by the detector's device work) and records, in issue order, every call into the
+ * kernel library with the node(s) it was made for and the number of device operations it
+ * became; it returns the number of entries.  ogle_rt_launch_plan_entry reads entry i: its
+ * label ("<node>#<type>#", the reference's TraceMe label, fbo_session.cc:140-153; the
+ * nodes of convolutions that went out as one batch are joined with '+') and its dispatch
+ * count.  A replayed hipGraph of the pass issues exactly this sequence, so a profiler's
+ * kernel trace of the replays can be attributed to layers position by position.
+ */
+int32_t ogle_rt_launch_plan(OgleSession* s, int32_t with_detect);
+int32_t ogle_rt_launch_plan_entry(OgleSession* s, int32_t i, const char** label,
+                                  int32_t* dispatches);
+
 /* Shape of a tensor by name (FindTensorByName): writes up to 8 dims, returns rank. */
 int32_t ogle_rt_tensor_shape(OgleSession* s, const char* name, int32_t* dims);
 /* Layout tag of a tensor as a TensorProto.DataFormat value (dlxnet.proto:7-30), or negative. */
@@ -157,8 +182,8 @@ int32_t ogle_rt_set_reorder(OgleSession* s, int32_t on);
  * Sibling fusion.  Two Conv nodes that read the same tensor with the same attributes (the
  * box and the class head of an SSD feature map) run as one launch that fetches the input
  * once and writes each node's channels to its own tensor; the reference draws them one
- * after the other.  ogle_rt_set_fuse_siblings(s, 0) before the first run keeps one launch
- * per node.  Results agree to summation order.
+ * after the other.  Off by default (one launch per node); ogle_rt_set_fuse_siblings(s, 1)
+ * before the first run switches it on.  Results agree to summation order.
  */
 int32_t ogle_rt_set_fuse_siblings(OgleSession* s, int32_t on);
 const char* ogle_rt_issue_order_name(OgleSession* s, int32_t i);

@@ -16,12 +16,17 @@ void set_error(const char* fmt, ...) {
   va_end(ap);
 }
 
+static thread_local int64_t g_launches = 0;
+
+void note_launch() { ++g_launches; }
+
 int32_t check_launch(const char* kernel) {
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     set_error("%s: launch failed: %s", kernel, hipGetErrorString(e));
     return OGLE_ERR_LAUNCH;
   }
+  ++g_launches;
   return OGLE_OK;
 }
 
@@ -151,7 +156,9 @@ using namespace ogle;
 
 extern "C" {
 
-int32_t ogle_hip_abi_version(void) { return 100; }
+int32_t ogle_hip_abi_version(void) { return 101; }
+
+int64_t ogle_hip_launch_count(void) { return g_launches; }
 
 const char* ogle_hip_last_error(void) { return g_error; }
 
@@ -267,7 +274,35 @@ int32_t ogle_hip_conv2d_noalloc(const OgleConvArgs* a, ogle_stream_t stream) {
   return launch_conv_direct(*a, as_stream(stream));
 }
 
+namespace {
+int32_t conv2d_batch_impl(const OgleConvArgs* args, int32_t count, int32_t* reduce_pending,
+                          ogle_stream_t stream);
+}
+
 int32_t ogle_hip_conv2d_batch(const OgleConvArgs* args, int32_t count, ogle_stream_t stream) {
+  return conv2d_batch_impl(args, count, nullptr, stream);
+}
+
+int32_t ogle_hip_conv2d_batch_begin(const OgleConvArgs* args, int32_t count,
+                                    int32_t* reduce_pending, ogle_stream_t stream) {
+  if (count > 0 && reduce_pending == nullptr)
+    return fail(OGLE_ERR_INVALID_ARG, "conv2d_batch_begin: reduce_pending is required");
+  return conv2d_batch_impl(args, count, reduce_pending, stream);
+}
+
+int32_t ogle_hip_conv2d_batch_finish(const OgleConvArgs* args, int32_t count, ogle_stream_t stream) {
+  if (count < 0 || (count > 0 && args == nullptr))
+    return fail(OGLE_ERR_INVALID_ARG, "conv2d_batch_finish: null args or negative count");
+  for (int i = 0; i < count; ++i) {
+    const int32_t st = validate_conv(&args[i], "conv2d_batch_finish");
+    if (st != OGLE_OK) return st;
+  }
+  return launch_conv_reduce(args, count, as_stream(stream));
+}
+
+namespace {
+int32_t conv2d_batch_impl(const OgleConvArgs* args, int32_t count, int32_t* reduce_pending,
+                          ogle_stream_t stream) {
   if (count < 0 || (count > 0 && args == nullptr))
     return fail(OGLE_ERR_INVALID_ARG, "conv2d_batch: null args or negative count");
   for (int i = 0; i < count; ++i) {
@@ -295,8 +330,9 @@ int32_t ogle_hip_conv2d_batch(const OgleConvArgs* args, int32_t count, ogle_stre
                     "conv2d_batch: a workspace overlaps another convolution's tensor");
     }
   }
-  return launch_conv_batch(args, count, as_stream(stream), direct_no_split);
+  return launch_conv_batch(args, count, as_stream(stream), direct_no_split, reduce_pending);
 }
+}  // namespace
 
 int32_t ogle_hip_dwconv2d(const OgleConvArgs* a, ogle_stream_t stream) {
   int32_t st = validate_conv(a, "dwconv2d");

@@ -21,8 +21,11 @@ inline int32_t fail(int32_t status, const char* what) {
   return status;
 }
 
-// Reports the launch status of the kernel just enqueued.
+// Reports the launch status of the kernel just enqueued (and counts it for
+// ogle_hip_launch_count).
 int32_t check_launch(const char* kernel);
+// Counts a device operation that is not one of the library's kernels (a copy).
+void note_launch();
 
 inline hipStream_t as_stream(ogle_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
 
@@ -82,8 +85,12 @@ __device__ __forceinline__ int xcd_swizzle(int pid, int grid) {
 int32_t launch_conv_igemm(const OgleConvArgs& a, hipStream_t s);   // returns OGLE_ERR_UNSUPPORTED if shape not eligible
 size_t conv_igemm_workspace_bytes(const OgleConvArgs& a);
 int32_t launch_conv_igemm_static_scratch(const OgleConvArgs& a, hipStream_t s);
+// reduce_pending != nullptr: split-K reductions are not launched; reduce_pending[i] says
+// whether convolution i still needs launch_conv_reduce.
 int32_t launch_conv_batch(const OgleConvArgs* args, int count, hipStream_t s,
-                          int32_t (*fallback)(const OgleConvArgs&, hipStream_t));
+                          int32_t (*fallback)(const OgleConvArgs&, hipStream_t),
+                          int32_t* reduce_pending = nullptr);
+int32_t launch_conv_reduce(const OgleConvArgs* args, int count, hipStream_t s);
 int32_t launch_conv_direct(const OgleConvArgs& a, hipStream_t s);
 int32_t launch_conv_dw(const OgleConvArgs& a, hipStream_t s);
 int32_t launch_pool(const OglePoolArgs& a, hipStream_t s);

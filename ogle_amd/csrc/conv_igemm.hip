@@ -867,7 +867,6 @@ constexpr long kComputeUnits = 256;
 constexpr int kRowBytesF32 = 64;   // bytes of K per tile row per slab, fp32
 
 bool is_pointwise(const OgleConvArgs& a);
-bool is_wave(int cfg);
 
 // Picks the output tile and the K split.  Problems with few output
 // tiles but a long contraction (the SSD heads, the small feature maps) are split
@@ -973,9 +972,11 @@ IgemmPlan plan_igemm(const OgleConvArgs& a, long m, bool allow_split) {
       p.splits = 1;
     }
   }
-  if (const char* e = getenv("OGLE_DEBUG_SPLITS")) { if (allow_split && !is_wave(p.cfg)) p.splits = atoi(e); }  // TEMP
   p.slabs_per_split = (p.ktiles + p.splits - 1) / p.splits;
-  if (p.splits > 1) p.slabs_per_split += p.slabs_per_split & 1;  // the K loop runs slab pairs
+  if (p.splits > 1) {
+    p.slabs_per_split += p.slabs_per_split & 1;  // the K loop runs slab pairs
+    p.splits = (p.ktiles + p.slabs_per_split - 1) / p.slabs_per_split;  // no empty ranges
+  }
   // (a split past the end of K would only add zeros; rounding splits down keeps the
   // divisor-or-multiple-of-8 shape, so empty splits are simply avoided by the cap above)
   // partial sums are kept in rows of the channel count rounded up to four
@@ -1180,7 +1181,8 @@ int32_t launch_conv_igemm(const OgleConvArgs& a, hipStream_t s) {
 // kernel that branches per workgroup; 128x128-tile problems fill the chip on their
 // own and are launched singly.  The others are launched one by one through `fallback`.
 int32_t launch_conv_batch(const OgleConvArgs* args, int count, hipStream_t s,
-                          int32_t (*fallback)(const OgleConvArgs&, hipStream_t)) {
+                          int32_t (*fallback)(const OgleConvArgs&, hipStream_t),
+                          int32_t* reduce_pending) {
   struct Item {
     int dtype, cfg;
     bool pw;
@@ -1188,6 +1190,7 @@ int32_t launch_conv_batch(const OgleConvArgs* args, int count, hipStream_t s,
   };
   std::vector<Item> items;
   for (int i = 0; i < count; ++i) {
+    if (reduce_pending != nullptr) reduce_pending[i] = 0;
     long m = 0;
     if (!igemm_eligible(args[i], &m)) {
       const int32_t st = fallback(args[i], s);
@@ -1196,6 +1199,7 @@ int32_t launch_conv_batch(const OgleConvArgs* args, int count, hipStream_t s,
     }
     const IgemmPlan p = final_plan(args[i], m);
     items.push_back(Item{args[i].dtype, p.cfg, is_pointwise(args[i]), prepare(args[i], m, p)});
+    if (reduce_pending != nullptr && p.splits > 1) reduce_pending[i] = 1;
   }
   auto mixable = [](const Item& it) {
     return it.cfg == CFG_64x64 || it.cfg == CFG_128x32 || is_wave(it.cfg);
@@ -1237,7 +1241,7 @@ int32_t launch_conv_batch(const OgleConvArgs* args, int count, hipStream_t s,
     }
     int32_t st = check_launch("conv_igemm_group");
     if (st != OGLE_OK) return st;
-    if (red.count == 0) continue;
+    if (red.count == 0 || reduce_pending != nullptr) continue;  // the caller finishes them later
     const dim3 rgrid((unsigned)red.first[red.count]), block(256);
     if (red.count == 1) {
       Prepared one{};
@@ -1252,6 +1256,38 @@ int32_t launch_conv_batch(const OgleConvArgs* args, int count, hipStream_t s,
       hipLaunchKernelGGL((splitk_reduce_group_kernel<float>), rgrid, block, 0, s, red);
     }
     st = check_launch("splitk_reduce_group");
+    if (st != OGLE_OK) return st;
+  }
+  return OGLE_OK;
+}
+
+// Finishes convolutions whose contraction was launched with the reduction left pending:
+// the plan is a function of the arguments alone, so it is recomputed here and names the
+// same partial-sum layout.  All reductions go out in one grid (16 problems per grid).
+int32_t launch_conv_reduce(const OgleConvArgs* args, int count, hipStream_t s) {
+  int at = 0;
+  while (at < count) {
+    ReduceGroup red{};
+    int dtype = -1;
+    for (; at < count && red.count < kMaxGroup; ++at) {
+      long m = 0;
+      if (!igemm_eligible(args[at], &m)) continue;
+      const IgemmPlan p = final_plan(args[at], m);
+      if (p.splits <= 1) continue;
+      if (dtype >= 0 && args[at].dtype != dtype) break;  // one storage type per grid
+      dtype = args[at].dtype;
+      const Prepared pr = prepare(args[at], m, p);
+      red.first[red.count + 1] = red.first[red.count] + (int)pr.reduce_grid;
+      red.p[red.count++] = pr.red;
+    }
+    if (red.count == 0) continue;
+    const dim3 rgrid((unsigned)red.first[red.count]), block(256);
+    if (dtype == OGLE_F16) {
+      hipLaunchKernelGGL((splitk_reduce_group_kernel<__half>), rgrid, block, 0, s, red);
+    } else {
+      hipLaunchKernelGGL((splitk_reduce_group_kernel<float>), rgrid, block, 0, s, red);
+    }
+    const int32_t st = check_launch("splitk_reduce_group");
     if (st != OGLE_OK) return st;
   }
   return OGLE_OK;

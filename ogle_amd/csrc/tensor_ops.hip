@@ -420,6 +420,7 @@ int32_t launch_transpose(const OgleTransposeArgs& a, hipStream_t s) {
       set_error("transpose: copy failed: %s", hipGetErrorString(e));
       return OGLE_ERR_LAUNCH;
     }
+    note_launch();
     return OGLE_OK;
   }
   if (esz == 4) {

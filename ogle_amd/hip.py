@@ -28,7 +28,8 @@ SYMBOLS = [
     "ogle_hip_expf", "ogle_hip_transpose", "ogle_hip_conv_workspace_bytes",
     "ogle_hip_conv2d_batch", "ogle_hip_ssd_topk_nms", "ogle_hip_unary", "ogle_hip_add",
     "ogle_hip_batchnorm", "ogle_hip_gemm", "ogle_hip_gemm_workspace_bytes",
-    "ogle_hip_conv2d_noalloc",
+    "ogle_hip_conv2d_noalloc", "ogle_hip_launch_count",
+    "ogle_hip_conv2d_batch_begin", "ogle_hip_conv2d_batch_finish",
 ]
 CONV_NOALLOC_SCRATCH_BYTES = 16 << 20
 UNARY_RELU, UNARY_CLIP = 0, 1
@@ -163,6 +164,7 @@ def lib():
         l.ogle_hip_registry_lookup.argtypes = [ctypes.c_char_p, ctypes.c_char_p,
                                                ctypes.POINTER(ctypes.c_int32)]
         l.ogle_hip_sync.argtypes = [ctypes.c_void_p]
+        l.ogle_hip_launch_count.restype = ctypes.c_int64
         l.ogle_hip_packed_filter_elems.restype = ctypes.c_int64
         l.ogle_hip_packed_filter_elems.argtypes = [ctypes.c_int32] * 5
         l.ogle_hip_pack_filter.argtypes = [ctypes.c_void_p, ctypes.c_void_p] + \
@@ -180,6 +182,9 @@ def lib():
                           ("ogle_hip_transpose", TransposeArgs)):
             getattr(l, name).argtypes = [ctypes.POINTER(typ), ctypes.c_void_p]
         l.ogle_hip_conv2d_batch.argtypes = [ctypes.POINTER(ConvArgs), ctypes.c_int32, ctypes.c_void_p]
+        l.ogle_hip_conv2d_batch_begin.argtypes = [ctypes.POINTER(ConvArgs), ctypes.c_int32,
+                                                  ctypes.POINTER(ctypes.c_int32), ctypes.c_void_p]
+        l.ogle_hip_conv2d_batch_finish.argtypes = [ctypes.POINTER(ConvArgs), ctypes.c_int32, ctypes.c_void_p]
         l.ogle_hip_conv_workspace_bytes.argtypes = [ctypes.POINTER(ConvArgs)]
         l.ogle_hip_conv_workspace_bytes.restype = ctypes.c_size_t
         l.ogle_hip_gemm_workspace_bytes.argtypes = [ctypes.POINTER(GemmArgs)]

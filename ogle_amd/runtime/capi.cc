@@ -11,6 +11,7 @@
 #include <vector>
 
 #include "opengl/core/fbo_session.h"
+#include "opengl/core/kernel.h"
 #include "opengl/core/kernel_registry.h"
 #include "opengl/core/tensor.h"
 #include "opengl/examples/ssd/detector.h"
@@ -24,6 +25,7 @@ struct OgleSession {
   std::vector<opengl::NodeTiming> timings;
   std::unique_ptr<opengl::Detector> detector;
   bool device_nms = true;
+  std::vector<opengl::Context::LaunchRecord> plan;
 };
 
 namespace {
@@ -204,6 +206,92 @@ int32_t ogle_rt_time_compute(OgleSession* s, int32_t warmup, int32_t iters, int3
     for (auto& e : ev) (void)hipEventDestroy(e);
     return 0;
   });
+}
+
+int32_t ogle_rt_time_without(OgleSession* s, const char* const* label_parts, int32_t n_parts,
+                             int32_t warmup, int32_t iters, int32_t with_detect, float* total_ms) {
+  return (int32_t)Guard([&]() -> int64_t {
+    CHECK(s->session->graph_captured(with_detect ? 1 : 0) || !with_detect || s->detector)
+        << "time the full pass first";
+    std::vector<std::string> parts;
+    for (int i = 0; i < n_parts; ++i) parts.emplace_back(label_parts[i]);
+    hipStream_t st = static_cast<hipStream_t>(s->context->stream());
+    opengl::DetectorOptions opt;
+    opt.device_nms = s->device_nms;
+    if (with_detect && !s->detector) {
+      s->detector = opengl::Detector::Create(s->session.get(), opt);
+      s->detector->EnqueueDetect(opt.output_names, 300, 300);
+      s->context->Finish();
+    }
+    const int slot = 2;
+    s->session->DropGraph(slot);
+    s->session->set_skip([parts](const opengl::Kernel* k) {
+      const std::string label = k->kernel_name() + "#" + k->kernel_type() + "#";
+      for (const std::string& p : parts)
+        if (label.find(p) != std::string::npos) return true;
+      return false;
+    });
+    float total = 0.f;
+    try {
+      if (with_detect)
+        s->session->CaptureGraph(slot, [&]() { s->detector->EnqueueDetect(opt.output_names, 300, 300); });
+      else
+        s->session->CaptureGraph(slot);
+      for (int i = 0; i < warmup; ++i) s->session->LaunchGraph(slot);
+      s->context->Finish();
+      hipEvent_t e0, e1;
+      if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess)
+        LOG(FATAL) << "hipEventCreate failed";
+      (void)hipEventRecord(e0, st);
+      for (int i = 0; i < iters; ++i) s->session->LaunchGraph(slot);
+      (void)hipEventRecord(e1, st);
+      s->context->Finish();
+      (void)hipEventElapsedTime(&total, e0, e1);
+      (void)hipEventDestroy(e0);
+      (void)hipEventDestroy(e1);
+    } catch (...) {
+      s->session->set_skip({});
+      s->session->DropGraph(slot);
+      throw;
+    }
+    s->session->set_skip({});
+    s->session->DropGraph(slot);
+    if (total_ms) *total_ms = total;
+    return 0;
+  });
+}
+
+int32_t ogle_rt_launch_plan(OgleSession* s, int32_t with_detect) {
+  return (int32_t)Guard([&]() -> int64_t {
+    opengl::DetectorOptions opt;
+    opt.device_nms = s->device_nms;
+    if (with_detect && !s->detector) {
+      s->detector = opengl::Detector::Create(s->session.get(), opt);
+      s->detector->EnqueueDetect(opt.output_names, 300, 300);  // first use allocates
+      s->context->Finish();
+    }
+    s->context->set_launch_log(true);
+    try {
+      s->session->Compute();
+      if (with_detect) s->detector->EnqueueDetect(opt.output_names, 300, 300);
+      s->context->Flush();
+    } catch (...) {
+      s->context->set_launch_log(false);
+      throw;
+    }
+    s->plan = s->context->launch_log();
+    s->context->set_launch_log(false);
+    s->context->Finish();
+    return (int64_t)s->plan.size();
+  });
+}
+
+int32_t ogle_rt_launch_plan_entry(OgleSession* s, int32_t i, const char** label,
+                                  int32_t* dispatches) {
+  if (s == nullptr || i < 0 || i >= (int32_t)s->plan.size()) return -1;
+  if (label) *label = s->plan[i].label.c_str();
+  if (dispatches) *dispatches = s->plan[i].dispatches;
+  return 0;
 }
 
 void* ogle_rt_alloc_pinned(size_t bytes) {

@@ -2,6 +2,9 @@
 
 #include <hip/hip_runtime_api.h>
 
+#include <dlfcn.h>
+
+#include <cstdlib>
 #include <cstring>
 #include <vector>
 
@@ -101,38 +104,149 @@ bool Context::Conflicts(const OgleConvArgs* pending, int n_pending, const MemRan
 }
 
 void Context::BeforeConv(const OgleConvArgs& args) {
-  if (pending_.empty()) return;
+  if (pending_.empty() && unreduced_.empty()) return;
   MemRange reads[3], writes[3];
   ConvRanges(args, reads, writes);
   if (pending_.size() >= 16 ||
       Conflicts(pending_.data(), static_cast<int>(pending_.size()), reads, 3, writes, 3))
-    Flush();
+    LaunchPending();
+  FinishReductions(reads, 3, writes, 3, false);
 }
 
 void Context::BeforeLaunch(const MemRange* reads, int n_reads, const MemRange* writes,
                            int n_writes) {
-  if (pending_.empty()) return;
+  if (pending_.empty() && unreduced_.empty()) return;
   if (Conflicts(pending_.data(), static_cast<int>(pending_.size()), reads, n_reads, writes, n_writes))
-    Flush();
+    LaunchPending();
+  FinishReductions(reads, n_reads, writes, n_writes, false);
+}
+
+// A convolution whose contraction is on the stream but whose reduction is not: what it
+// still reads is its bias and its partial sums, what it still writes its output(s).
+// Its input and filter are free again (later work on the stream is ordered after the
+// contraction).
+void Context::FinishReductions(const MemRange* reads, int n_reads, const MemRange* writes,
+                               int n_writes, bool all) {
+  if (unreduced_.empty()) return;
+  std::vector<OgleConvArgs> now, keep;
+  std::vector<std::string> now_labels, keep_labels;
+  for (size_t i = 0; i < unreduced_.size(); ++i) {
+    bool hit = all;
+    if (!hit) {
+      OgleConvArgs c = unreduced_[i];
+      c.input_dev = nullptr;   // no longer read
+      c.filter_dev = nullptr;
+      hit = Conflicts(&c, 1, reads, n_reads, writes, n_writes);
+    }
+    (hit ? now : keep).push_back(unreduced_[i]);
+    (hit ? now_labels : keep_labels).push_back(unreduced_labels_[i]);
+  }
+  if (now.empty()) return;
+  unreduced_.swap(keep);
+  unreduced_labels_.swap(keep_labels);
+  if (!current_label_.empty()) LogLaunches(current_label_, node_count_before_);
+  const int64_t before = ogle_hip_launch_count();
+  const int32_t st = ogle_hip_conv2d_batch_finish(now.data(), static_cast<int32_t>(now.size()), stream());
+  if (st != OGLE_OK)
+    LOG(FATAL) << "ogle_hip_conv2d_batch_finish: " << ogle_hip_status_string(st) << ": "
+               << ogle_hip_last_error();
+  if (log_launches_) {
+    std::string joined = "reduce:";
+    for (size_t i = 0; i < now_labels.size(); ++i) joined += (i ? "+" : "") + now_labels[i];
+    LogLaunches(joined, before);
+  } else {
+    node_count_before_ = ogle_hip_launch_count();
+  }
+  if (pending_.empty() && unreduced_.empty()) workspace_used_ = 0;
 }
 
 void Context::EnqueueConv(const OgleConvArgs& args) {
   pending_.push_back(args);
+  pending_labels_.push_back(current_label_);
   if (!batching_) Flush();
 }
 
-void Context::Flush() {
+namespace {
+// roctx, looked up at run time so that the runtime has no link-time dependency on a
+// profiler library; absent library or OGLE_ROCTX unset: no ranges.
+struct Roctx {
+  int (*push)(const char*) = nullptr;
+  int (*pop)() = nullptr;
+  Roctx() {
+    const char* env = std::getenv("OGLE_ROCTX");
+    if (env == nullptr || env[0] == '\0' || env[0] == '0') return;
+    void* lib = dlopen("librocprofiler-sdk-roctx.so", RTLD_NOW | RTLD_GLOBAL);
+    if (lib == nullptr) lib = dlopen("libroctx64.so", RTLD_NOW | RTLD_GLOBAL);
+    if (lib == nullptr) return;
+    push = reinterpret_cast<int (*)(const char*)>(dlsym(lib, "roctxRangePushA"));
+    pop = reinterpret_cast<int (*)()>(dlsym(lib, "roctxRangePop"));
+    if (push == nullptr || pop == nullptr) push = nullptr;
+  }
+};
+Roctx& roctx() {
+  static Roctx r;
+  return r;
+}
+}  // namespace
+
+void Context::BeginNode(const std::string& label) {
+  current_label_ = label;
+  node_count_before_ = ogle_hip_launch_count();
+  if (roctx().push != nullptr) roctx().push(label.c_str());
+}
+
+void Context::EndNode() {
+  // what the node launched directly (deferred convolutions are logged at Flush, and a
+  // Flush inside the node has already moved the mark past its launches)
+  LogLaunches(current_label_, node_count_before_);
+  current_label_.clear();
+  if (roctx().push != nullptr) roctx().pop();
+}
+
+void Context::LogLaunches(const std::string& label, int64_t count_before) {
+  const int64_t now = ogle_hip_launch_count();
+  if (log_launches_ && now > count_before)
+    launch_log_.push_back({label, static_cast<int>(now - count_before)});
+  node_count_before_ = now;
+}
+
+void Context::LaunchPending() {
   if (pending_.empty()) {
-    workspace_used_ = 0;
+    pending_labels_.clear();
+    if (unreduced_.empty()) workspace_used_ = 0;
     return;
   }
   std::vector<OgleConvArgs> batch;
   batch.swap(pending_);
-  workspace_used_ = 0;
-  const int32_t st = ogle_hip_conv2d_batch(batch.data(), static_cast<int32_t>(batch.size()), stream());
+  std::vector<std::string> labels;
+  labels.swap(pending_labels_);
+  // launches the running node made itself before this point belong to that node
+  if (!current_label_.empty()) LogLaunches(current_label_, node_count_before_);
+  const int64_t before = ogle_hip_launch_count();
+  std::vector<int32_t> open(batch.size(), 0);
+  const int32_t st = ogle_hip_conv2d_batch_begin(batch.data(), static_cast<int32_t>(batch.size()),
+                                                 open.data(), stream());
+  if (log_launches_) {
+    std::string joined;
+    for (const std::string& l : labels) joined += (joined.empty() ? "" : "+") + l;
+    LogLaunches(joined, before);
+  } else {
+    node_count_before_ = ogle_hip_launch_count();
+  }
   if (st != OGLE_OK)
-    LOG(FATAL) << "ogle_hip_conv2d_batch: " << ogle_hip_status_string(st) << ": "
+    LOG(FATAL) << "ogle_hip_conv2d_batch_begin: " << ogle_hip_status_string(st) << ": "
                << ogle_hip_last_error();
+  for (size_t i = 0; i < batch.size(); ++i)
+    if (open[i]) {
+      unreduced_.push_back(batch[i]);
+      unreduced_labels_.push_back(labels[i]);
+    }
+  if (unreduced_.empty()) workspace_used_ = 0;
+}
+
+void Context::Flush() {
+  LaunchPending();
+  FinishReductions(nullptr, 0, nullptr, 0, true);
 }
 
 Context::~Context() {

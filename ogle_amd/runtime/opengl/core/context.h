@@ -71,12 +71,38 @@ class Context {
   // second output).
   static void ConvRanges(const OgleConvArgs& a, MemRange reads[3], MemRange writes[3]);
   void EnqueueConv(const OgleConvArgs& args);
+  // Launches everything that is still held back: the deferred convolutions and the
+  // reductions left pending (below).
   void Flush();
   void set_batching(bool on) {
     Flush();
     batching_ = on;
   }
-  size_t pending_convs() const { return pending_.size(); }
+  size_t pending_convs() const { return pending_.size() + unreduced_.size(); }
+
+  // Launch log.  While it is switched on, every call into the kernel library is recorded
+  // with the node(s) it was made for and the number of device operations it became
+  // (ogle_hip_launch_count before and after): the dispatch sequence of a pass, in order.
+  // Deferred convolutions are recorded when their batch goes out, as one entry that names
+  // every node of the batch (they share grids).  A trace of the replayed pass has exactly
+  // this sequence per replay.
+  struct LaunchRecord {
+    std::string label;  // "<node>#<type>#", several joined with '+'
+    int dispatches;
+  };
+  void set_launch_log(bool on) {
+    log_launches_ = on;
+    launch_log_.clear();
+  }
+  const std::vector<LaunchRecord>& launch_log() const { return launch_log_; }
+  // The node whose Compute is running: the label of what it launches.  With
+  // OGLE_ROCTX=1 the node is also bracketed by a roctx range of that name (the
+  // reference's per-node TraceMe scopes, fbo_session.cc:128-151), if the roctx
+  // library can be loaded.
+  void BeginNode(const std::string& label);
+  void EndNode();
+  // Brackets one call into the kernel library made outside a node (the detector).
+  void LogLaunches(const std::string& label, int64_t count_before);
 
   void Finish();  // glFinish: waits for the stream
   void Reset() {}
@@ -86,8 +112,24 @@ class Context {
   void* workspace_ = nullptr;
   size_t workspace_bytes_ = 0;
   size_t workspace_used_ = 0;
+  // Launches the deferred convolutions (ogle_hip_conv2d_batch_begin).  Convolutions whose
+  // plan splits K leave their partial sums in their workspace slice and move to
+  // unreduced_: their reduction is only launched when something touches their output,
+  // bias or workspace (FinishReductions with those ranges) or at Flush, so that all
+  // reductions still open at that point share one grid.  Workspace slices are recycled
+  // once nothing is pending or unreduced.
+  void LaunchPending();
+  void FinishReductions(const MemRange* reads, int n_reads, const MemRange* writes, int n_writes,
+                        bool all);
   std::vector<OgleConvArgs> pending_;
+  std::vector<std::string> pending_labels_;
+  std::vector<OgleConvArgs> unreduced_;
+  std::vector<std::string> unreduced_labels_;
   bool batching_ = true;
+  bool log_launches_ = false;
+  std::vector<LaunchRecord> launch_log_;
+  std::string current_label_;
+  int64_t node_count_before_ = 0;
   std::map<std::string, std::unique_ptr<Program>> programs_;
 };
 

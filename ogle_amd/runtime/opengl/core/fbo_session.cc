@@ -26,8 +26,8 @@ FBOSession::FBOSession(Context* context) : context_(context) {
   context_->Reset();
   const char* env = std::getenv("OGLE_FILE_ORDER");
   if (env != nullptr && env[0] != '\0' && env[0] != '0') reorder_ = false;
-  env = std::getenv("OGLE_NO_SIBLING_FUSION");
-  if (env != nullptr && env[0] != '\0' && env[0] != '0') fuse_siblings_ = false;
+  env = std::getenv("OGLE_SIBLING_FUSION");
+  if (env != nullptr && env[0] != '\0' && env[0] != '0') fuse_siblings_ = true;
 }
 
 FBOSession::~FBOSession() {
@@ -358,7 +358,7 @@ void FBOSession::BuildSchedule() {
 
   // cost model: microseconds at a sustained MFMA rate, with a floor per launch
   constexpr double kMacPerUs = 45e6;  // ~90 TFLOP/s
-  constexpr double kFloorUs = 16.0;  // a dependent launch plus its split-K reduction
+  constexpr double kFloorUs = 10.0;  // a small dependent launch (reductions are finished together later)
   std::vector<double> load(groups, 0.0);
   std::vector<int> members(groups, 0);
   for (int i = 0; i < n; ++i)
@@ -429,9 +429,17 @@ std::vector<std::string> FBOSession::IssueOrder() const {
 
 void FBOSession::Compute() {
   CHECK(finalized_) << "Please Setup Session First";
-  for (Kernel* kernel : order_) kernel->Compute();
+  for (Kernel* kernel : order_) {
+    if (skip_ && skip_(kernel)) {
+      // a directly launched node would have sent the deferred batch out before it ran:
+      // keep the batches of the remaining nodes as they are in the full pass
+      if (!kernel->Deferrable() && !kernel->absorbed()) context_->Flush();
+      continue;
+    }
+    kernel->Compute();
+  }
   context_->Flush();  // convolutions still deferred at the end of the pass
-  computed_once_ = true;
+  if (!skip_) computed_once_ = true;
 }
 
 void FBOSession::Run(const NamedTensorList& inputs_cpu) {
@@ -442,13 +450,16 @@ void FBOSession::Run(const NamedTensorList& inputs_cpu) {
 void FBOSession::RunProfiled(std::vector<NodeTiming>* timings) {
   CHECK(finalized_) << "Please Setup Session First";
   hipStream_t s = static_cast<hipStream_t>(context_->stream());
-  const std::vector<Kernel*>& live = order_;
+  // file order, every node whole: per-node timing wants nothing deferred across nodes
+  std::vector<Kernel*> live;
+  for (auto& kernel : kernels_)
+    if (!CheckKernelReady(kernel.get())) live.push_back(kernel.get());
   std::vector<hipEvent_t> ev(live.size() + 1);
   for (auto& e : ev) OGLE_HIP_CALL(hipEventCreate(&e));
   OGLE_HIP_CALL(hipEventRecord(ev[0], s));
   for (size_t i = 0; i < live.size(); ++i) {
     live[i]->Compute();
-    context_->Flush();  // per-node timing: nothing stays deferred across nodes
+    context_->Flush();
     OGLE_HIP_CALL(hipEventRecord(ev[i + 1], s));
   }
   OGLE_HIP_CALL(hipStreamSynchronize(s));

@@ -52,7 +52,7 @@ class FBOSession {
   // Records one Compute() pass into a hipGraph (once per slot) and replays it.
   // `after_pass`, if given, enqueues more work on the context's stream (a detector's
   // post-processing) that is recorded into the same graph; it must not allocate.
-  static constexpr int kGraphSlots = 2;
+  static constexpr int kGraphSlots = 3;
   void CaptureGraph(int slot = 0, const std::function<void()>& after_pass = {});
   void LaunchGraph(int slot = 0);
   bool graph_captured(int slot = 0) const { return graph_exec_[slot] != nullptr; }
@@ -77,10 +77,18 @@ class FBOSession {
   void set_reorder(bool on) { reorder_ = on; }
   bool reorder() const { return reorder_; }
   // Whether Setup may run two Conv nodes that read the same tensor with the same
-  // attributes as one launch (OGLE_NO_SIBLING_FUSION=1 also switches it off).  Takes
-  // effect at the first Run.
+  // attributes as one launch (OGLE_SIBLING_FUSION=1 also switches it on).  Off by
+  // default: a fused pair fetches its input once, but its wide tile cannot share a grid
+  // with the small convolutions of a serial chain the way the two separate heads do, and
+  // on MobileNet-SSD at batch 16 the pass measured 5 % slower with it.  Takes effect at
+  // the first Run.
   void set_fuse_siblings(bool on) { fuse_siblings_ = on; }
   bool fuse_siblings() const { return fuse_siblings_; }
+  // Nodes for which `skip` returns true are left out of every following Compute() (and of
+  // a graph recorded from it); an empty function restores the full pass.  For measurement
+  // only: the time of a pass without a family of nodes, subtracted from the time of the
+  // full pass, is what that family costs inside the pass.  Outputs are stale meanwhile.
+  void set_skip(const std::function<bool(const Kernel*)>& skip) { skip_ = skip; }
   // Node names in the order Compute() issues them (after the first Run).
   std::vector<std::string> IssueOrder() const;
 
@@ -102,11 +110,12 @@ class FBOSession {
   std::vector<bool> ready_;
   bool allow_resized_ = false;
   bool reorder_ = true;
-  bool fuse_siblings_ = true;
+  bool fuse_siblings_ = false;
   std::vector<Kernel*> order_;  // the per-pass kernels in issue order (not owned)
+  std::function<bool(const Kernel*)> skip_;
   IntList default_input_sizes_;
-  void* graph_[kGraphSlots] = {nullptr, nullptr};       // hipGraph_t
-  void* graph_exec_[kGraphSlots] = {nullptr, nullptr};  // hipGraphExec_t
+  void* graph_[kGraphSlots] = {};       // hipGraph_t
+  void* graph_exec_[kGraphSlots] = {};  // hipGraphExec_t
 };
 
 }  // namespace opengl

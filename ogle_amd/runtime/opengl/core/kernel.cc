@@ -2,6 +2,7 @@
 
 #include <sstream>
 
+#include "opengl/core/context.h"
 #include "opengl/core/fbo_session.h"
 #include "opengl/core/tensor.h"
 
@@ -21,7 +22,15 @@ void Kernel::Setup(const dlxnet::NodeProto& node, FBOSession* session) {
   SetupAttr(node.attr());
 }
 
-void Kernel::Compute() { Compute(input_tensors_, output_tensors_); }
+void Kernel::Compute() {
+  struct Scope {  // closes the node's range also when Compute throws
+    Context* c;
+    ~Scope() { c->EndNode(); }
+  };
+  context_->BeginNode(kernel_name_ + "#" + kernel_type_ + "#");
+  Scope scope{context_};
+  Compute(input_tensors_, output_tensors_);
+}
 
 DataFormat Kernel::GetOutputDFormat(int i) const {
   CHECK_GE(i, 0);

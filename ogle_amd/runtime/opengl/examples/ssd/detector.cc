@@ -105,8 +105,10 @@ void Detector::EnqueuePostprocess(const TensorNameList& names, int raw_width, in
   a.kept_rect_dev = static_cast<int32_t*>(rect_dev_->device_ptr());
   session_->context()->Flush();
   hipStream_t s = static_cast<hipStream_t>(session_->context()->stream());
+  const int64_t before = ogle_hip_launch_count();
   const int32_t st = ogle_hip_ssd_detect(&a, s);
   if (st != OGLE_OK) LOG(FATAL) << "ogle_hip_ssd_detect: " << ogle_hip_last_error();
+  session_->context()->LogLaunches("detector.score_filter#Detector#", before);
 }
 
 void Detector::Readback() {
@@ -219,8 +221,10 @@ void Detector::EnqueueTopkNms() {
   a.final_box_dev = static_cast<float*>(fbox_dev_->device_ptr());
   a.final_rect_dev = static_cast<int32_t*>(frect_dev_->device_ptr());
   hipStream_t s = static_cast<hipStream_t>(session_->context()->stream());
+  const int64_t before = ogle_hip_launch_count();
   const int32_t st = ogle_hip_ssd_topk_nms(&a, s);
   if (st != OGLE_OK) LOG(FATAL) << "ogle_hip_ssd_topk_nms: " << ogle_hip_last_error();
+  session_->context()->LogLaunches("detector.topk_nms#Detector#", before);
 }
 
 void Detector::ReadbackFinal(std::vector<std::vector<BoxInfo>>* final_boxes) {

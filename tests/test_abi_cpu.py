@@ -21,7 +21,7 @@ def test_library_exports_every_declared_symbol():
     lib = H.lib()
     for name in declared:
         assert getattr(lib, name) is not None
-    assert lib.ogle_hip_abi_version() == 100
+    assert lib.ogle_hip_abi_version() == 101
 
 
 def test_registry_covers_the_reference_shader_table():

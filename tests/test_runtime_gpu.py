@@ -623,3 +623,40 @@ def test_unaligned_head_also_read_by_another_node_keeps_its_own_buffer(second_re
     else:
         assert sess.tensor_device_ptr("a") == base
         assert sess.tensor_device_ptr("b") == base + 2268
+
+
+def test_sibling_heads_fused_into_one_launch():
+    """With sibling fusion on, the box and class head of a feature map run as one contraction
+    with two destinations (OgleConvArgs.output2_dev).  Every head output still matches the
+    oracle on the device's own feature map, and agrees with the one-launch-per-node run to
+    summation order; the absorbed node no longer launches anything."""
+    g, info = models.mobilenet_v1_ssd(4, seed=77, with_weights=True)
+    x = rng(78).uniform(-1, 1, (4, 300, 300, 3)).astype(np.float32)
+    runs = {}
+    for fuse in (False, True):
+        sess = session.Session()
+        sess.set_fuse_siblings(fuse)
+        sess.load_graph(g)
+        sess.run({"input": x})
+        plan = sess.launch_plan()
+        runs[fuse] = ({n: sess.get_output(n, "ANY") for n in
+                       ["box_preds", "cls_logits"] + ["head%d.%s" % (i, k) for i in range(6) for k in ("loc", "conf")]},
+                      plan, sess)
+    labels = " ".join(l for l, _ in runs[True][1])
+    assert "head0.loc#Conv#" in labels and "head0.conf#Conv#" not in labels   # absorbed by its sibling
+    assert "head0.conf#Conv#" in " ".join(l for l, _ in runs[False][1])
+    feats = ["block11.pw", "block13.pw", "extra1.conv", "extra2.conv", "extra3.conv", "extra4.conv"]
+    sess = runs[True][2]
+    for i, feat in enumerate(feats):
+        xin = sess.get_output(feat, "NHWC")
+        for kind in ("loc", "conf"):
+            name = "head%d.%s" % (i, kind)
+            w, b = info["weights"][name]
+            ref = O.conv2d(xin, w, b, 1, 1)
+            got = runs[True][0][name].reshape(ref.shape)
+            assert_conv_close(got, ref, O.conv2d_abs(xin, w, b, 1, 1), FP32_RTOL, "fused " + name)
+    for n in ("box_preds", "cls_logits"):
+        a, b = runs[True][0][n], runs[False][0][n]
+        assert np.abs(a - b).max() <= 2e-5 * np.abs(b).max(), n
+    sess.compute(graph=True)
+    np.testing.assert_array_equal(sess.get_output("cls_logits", "ANY"), runs[True][0]["cls_logits"])
