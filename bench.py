@@ -40,43 +40,62 @@ def build_session(batch, seed=20240005, input_seed=None):
     return s, info
 
 
-FAMILIES = [
-    # name, bound, which layers, label parts that select the family's nodes
-    ("pointwise 1x1 backbone (MFMA implicit GEMM)", "mfma",
-     lambda l: l["kind"] == "pw" and l["name"].startswith("block"),
-     ["block%d.pw#" % i for i in range(1, 14)]),
-    ("depthwise 3x3", "hbm", lambda l: l["kind"] == "dw", ["block%d.dw#" % i for i in range(1, 14)]),
-    ("SSD heads + extras chain (dense 3x3 and 1x1, MFMA implicit GEMM)", "mfma",
-     lambda l: l["name"].startswith("head") or l["name"].startswith("extra"), ["head", "extra"]),
-    ("dense 3x3 stem (direct MFMA)", "hbm", lambda l: l["name"] == "conv0", ["conv0#"]),
-]
+def family_of(nodes, layers):
+    """Kernel family of one entry of the launch plan, from the nodes it was launched for."""
+    fams = set()
+    for n in nodes:
+        l = layers.get(n)
+        if l is None:
+            fams.add("concat + detector tail (decode / score filter, top-k + NMS)")
+        elif n.startswith("head") or n.startswith("extra"):
+            fams.add("SSD heads + extras chain (dense 3x3 and 1x1, MFMA implicit GEMM)")
+        elif l["kind"] == "pw":
+            fams.add("pointwise 1x1 backbone (MFMA implicit GEMM)")
+        elif l["kind"] == "dw":
+            fams.add("depthwise 3x3")
+        else:
+            fams.add("dense 3x3 stem (direct MFMA)")
+    return " + ".join(sorted(fams))
 
 
-def per_family_roofline(sess, info, batch, full_ms, steps, warmup):
-    """What each kernel family costs INSIDE the replayed pass: the pass is recorded again
-    without the family's nodes and timed the same way (HIP events on the session's stream around
-    `steps` graph replays); full minus without is the family's time, launch gaps and tails
-    included, so the rows add up to the pass.  FLOPs / bytes are the layers' algorithmic work."""
-    plan = sess.launch_plan(with_detect=True)
+def per_family_roofline(sess, info, batch, passes):
+    """Kernel time per family from the kernels' own durations: every kernel of `passes` eager
+    passes carries a start / stop HIP event pair that the device stamps with the kernel's begin
+    and end (ogle_hip_kernel_timing_begin), the same quantity a rocprofv3 kernel trace reports,
+    and the launch plan says which node(s) each kernel ran for.  FLOPs / bytes are the layers'
+    algorithmic work (2 x multiply-adds; input + weights + bias + output once each)."""
+    import re
+    layers = {l["name"]: l for l in info["layers"]}
+    fams, per_label = {}, {}
+    dispatches = 0
+    for p in range(passes):
+        plan = sess.launch_plan(with_detect=True, durations=True)
+        dispatches = sum(len(us) for _, us in plan)
+        for label, us in plan:
+            nodes = [m[0] for m in re.findall(r"([^#+:]+)#([A-Za-z0-9_]+)#", label)]
+            name = family_of(nodes, layers)
+            f = fams.setdefault(name, dict(us=0.0, flops=0.0, bytes=0.0, launches=0, layers=0))
+            f["us"] += sum(us) / passes
+            per_label[label] = per_label.get(label, 0.0) + sum(us) / passes
+            if p == 0:
+                f["launches"] += len(us)
+                if not label.startswith("reduce:"):
+                    for n in nodes:
+                        if n in layers:
+                            f["layers"] += 1
+                            f["flops"] += layers[n]["flops_per_image"] * batch
+                            f["bytes"] += layers[n]["act_bytes_per_image"] * batch + layers[n]["weight_bytes"]
     out = []
-    for name, bound, pick, parts in FAMILIES:
-        layers = [l for l in info["layers"] if pick(l)]
-        names = {l["name"] for l in layers}
-        launches = sum(k for label, k in plan if {p.split("#")[0] for p in label.split("+")} & names)
-        without = sess.time_without(parts, warmup, steps, with_detect=True) / steps
-        ms = max(full_ms - without, 1e-6)
-        flops = float(sum(l["flops_per_image"] for l in layers)) * batch
-        nbytes = float(sum(l["act_bytes_per_image"] * batch + l["weight_bytes"] for l in layers))
-        tflops, gbs = flops / ms / 1e9, nbytes / ms / 1e6
-        out.append(dict(kernel=name, layers=len(layers), launches=launches, ms_per_step=round(ms, 4),
-                        avg_launch_us=round(ms * 1e3 / max(launches, 1), 2), bound=bound,
+    for name, f in fams.items():
+        bound = "mfma" if "MFMA implicit GEMM" in name else "hbm"
+        tflops, gbs = f["flops"] / f["us"] / 1e6, f["bytes"] / f["us"] / 1e3
+        out.append(dict(kernel=name, layers=f["layers"], launches=f["launches"], ms_per_step=round(f["us"] / 1e3, 4),
+                        avg_launch_us=round(f["us"] / max(f["launches"], 1), 2), bound=bound,
                         tflops=round(tflops, 2), gbs=round(gbs, 1),
                         frac=round(gbs / HBM_PEAK_GBS if bound == "hbm" else tflops / MFMA_F32_PEAK_TFLOPS, 4),
-                        flops_per_step=flops, bytes_per_step=nbytes))
-    # what is left: transposes / reshapes (views), the two concats, decode + score filter, top-k + NMS
-    rest = full_ms - sum(f["ms_per_step"] for f in out)
+                        flops_per_step=f["flops"], bytes_per_step=f["bytes"]))
     out.sort(key=lambda d: -d["ms_per_step"])
-    return out, rest, plan
+    return out, sum(f["us"] for f in fams.values()) / 1e3, dispatches
 
 
 def calibration_copy(megabytes=256, launches=3):
@@ -463,8 +482,7 @@ def main():
         for pb in pinned:
             pb.close()
 
-    fams, other_ms, plan = per_family_roofline(sess, info, args.batch, total_ms / args.steps,
-                                               min(args.steps, 100), min(args.warmup, 10))
+    fams, kernel_sum_ms, dispatches = per_family_roofline(sess, info, args.batch, passes=10)
     dom = fams[0]
     roofline = dict(bound=dom["bound"], kernel=dom["kernel"],
                     achieved=dom["gbs"] if dom["bound"] == "hbm" else dom["tflops"],
@@ -472,8 +490,8 @@ def main():
                     unit="GB/s" if dom["bound"] == "hbm" else "TFLOP/s", frac=dom["frac"],
                     traffic=read_traffic_summary(dom["kernel"]), launches_per_step=dom["launches"],
                     avg_launch_us=dom["avg_launch_us"],
-                    measured="HIP events on the session's stream around graph replays of the pass with and "
-                             "without the family's nodes (difference / launches)",
+                    measured="start / stop HIP events carried by every kernel of 10 eager passes (stamped "
+                             "by the device with the kernel's own begin and end), summed over the family",
                     algorithmic_per_step=dom["flops_per_step"] if dom["bound"] == "mfma" else dom["bytes_per_step"])
 
     # batch-1 latency: each pass waits for the previous one
@@ -504,8 +522,8 @@ def main():
         "network_tflops": round(2803531136 * args.batch / (ms_per_step * 1e-3) / 1e12, 2),
         "roofline": roofline,
         "kernels": fams,
-        "non_conv_ms_per_step": round(other_ms, 4),
-        "dispatches_per_step": sum(k for _, k in plan),
+        "kernel_time_sum_ms_per_step": round(kernel_sum_ms, 4),
+        "dispatches_per_step": dispatches,
         "with_host_upload": upload,
     }
     if not args.skip_kernel_table:

@@ -83,6 +83,20 @@ int32_t ogle_hip_abi_version(void);
  * profiler trace of a replayed pass is lined up with the graph's nodes. */
 int64_t ogle_hip_launch_count(void);
 
+/*
+ * Kernel timing.  Between _begin and _end every kernel the calling thread launches through
+ * this library carries its own start / stop HIP events, stamped by the device with the
+ * kernel's own begin and end (no launch gaps, unlike events recorded between launches), so
+ * the durations are the ones a profiler's kernel trace shows.  _end waits for the kernels,
+ * writes their durations in launch order (one entry per device operation counted by
+ * ogle_hip_launch_count; 0 for an operation that is not a kernel) and returns how many
+ * there were (may exceed `capacity`), or a negative status.  Not for use while the stream
+ * is being captured.  The reference's counterpart is its per-node TraceMe scope with
+ * glFinish (ogl_runtime/opengl/core/fbo_session.cc:128-151).
+ */
+int32_t ogle_hip_kernel_timing_begin(void);
+int64_t ogle_hip_kernel_timing_end(float* microseconds, int64_t capacity);
+
 /* Message of the calling thread's most recent failure ("" if none). */
 const char* ogle_hip_last_error(void);
 const char* ogle_hip_status_string(int32_t status);

@@ -117,29 +117,22 @@ int32_t ogle_rt_profile_entry(OgleSession* s, int32_t i, const char** label, con
                               float* ms);
 
 /*
- * Time of `iters` replays (after `warmup`) of the pass WITHOUT the nodes whose label
- * "<node>#<type>#" contains one of the n_parts strings in label_parts, recorded as its own
- * hipGraph and timed with HIP events on the session's stream like ogle_rt_time_compute.
- * The difference to the full pass is what those nodes cost inside the pass, launch gaps
- * and all: a per-family time that adds up to the pass.  Outputs are stale afterwards until
- * the next full pass.
- */
-int32_t ogle_rt_time_without(OgleSession* s, const char* const* label_parts, int32_t n_parts,
-                             int32_t warmup, int32_t iters, int32_t with_detect, float* total_ms);
-
-/*
  * Dispatch sequence of a pass.  ogle_rt_launch_plan makes one eager pass (with_detect:
  * followed by the detector's device work) and records, in issue order, every call into the
  * kernel library with the node(s) it was made for and the number of device operations it
  * became; it returns the number of entries.  ogle_rt_launch_plan_entry reads entry i: its
  * label ("<node>#<type>#", the reference's TraceMe label, fbo_session.cc:140-153; the
- * nodes of convolutions that went out as one batch are joined with '+') and its dispatch
- * count.  A replayed hipGraph of the pass issues exactly this sequence, so a profiler's
- * kernel trace of the replays can be attributed to layers position by position.
+ * nodes of convolutions that went out as one batch are joined with '+'; "reduce:" marks
+ * the grid that finishes their split-K reductions), its dispatch count, and the duration
+ * of each of its device operations in that pass (up to `capacity` values), taken from
+ * events the device stamps with the kernel's own begin and end
+ * (ogle_hip_kernel_timing_begin).  A replayed hipGraph of the pass issues exactly this
+ * sequence, so a profiler's kernel trace of the replays can be attributed to layers
+ * position by position, and the durations here are the same quantity that trace shows.
  */
 int32_t ogle_rt_launch_plan(OgleSession* s, int32_t with_detect);
 int32_t ogle_rt_launch_plan_entry(OgleSession* s, int32_t i, const char** label,
-                                  int32_t* dispatches);
+                                  int32_t* dispatches, float* microseconds, int32_t capacity);
 
 /* Shape of a tensor by name (FindTensorByName): writes up to 8 dims, returns rank. */
 int32_t ogle_rt_tensor_shape(OgleSession* s, const char* name, int32_t* dims);

@@ -2,6 +2,8 @@
 // dispatch from op-level entry points to the HIP launchers.
 #include <cstring>
 #include <string>
+#include <utility>
+#include <vector>
 
 #include "common.h"
 
@@ -18,7 +20,32 @@ void set_error(const char* fmt, ...) {
 
 static thread_local int64_t g_launches = 0;
 
-void note_launch() { ++g_launches; }
+// Kernel timing state of the calling thread: one (start, stop) event pair per launch, in
+// launch order; a device operation that is not a kernel holds a null pair.
+struct TimingState {
+  bool on = false;
+  std::vector<std::pair<hipEvent_t, hipEvent_t>> events;
+};
+static thread_local TimingState g_timing;
+
+bool next_timing_events(hipEvent_t* start, hipEvent_t* stop) {
+  if (!g_timing.on) return false;
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) {
+    if (e0 != nullptr) (void)hipEventDestroy(e0);
+    g_timing.on = false;  // cannot time: fall back to plain launches
+    return false;
+  }
+  g_timing.events.emplace_back(e0, e1);
+  *start = e0;
+  *stop = e1;
+  return true;
+}
+
+void note_launch() {
+  ++g_launches;
+  if (g_timing.on) g_timing.events.emplace_back(nullptr, nullptr);
+}
 
 int32_t check_launch(const char* kernel) {
   const hipError_t e = hipGetLastError();
@@ -159,6 +186,38 @@ extern "C" {
 int32_t ogle_hip_abi_version(void) { return 101; }
 
 int64_t ogle_hip_launch_count(void) { return g_launches; }
+
+int32_t ogle_hip_kernel_timing_begin(void) {
+  for (auto& e : g_timing.events) {
+    if (e.first != nullptr) (void)hipEventDestroy(e.first);
+    if (e.second != nullptr) (void)hipEventDestroy(e.second);
+  }
+  g_timing.events.clear();
+  g_timing.on = true;
+  return OGLE_OK;
+}
+
+int64_t ogle_hip_kernel_timing_end(float* microseconds, int64_t capacity) {
+  g_timing.on = false;
+  const int64_t n = (int64_t)g_timing.events.size();
+  int32_t status = OGLE_OK;
+  for (int64_t i = 0; i < n; ++i) {
+    auto& e = g_timing.events[i];
+    float ms = 0.f;
+    if (e.first != nullptr) {
+      if (hipEventSynchronize(e.second) != hipSuccess ||
+          hipEventElapsedTime(&ms, e.first, e.second) != hipSuccess) {
+        set_error("kernel_timing_end: event %lld could not be read", (long long)i);
+        status = OGLE_ERR_LAUNCH;
+      }
+      (void)hipEventDestroy(e.first);
+      (void)hipEventDestroy(e.second);
+    }
+    if (microseconds != nullptr && i < capacity) microseconds[i] = ms * 1e3f;
+  }
+  g_timing.events.clear();
+  return status != OGLE_OK ? status : n;
+}
 
 const char* ogle_hip_last_error(void) { return g_error; }
 

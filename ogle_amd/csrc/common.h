@@ -2,6 +2,7 @@
 #ifndef OGLE_CSRC_COMMON_H_
 #define OGLE_CSRC_COMMON_H_
 
+#include <hip/hip_ext.h>
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 
@@ -28,6 +29,24 @@ int32_t check_launch(const char* kernel);
 void note_launch();
 
 inline hipStream_t as_stream(ogle_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+
+// Kernel timing (ogle_hip_kernel_timing_begin / _end): while it is on for the calling
+// thread, every kernel is launched with a start and a stop event of its own, which the
+// runtime stamps with the kernel's own begin and end on the device.  next_timing_events
+// hands out the pair for the next launch, or returns false when timing is off.
+bool next_timing_events(hipEvent_t* start, hipEvent_t* stop);
+
+// Every kernel of the library is launched through this.
+template <typename F, typename... Args>
+inline void launch(F kernel, const dim3& grid, const dim3& block, unsigned shared_bytes,
+                   hipStream_t stream, Args... args) {
+  hipEvent_t e0, e1;
+  if (next_timing_events(&e0, &e1)) {
+    hipExtLaunchKernelGGL(kernel, grid, block, shared_bytes, stream, e0, e1, 0, args...);
+  } else {
+    hipLaunchKernelGGL(kernel, grid, block, shared_bytes, stream, args...);
+  }
+}
 
 inline int ceil_div(long a, long b) { return static_cast<int>((a + b - 1) / b); }
 

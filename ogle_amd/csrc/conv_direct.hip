@@ -248,7 +248,7 @@ int32_t run_direct(const OgleConvArgs& a, hipStream_t s) {
       if (kidx >= ktot) taps.dy[kidx] = -0x40000000;
     }
 #define OGLE_STEM_CASE(KS)                                                                        \
-  hipLaunchKernelGGL((conv_stem_mfma<T, KS>), dim3(blocks), dim3(256), 0, s, x, w, a.bias_dev, y,  \
+  launch((conv_stem_mfma<T, KS>), dim3(blocks), dim3(256), 0, s, x, w, a.bias_dev, y,  \
                      a.in_h, a.in_w, a.in_c, a.out_h, a.out_w, a.out_c, a.stride, ep, ktot,       \
                      (int)pixels_all, tiles_m, (unsigned)x_bytes, (unsigned)y_bytes, taps)
     if (ks <= 5) OGLE_STEM_CASE(5);
@@ -268,11 +268,11 @@ int32_t run_direct(const OgleConvArgs& a, hipStream_t s) {
     if (blocks > 256 * 32) blocks = 256 * 32;
     if (blocks < 1) blocks = 1;
     if (wide) {
-      hipLaunchKernelGGL((conv_direct_small_k<T, 16>), dim3(blocks), dim3(256), lds, s, x, w,
+      launch((conv_direct_small_k<T, 16>), dim3(blocks), dim3(256), lds, s, x, w,
                          a.bias_dev, y, a.n, a.in_h, a.in_w, a.in_c, a.out_h, a.out_w, a.out_c,
                          a.kernel_size, a.stride, a.padding, a.dilation, ep, ktot);
     } else {
-      hipLaunchKernelGGL((conv_direct_small_k<T, 4>), dim3(blocks), dim3(256), lds, s, x, w,
+      launch((conv_direct_small_k<T, 4>), dim3(blocks), dim3(256), lds, s, x, w,
                          a.bias_dev, y, a.n, a.in_h, a.in_w, a.in_c, a.out_h, a.out_w, a.out_c,
                          a.kernel_size, a.stride, a.padding, a.dilation, ep, ktot);
     }
@@ -282,7 +282,7 @@ int32_t run_direct(const OgleConvArgs& a, hipStream_t s) {
   int blocks = ceil_div(total, 256);
   if (blocks > 256 * 64) blocks = 256 * 64;
   if (blocks < 1) blocks = 1;
-  hipLaunchKernelGGL((conv_direct_general<T>), dim3(blocks), dim3(256), 0, s, x, w, a.bias_dev,
+  launch((conv_direct_general<T>), dim3(blocks), dim3(256), 0, s, x, w, a.bias_dev,
                      y, a.n, a.in_h, a.in_w, a.in_c, a.out_h, a.out_w, a.out_c, a.kernel_size,
                      a.stride, a.padding, a.dilation, a.group, ep);
   return check_launch("conv_direct_general");

@@ -254,7 +254,7 @@ int32_t launch_rows(const OgleConvArgs& a, hipStream_t s, const Epilogue& ep, in
   const int segs = (a.out_h + seg_rows - 1) / seg_rows, cols = (a.out_w + Q - 1) / Q, cv = a.in_c / V;
   const long total = (long)a.n * segs * cols * cv;
   const int blocks = (ceil_div(total, 256) + 7) / 8 * 8;  // whole XCD rounds
-  hipLaunchKernelGGL((dwconv3x3_rows<T, S, Q, PF>), dim3(blocks), dim3(256), 0, s,
+  launch((dwconv3x3_rows<T, S, Q, PF>), dim3(blocks), dim3(256), 0, s,
                      static_cast<const T*>(a.input_dev), static_cast<const T*>(a.filter_dev),
                      a.bias_dev, static_cast<T*>(a.output_dev), a.in_h, a.in_w, a.in_c, a.out_h,
                      a.out_w, a.padding, ep,
@@ -296,7 +296,7 @@ int32_t run_dw(const OgleConvArgs& a, hipStream_t s) {
   int blocks = ceil_div(total, 256);
   if (blocks > 256 * 64) blocks = 256 * 64;
   if (blocks < 1) blocks = 1;
-  hipLaunchKernelGGL((dwconv_general<T>), dim3(blocks), dim3(256), 0, s,
+  launch((dwconv_general<T>), dim3(blocks), dim3(256), 0, s,
                      static_cast<const T*>(a.input_dev), static_cast<const T*>(a.filter_dev),
                      a.bias_dev, static_cast<T*>(a.output_dev), a.n, a.in_h, a.in_w, a.in_c,
                      a.out_h, a.out_w, a.kernel_size, a.stride, a.padding, a.dilation, ep);

@@ -1099,29 +1099,29 @@ Prepared prepare(const OgleConvArgs& a, long m, const IgemmPlan& p) {
 #define OGLE_IGEMM_DISPATCH_C(K, T, ROWB, PW, cfg, grid, s, arg)                             \
   switch (cfg) {                                                                             \
     case CFG_128x128:                                                                        \
-      hipLaunchKernelGGL((K<T, 128, 128, 2, 2, ROWB, PW>), dim3(grid), dim3(256), 0, s, arg); \
+      launch((K<T, 128, 128, 2, 2, ROWB, PW>), dim3(grid), dim3(256), 0, s, arg); \
       break;                                                                                 \
     case CFG_128x64:                                                                         \
-      hipLaunchKernelGGL((K<T, 128, 64, 2, 2, ROWB, PW>), dim3(grid), dim3(256), 0, s, arg);  \
+      launch((K<T, 128, 64, 2, 2, ROWB, PW>), dim3(grid), dim3(256), 0, s, arg);  \
       break;                                                                                 \
     case CFG_64x64:                                                                          \
-      hipLaunchKernelGGL((K<T, 64, 64, 2, 2, ROWB, PW>), dim3(grid), dim3(256), 0, s, arg);   \
+      launch((K<T, 64, 64, 2, 2, ROWB, PW>), dim3(grid), dim3(256), 0, s, arg);   \
       break;                                                                                 \
     case CFG_128x96:                                                                         \
-      hipLaunchKernelGGL((K<T, 128, 96, 4, 1, ROWB, PW>), dim3(grid), dim3(256), 0, s, arg);  \
+      launch((K<T, 128, 96, 4, 1, ROWB, PW>), dim3(grid), dim3(256), 0, s, arg);  \
       break;                                                                                 \
     case CFG_128x160:                                                                        \
-      hipLaunchKernelGGL((K<T, 128, 160, 4, 1, ROWB, PW>), dim3(grid), dim3(256), 0, s, arg); \
+      launch((K<T, 128, 160, 4, 1, ROWB, PW>), dim3(grid), dim3(256), 0, s, arg); \
       break;                                                                                 \
     default:                                                                                 \
-      hipLaunchKernelGGL((K<T, 128, 32, 4, 1, ROWB, PW>), dim3(grid), dim3(256), 0, s, arg);  \
+      launch((K<T, 128, 32, 4, 1, ROWB, PW>), dim3(grid), dim3(256), 0, s, arg);  \
       break;                                                                                 \
   }
 
 void launch_wave(int dtype, bool pw, int cfg, const Prepared& pr, hipStream_t s) {
   const dim3 grid(pr.grid), block(256);
 #define OGLE_WAVE_LAUNCH(T, PW, TS) \
-  hipLaunchKernelGGL((conv_igemm_wave_kernel<T, PW, TS>), grid, block, 0, s, pr.prob)
+  launch((conv_igemm_wave_kernel<T, PW, TS>), grid, block, 0, s, pr.prob)
 #define OGLE_WAVE_PICK(T)                                                 \
   if (cfg == CFG_WAVE32) {                                                \
     if (pw) OGLE_WAVE_LAUNCH(T, true, 32); else OGLE_WAVE_LAUNCH(T, false, 32); \
@@ -1141,10 +1141,10 @@ template <typename T>
 void launch_reduce_single(const Prepared& pr, hipStream_t s) {
   const dim3 grid(pr.reduce_grid), block(256);
   switch (pr.reduce_lanes) {
-    case 8: hipLaunchKernelGGL((splitk_reduce_kernel<T, 8>), grid, block, 0, s, pr.red); break;
-    case 4: hipLaunchKernelGGL((splitk_reduce_kernel<T, 4>), grid, block, 0, s, pr.red); break;
-    case 2: hipLaunchKernelGGL((splitk_reduce_kernel<T, 2>), grid, block, 0, s, pr.red); break;
-    default: hipLaunchKernelGGL((splitk_reduce_kernel<T, 1>), grid, block, 0, s, pr.red); break;
+    case 8: launch((splitk_reduce_kernel<T, 8>), grid, block, 0, s, pr.red); break;
+    case 4: launch((splitk_reduce_kernel<T, 4>), grid, block, 0, s, pr.red); break;
+    case 2: launch((splitk_reduce_kernel<T, 2>), grid, block, 0, s, pr.red); break;
+    default: launch((splitk_reduce_kernel<T, 1>), grid, block, 0, s, pr.red); break;
   }
 }
 
@@ -1234,9 +1234,9 @@ int32_t launch_conv_batch(const OgleConvArgs* args, int count, hipStream_t s,
     } else if (uniform && !is_wave(head.cfg)) {
       OGLE_IGEMM_DISPATCH(conv_igemm_group_kernel, head.dtype, head.cfg, head.pw, grid, s, grp);
     } else if (head.dtype == OGLE_F16) {
-      hipLaunchKernelGGL((conv_igemm_mixed_kernel<__half, 128>), dim3(grid), dim3(256), 0, s, grp);
+      launch((conv_igemm_mixed_kernel<__half, 128>), dim3(grid), dim3(256), 0, s, grp);
     } else {
-      hipLaunchKernelGGL((conv_igemm_mixed_kernel<float, kRowBytesF32>), dim3(grid), dim3(256), 0,
+      launch((conv_igemm_mixed_kernel<float, kRowBytesF32>), dim3(grid), dim3(256), 0,
                          s, grp);
     }
     int32_t st = check_launch("conv_igemm_group");
@@ -1251,9 +1251,9 @@ int32_t launch_conv_batch(const OgleConvArgs* args, int count, hipStream_t s,
       if (head.dtype == OGLE_F16) launch_reduce_single<__half>(one, s);
       else launch_reduce_single<float>(one, s);
     } else if (head.dtype == OGLE_F16) {
-      hipLaunchKernelGGL((splitk_reduce_group_kernel<__half>), rgrid, block, 0, s, red);
+      launch((splitk_reduce_group_kernel<__half>), rgrid, block, 0, s, red);
     } else {
-      hipLaunchKernelGGL((splitk_reduce_group_kernel<float>), rgrid, block, 0, s, red);
+      launch((splitk_reduce_group_kernel<float>), rgrid, block, 0, s, red);
     }
     st = check_launch("splitk_reduce_group");
     if (st != OGLE_OK) return st;
@@ -1283,9 +1283,9 @@ int32_t launch_conv_reduce(const OgleConvArgs* args, int count, hipStream_t s) {
     if (red.count == 0) continue;
     const dim3 rgrid((unsigned)red.first[red.count]), block(256);
     if (dtype == OGLE_F16) {
-      hipLaunchKernelGGL((splitk_reduce_group_kernel<__half>), rgrid, block, 0, s, red);
+      launch((splitk_reduce_group_kernel<__half>), rgrid, block, 0, s, red);
     } else {
-      hipLaunchKernelGGL((splitk_reduce_group_kernel<float>), rgrid, block, 0, s, red);
+      launch((splitk_reduce_group_kernel<float>), rgrid, block, 0, s, red);
     }
     const int32_t st = check_launch("splitk_reduce_group");
     if (st != OGLE_OK) return st;

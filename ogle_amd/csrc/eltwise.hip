@@ -196,11 +196,11 @@ int32_t launch_unary(const OgleUnaryArgs& a, hipStream_t s) {
   const UnaryOp f{a.op, a.min_value, a.max_value};
   const dim3 grid(grid_for(a.count / kVec + 1));
   if (a.dtype == OGLE_F16) {
-    hipLaunchKernelGGL((unary_kernel<__half>), grid, dim3(256), 0, s,
+    launch((unary_kernel<__half>), grid, dim3(256), 0, s,
                        static_cast<const __half*>(a.input_dev), static_cast<__half*>(a.output_dev),
                        (long)a.count, f);
   } else {
-    hipLaunchKernelGGL((unary_kernel<float>), grid, dim3(256), 0, s,
+    launch((unary_kernel<float>), grid, dim3(256), 0, s,
                        static_cast<const float*>(a.input_dev), static_cast<float*>(a.output_dev),
                        (long)a.count, f);
   }
@@ -211,11 +211,11 @@ int32_t launch_binary(const OgleBinaryArgs& a, hipStream_t s) {
   if (a.count == 0) return OGLE_OK;
   const dim3 grid(grid_for(a.count / kVec + 1));
   if (a.dtype == OGLE_F16) {
-    hipLaunchKernelGGL((add_kernel<__half>), grid, dim3(256), 0, s,
+    launch((add_kernel<__half>), grid, dim3(256), 0, s,
                        static_cast<const __half*>(a.a_dev), static_cast<const __half*>(a.b_dev),
                        static_cast<__half*>(a.output_dev), (long)a.count);
   } else {
-    hipLaunchKernelGGL((add_kernel<float>), grid, dim3(256), 0, s,
+    launch((add_kernel<float>), grid, dim3(256), 0, s,
                        static_cast<const float*>(a.a_dev), static_cast<const float*>(a.b_dev),
                        static_cast<float*>(a.output_dev), (long)a.count);
   }
@@ -229,7 +229,7 @@ int32_t launch_batchnorm(const OgleBatchNormArgs& a, hipStream_t s) {
                    aligned16(a.mean_dev) && aligned16(a.var_dev);
   const dim3 grid(grid_for(vec ? total / 4 : total));
 #define OGLE_BN_LAUNCH(T, VEC)                                                                   \
-  hipLaunchKernelGGL((batchnorm_kernel<T, VEC>), grid, dim3(256), 0, s,                          \
+  launch((batchnorm_kernel<T, VEC>), grid, dim3(256), 0, s,                          \
                      static_cast<const T*>(a.input_dev), a.gamma_dev, a.beta_dev, a.mean_dev,    \
                      a.var_dev, static_cast<T*>(a.output_dev), total, a.channels, a.epsilon)
   if (a.dtype == OGLE_F16) {
@@ -280,7 +280,7 @@ int32_t launch_gemm(const OgleGemmArgs& a, hipStream_t s) {
     if (st != OGLE_ERR_UNSUPPORTED) return st;
   }
   const dim3 grid((a.n + kGemmBN - 1) / kGemmBN, (a.m + kGemmBM - 1) / kGemmBM);
-  hipLaunchKernelGGL(gemm_general_kernel, grid, dim3(256), 0, s, a.a_dev, a.b_dev, a.c_dev, a.y_dev,
+  launch(gemm_general_kernel, grid, dim3(256), 0, s, a.a_dev, a.b_dev, a.c_dev, a.y_dev,
                      a.m, a.n, a.k, a.trans_b, a.c_rank, a.alpha, a.beta);
   return check_launch("gemm_general_kernel");
 }

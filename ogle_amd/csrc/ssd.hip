@@ -573,10 +573,10 @@ int32_t launch_topk_nms(const OgleNmsArgs& a, hipStream_t s) {
   p.out_box = reinterpret_cast<float4*>(a.final_box_dev);
   p.out_rect = reinterpret_cast<int4*>(a.final_rect_dev);
   if (a.kept_count_dev == nullptr) {
-    hipLaunchKernelGGL(ssd_topk_nms_kernel<true>, dim3((unsigned)a.batch), dim3(kNmsThreads),
+    launch(ssd_topk_nms_kernel<true>, dim3((unsigned)a.batch), dim3(kNmsThreads),
                        topk_nms_lds_bytes(a.stride, a.topk), s, p);
   } else {
-    hipLaunchKernelGGL(ssd_topk_nms_kernel<false>, dim3((unsigned)a.batch), dim3(kNmsThreads),
+    launch(ssd_topk_nms_kernel<false>, dim3((unsigned)a.batch), dim3(kNmsThreads),
                        topk_nms_lds_bytes(a.stride, a.topk), s, p);
   }
   return check_launch("ssd_topk_nms_kernel");
@@ -587,7 +587,7 @@ int32_t launch_decode(const OgleDecodeArgs& a, hipStream_t s) {
   if (total == 0) return OGLE_OK;
   long blocks = (total + 255) / 256;
   if (blocks > 4096) blocks = 4096;
-  hipLaunchKernelGGL(ssd_decode_kernel, dim3((unsigned)blocks), dim3(256), 0, s,
+  launch(ssd_decode_kernel, dim3((unsigned)blocks), dim3(256), 0, s,
                      reinterpret_cast<const float4*>(a.prediction_dev),
                      reinterpret_cast<const float4*>(a.anchors_dev),
                      reinterpret_cast<float4*>(a.boxes_dev), a.batch, a.priors,
@@ -616,15 +616,15 @@ int32_t launch_detect(const OgleDetectArgs& a, hipStream_t s) {
   const bool sparse = p.kept_count == nullptr;  // validated: all outputs given, batch <= 65535
   if (sparse && a.priors == 0) return OGLE_OK;
   if (sparse || (all_outputs && a.priors > 256 && a.batch <= 65535)) {
-    hipLaunchKernelGGL(ssd_score_kernel,
+    launch(ssd_score_kernel,
                        dim3((unsigned)((a.priors + kScorePriors - 1) / kScorePriors), (unsigned)a.batch),
                        dim3(256), sizeof(float) * kScorePriors * (size_t)a.classes, s, p);
     const int32_t st = check_launch("ssd_score_kernel");
     if (st != OGLE_OK || sparse) return st;
-    hipLaunchKernelGGL(ssd_compact_kernel, dim3((unsigned)a.batch), dim3(kCompactThreads), 0, s, p);
+    launch(ssd_compact_kernel, dim3((unsigned)a.batch), dim3(kCompactThreads), 0, s, p);
     return check_launch("ssd_compact_kernel");
   }
-  hipLaunchKernelGGL(ssd_detect_kernel, dim3((unsigned)a.batch), dim3(256), lds, s, p);
+  launch(ssd_detect_kernel, dim3((unsigned)a.batch), dim3(256), lds, s, p);
   return check_launch("ssd_detect_kernel");
 }
 
@@ -632,7 +632,7 @@ int32_t launch_expf(const float* x, float* y, int64_t n, hipStream_t s) {
   if (n == 0) return OGLE_OK;
   long blocks = (n + 255) / 256;
   if (blocks > 8192) blocks = 8192;
-  hipLaunchKernelGGL(expf_kernel, dim3((unsigned)blocks), dim3(256), 0, s, x, y, (long)n);
+  launch(expf_kernel, dim3((unsigned)blocks), dim3(256), 0, s, x, y, (long)n);
   return check_launch("expf_kernel");
 }
 

@@ -297,7 +297,7 @@ int32_t run_pool(const OglePoolArgs& a, hipStream_t s) {
   const bool whole_image = a.padding == 0 && a.stride == 1 && a.kernel_size == a.in_h &&
                            a.kernel_size == a.in_w && a.pool_type != OGLE_POOL_MAX;
   if (whole_image && a.kernel_size * a.kernel_size >= 16) {
-    hipLaunchKernelGGL((global_avg_kernel<T>), dim3((a.c + 63) / 64, a.n), dim3(256), 0, s, x, y,
+    launch((global_avg_kernel<T>), dim3((a.c + 63) / 64, a.n), dim3(256), 0, s, x, y,
                        a.in_h * a.in_w, a.c);
     return check_launch("global_avg_kernel");
   }
@@ -308,7 +308,7 @@ int32_t run_pool(const OglePoolArgs& a, hipStream_t s) {
         x_bytes < 0x7fffffffL && y_bytes < 0x7fffffffL && total4 > 0) {
       const dim3 grid((unsigned)(((total4 + 255) / 256 + 7) / 8 * 8));  // whole XCD rounds
 #define OGLE_POOL_SMALL(K)                                                                        \
-  hipLaunchKernelGGL((pool_small_kernel<K>), grid, dim3(256), 0, s, x, y, a.in_h, a.in_w, a.c,    \
+  launch((pool_small_kernel<K>), grid, dim3(256), 0, s, x, y, a.in_h, a.in_w, a.c,    \
                      a.out_h, a.out_w, a.stride, a.padding, a.pool_type, (unsigned)total4,        \
                      (unsigned)x_bytes, (unsigned)y_bytes, make_pool_div((unsigned)(a.c / 4)),    \
                      make_pool_div((unsigned)a.out_w), make_pool_div((unsigned)a.out_h))
@@ -320,12 +320,12 @@ int32_t run_pool(const OglePoolArgs& a, hipStream_t s) {
   }
   if (a.c % 4 == 0) {
     const long total = (long)a.n * a.out_h * a.out_w * (a.c / 4);
-    hipLaunchKernelGGL((pool_kernel<T, 4>), dim3(grid_for(total, 256 * 64)), dim3(256), 0, s, x,
+    launch((pool_kernel<T, 4>), dim3(grid_for(total, 256 * 64)), dim3(256), 0, s, x,
                        y, a.n, a.in_h, a.in_w, a.c, a.out_h, a.out_w, a.kernel_size, a.stride,
                        a.padding, a.pool_type);
   } else {
     const long total = (long)a.n * a.out_h * a.out_w * a.c;
-    hipLaunchKernelGGL((pool_kernel<T, 1>), dim3(grid_for(total, 256 * 64)), dim3(256), 0, s, x,
+    launch((pool_kernel<T, 1>), dim3(grid_for(total, 256 * 64)), dim3(256), 0, s, x,
                        y, a.n, a.in_h, a.in_w, a.c, a.out_h, a.out_w, a.kernel_size, a.stride,
                        a.padding, a.pool_type);
   }
@@ -373,15 +373,15 @@ int32_t launch_concat(const OgleConcatArgs& a, hipStream_t s) {
     }
     p.out_run /= vec;
     p.total = a.outer * p.out_run;
-    hipLaunchKernelGGL((concat_kernel<uint4>), dim3(grid_for(p.total)), dim3(256), 0, s, p,
+    launch((concat_kernel<uint4>), dim3(grid_for(p.total)), dim3(256), 0, s, p,
                        static_cast<uint4*>(a.output_dev));
   } else if (esz == 4) {
     p.total = a.outer * p.out_run;
-    hipLaunchKernelGGL((concat_kernel<uint32_t>), dim3(grid_for(p.total)), dim3(256), 0, s, p,
+    launch((concat_kernel<uint32_t>), dim3(grid_for(p.total)), dim3(256), 0, s, p,
                        static_cast<uint32_t*>(a.output_dev));
   } else {
     p.total = a.outer * p.out_run;
-    hipLaunchKernelGGL((concat_kernel<uint16_t>), dim3(grid_for(p.total)), dim3(256), 0, s, p,
+    launch((concat_kernel<uint16_t>), dim3(grid_for(p.total)), dim3(256), 0, s, p,
                        static_cast<uint16_t*>(a.output_dev));
   }
   return check_launch("concat_kernel");
@@ -424,11 +424,11 @@ int32_t launch_transpose(const OgleTransposeArgs& a, hipStream_t s) {
     return OGLE_OK;
   }
   if (esz == 4) {
-    hipLaunchKernelGGL((transpose_kernel<uint32_t>), dim3(grid_for(p.total)), dim3(256), 0, s, p,
+    launch((transpose_kernel<uint32_t>), dim3(grid_for(p.total)), dim3(256), 0, s, p,
                        static_cast<const uint32_t*>(a.input_dev),
                        static_cast<uint32_t*>(a.output_dev));
   } else {
-    hipLaunchKernelGGL((transpose_kernel<uint16_t>), dim3(grid_for(p.total)), dim3(256), 0, s, p,
+    launch((transpose_kernel<uint16_t>), dim3(grid_for(p.total)), dim3(256), 0, s, p,
                        static_cast<const uint16_t*>(a.input_dev),
                        static_cast<uint16_t*>(a.output_dev));
   }
@@ -440,10 +440,10 @@ int32_t launch_pack_filter(const float* src, void* dst, int layout, int dtype, i
   const long total = (long)o * i * kh * kw;
   if (total == 0) return OGLE_OK;
   if (dtype == OGLE_F16) {
-    hipLaunchKernelGGL((pack_filter_kernel<__half>), dim3(grid_for(total)), dim3(256), 0, s, src,
+    launch((pack_filter_kernel<__half>), dim3(grid_for(total)), dim3(256), 0, s, src,
                        static_cast<__half*>(dst), layout, o, i, kh, kw);
   } else {
-    hipLaunchKernelGGL((pack_filter_kernel<float>), dim3(grid_for(total)), dim3(256), 0, s, src,
+    launch((pack_filter_kernel<float>), dim3(grid_for(total)), dim3(256), 0, s, src,
                        static_cast<float*>(dst), layout, o, i, kh, kw);
   }
   return check_launch("pack_filter_kernel");
@@ -453,16 +453,16 @@ int32_t launch_convert(const void* src, int sdt, void* dst, int ddt, int64_t n, 
   if (n == 0) return OGLE_OK;
   const dim3 grid(grid_for(n));
   if (sdt == OGLE_F32 && ddt == OGLE_F16) {
-    hipLaunchKernelGGL((convert_kernel<float, __half>), grid, dim3(256), 0, s,
+    launch((convert_kernel<float, __half>), grid, dim3(256), 0, s,
                        static_cast<const float*>(src), static_cast<__half*>(dst), (long)n);
   } else if (sdt == OGLE_F16 && ddt == OGLE_F32) {
-    hipLaunchKernelGGL((convert_kernel<__half, float>), grid, dim3(256), 0, s,
+    launch((convert_kernel<__half, float>), grid, dim3(256), 0, s,
                        static_cast<const __half*>(src), static_cast<float*>(dst), (long)n);
   } else if (sdt == OGLE_F32 && ddt == OGLE_F32) {
-    hipLaunchKernelGGL((convert_kernel<float, float>), grid, dim3(256), 0, s,
+    launch((convert_kernel<float, float>), grid, dim3(256), 0, s,
                        static_cast<const float*>(src), static_cast<float*>(dst), (long)n);
   } else {
-    hipLaunchKernelGGL((convert_kernel<__half, __half>), grid, dim3(256), 0, s,
+    launch((convert_kernel<__half, __half>), grid, dim3(256), 0, s,
                        static_cast<const __half*>(src), static_cast<__half*>(dst), (long)n);
   }
   return check_launch("convert_kernel");

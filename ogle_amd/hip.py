@@ -30,6 +30,7 @@ SYMBOLS = [
     "ogle_hip_batchnorm", "ogle_hip_gemm", "ogle_hip_gemm_workspace_bytes",
     "ogle_hip_conv2d_noalloc", "ogle_hip_launch_count",
     "ogle_hip_conv2d_batch_begin", "ogle_hip_conv2d_batch_finish",
+    "ogle_hip_kernel_timing_begin", "ogle_hip_kernel_timing_end",
 ]
 CONV_NOALLOC_SCRATCH_BYTES = 16 << 20
 UNARY_RELU, UNARY_CLIP = 0, 1
@@ -165,6 +166,8 @@ def lib():
                                                ctypes.POINTER(ctypes.c_int32)]
         l.ogle_hip_sync.argtypes = [ctypes.c_void_p]
         l.ogle_hip_launch_count.restype = ctypes.c_int64
+        l.ogle_hip_kernel_timing_end.restype = ctypes.c_int64
+        l.ogle_hip_kernel_timing_end.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_int64]
         l.ogle_hip_packed_filter_elems.restype = ctypes.c_int64
         l.ogle_hip_packed_filter_elems.argtypes = [ctypes.c_int32] * 5
         l.ogle_hip_pack_filter.argtypes = [ctypes.c_void_p, ctypes.c_void_p] + \

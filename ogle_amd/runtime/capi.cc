@@ -26,6 +26,7 @@ struct OgleSession {
   std::unique_ptr<opengl::Detector> detector;
   bool device_nms = true;
   std::vector<opengl::Context::LaunchRecord> plan;
+  std::vector<float> plan_us;  // duration of every device operation of the plan, in order
 };
 
 namespace {
@@ -208,59 +209,6 @@ int32_t ogle_rt_time_compute(OgleSession* s, int32_t warmup, int32_t iters, int3
   });
 }
 
-int32_t ogle_rt_time_without(OgleSession* s, const char* const* label_parts, int32_t n_parts,
-                             int32_t warmup, int32_t iters, int32_t with_detect, float* total_ms) {
-  return (int32_t)Guard([&]() -> int64_t {
-    CHECK(s->session->graph_captured(with_detect ? 1 : 0) || !with_detect || s->detector)
-        << "time the full pass first";
-    std::vector<std::string> parts;
-    for (int i = 0; i < n_parts; ++i) parts.emplace_back(label_parts[i]);
-    hipStream_t st = static_cast<hipStream_t>(s->context->stream());
-    opengl::DetectorOptions opt;
-    opt.device_nms = s->device_nms;
-    if (with_detect && !s->detector) {
-      s->detector = opengl::Detector::Create(s->session.get(), opt);
-      s->detector->EnqueueDetect(opt.output_names, 300, 300);
-      s->context->Finish();
-    }
-    const int slot = 2;
-    s->session->DropGraph(slot);
-    s->session->set_skip([parts](const opengl::Kernel* k) {
-      const std::string label = k->kernel_name() + "#" + k->kernel_type() + "#";
-      for (const std::string& p : parts)
-        if (label.find(p) != std::string::npos) return true;
-      return false;
-    });
-    float total = 0.f;
-    try {
-      if (with_detect)
-        s->session->CaptureGraph(slot, [&]() { s->detector->EnqueueDetect(opt.output_names, 300, 300); });
-      else
-        s->session->CaptureGraph(slot);
-      for (int i = 0; i < warmup; ++i) s->session->LaunchGraph(slot);
-      s->context->Finish();
-      hipEvent_t e0, e1;
-      if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess)
-        LOG(FATAL) << "hipEventCreate failed";
-      (void)hipEventRecord(e0, st);
-      for (int i = 0; i < iters; ++i) s->session->LaunchGraph(slot);
-      (void)hipEventRecord(e1, st);
-      s->context->Finish();
-      (void)hipEventElapsedTime(&total, e0, e1);
-      (void)hipEventDestroy(e0);
-      (void)hipEventDestroy(e1);
-    } catch (...) {
-      s->session->set_skip({});
-      s->session->DropGraph(slot);
-      throw;
-    }
-    s->session->set_skip({});
-    s->session->DropGraph(slot);
-    if (total_ms) *total_ms = total;
-    return 0;
-  });
-}
-
 int32_t ogle_rt_launch_plan(OgleSession* s, int32_t with_detect) {
   return (int32_t)Guard([&]() -> int64_t {
     opengl::DetectorOptions opt;
@@ -270,27 +218,41 @@ int32_t ogle_rt_launch_plan(OgleSession* s, int32_t with_detect) {
       s->detector->EnqueueDetect(opt.output_names, 300, 300);  // first use allocates
       s->context->Finish();
     }
+    s->context->Finish();
     s->context->set_launch_log(true);
+    (void)ogle_hip_kernel_timing_begin();
     try {
       s->session->Compute();
       if (with_detect) s->detector->EnqueueDetect(opt.output_names, 300, 300);
       s->context->Flush();
     } catch (...) {
       s->context->set_launch_log(false);
+      (void)ogle_hip_kernel_timing_end(nullptr, 0);
       throw;
     }
     s->plan = s->context->launch_log();
     s->context->set_launch_log(false);
+    int64_t dispatches = 0;
+    for (const auto& r : s->plan) dispatches += r.dispatches;
+    std::vector<float> us(static_cast<size_t>(dispatches > 0 ? dispatches : 1), 0.f);
+    const int64_t timed = ogle_hip_kernel_timing_end(us.data(), dispatches);
     s->context->Finish();
+    CHECK(timed == dispatches) << "kernel timing saw " << timed << " device operations, the launch log "
+                               << dispatches << " (" << ogle_hip_last_error() << ")";
+    s->plan_us.assign(us.begin(), us.begin() + dispatches);
     return (int64_t)s->plan.size();
   });
 }
 
 int32_t ogle_rt_launch_plan_entry(OgleSession* s, int32_t i, const char** label,
-                                  int32_t* dispatches) {
+                                  int32_t* dispatches, float* microseconds, int32_t capacity) {
   if (s == nullptr || i < 0 || i >= (int32_t)s->plan.size()) return -1;
   if (label) *label = s->plan[i].label.c_str();
   if (dispatches) *dispatches = s->plan[i].dispatches;
+  size_t at = 0;
+  for (int32_t j = 0; j < i; ++j) at += s->plan[j].dispatches;
+  for (int32_t k = 0; k < s->plan[i].dispatches && k < capacity && microseconds != nullptr; ++k)
+    microseconds[k] = s->plan_us[at + k];
   return 0;
 }
 

@@ -430,16 +430,10 @@ std::vector<std::string> FBOSession::IssueOrder() const {
 void FBOSession::Compute() {
   CHECK(finalized_) << "Please Setup Session First";
   for (Kernel* kernel : order_) {
-    if (skip_ && skip_(kernel)) {
-      // a directly launched node would have sent the deferred batch out before it ran:
-      // keep the batches of the remaining nodes as they are in the full pass
-      if (!kernel->Deferrable() && !kernel->absorbed()) context_->Flush();
-      continue;
-    }
     kernel->Compute();
   }
   context_->Flush();  // convolutions still deferred at the end of the pass
-  if (!skip_) computed_once_ = true;
+  computed_once_ = true;
 }
 
 void FBOSession::Run(const NamedTensorList& inputs_cpu) {

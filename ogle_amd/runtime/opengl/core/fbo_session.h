@@ -52,7 +52,7 @@ class FBOSession {
   // Records one Compute() pass into a hipGraph (once per slot) and replays it.
   // `after_pass`, if given, enqueues more work on the context's stream (a detector's
   // post-processing) that is recorded into the same graph; it must not allocate.
-  static constexpr int kGraphSlots = 3;
+  static constexpr int kGraphSlots = 2;
   void CaptureGraph(int slot = 0, const std::function<void()>& after_pass = {});
   void LaunchGraph(int slot = 0);
   bool graph_captured(int slot = 0) const { return graph_exec_[slot] != nullptr; }
@@ -84,11 +84,6 @@ class FBOSession {
   // the first Run.
   void set_fuse_siblings(bool on) { fuse_siblings_ = on; }
   bool fuse_siblings() const { return fuse_siblings_; }
-  // Nodes for which `skip` returns true are left out of every following Compute() (and of
-  // a graph recorded from it); an empty function restores the full pass.  For measurement
-  // only: the time of a pass without a family of nodes, subtracted from the time of the
-  // full pass, is what that family costs inside the pass.  Outputs are stale meanwhile.
-  void set_skip(const std::function<bool(const Kernel*)>& skip) { skip_ = skip; }
   // Node names in the order Compute() issues them (after the first Run).
   std::vector<std::string> IssueOrder() const;
 
@@ -112,7 +107,6 @@ class FBOSession {
   bool reorder_ = true;
   bool fuse_siblings_ = false;
   std::vector<Kernel*> order_;  // the per-pass kernels in issue order (not owned)
-  std::function<bool(const Kernel*)> skip_;
   IntList default_input_sizes_;
   void* graph_[kGraphSlots] = {};       // hipGraph_t
   void* graph_exec_[kGraphSlots] = {};  // hipGraphExec_t

@@ -26,7 +26,6 @@ SYMBOLS = [
     "ogle_rt_set_reorder", "ogle_rt_issue_order_name", "ogle_rt_set_device_nms",
     "ogle_rt_detect_results", "ogle_rt_graph_captured", "ogle_rt_hazard_conflicts",
     "ogle_rt_set_fuse_siblings", "ogle_rt_launch_plan", "ogle_rt_launch_plan_entry",
-    "ogle_rt_time_without",
 ]
 
 
@@ -78,9 +77,8 @@ def lib():
         l.ogle_rt_free_pinned.restype = None
         l.ogle_rt_profile.argtypes = [vp]
         l.ogle_rt_launch_plan.argtypes = [vp, i32]
-        l.ogle_rt_time_without.argtypes = [vp, ctypes.POINTER(cp), i32, i32, i32, i32,
-                                           ctypes.POINTER(ctypes.c_float)]
-        l.ogle_rt_launch_plan_entry.argtypes = [vp, i32, ctypes.POINTER(cp), ctypes.POINTER(i32)]
+        l.ogle_rt_launch_plan_entry.argtypes = [vp, i32, ctypes.POINTER(cp), ctypes.POINTER(i32),
+                                                ctypes.POINTER(ctypes.c_float), i32]
         l.ogle_rt_profile_entry.argtypes = [vp, i32, ctypes.POINTER(cp), ctypes.POINTER(cp),
                                             ctypes.POINTER(ctypes.c_float)]
         l.ogle_rt_tensor_shape.argtypes = [vp, cp, ctypes.POINTER(i32)]
@@ -274,24 +272,18 @@ class Session:
             out.append((label.value.decode(), typ.value.decode(), float(ms.value)))
         return out
 
-    def time_without(self, label_parts, warmup, iters, with_detect=False):
-        """Total ms of `iters` graph replays of the pass without the nodes whose label contains
-        one of `label_parts` (see ogle_rt_time_without)."""
-        arr = (ctypes.c_char_p * len(label_parts))(*[p.encode() for p in label_parts])
-        total = ctypes.c_float(0)
-        _check(lib().ogle_rt_time_without(self._h, arr, len(label_parts), warmup, iters,
-                                          1 if with_detect else 0, ctypes.byref(total)))
-        return float(total.value)
-
-    def launch_plan(self, with_detect=False):
-        """Dispatch sequence of one pass: list of (label, dispatches) in issue order; a label
-        is "<node>#<type>#", several joined with '+' for convolutions that share grids."""
+    def launch_plan(self, with_detect=False, durations=False):
+        """Dispatch sequence of one (eager) pass: list of (label, dispatches) in issue order; a
+        label is "<node>#<type>#", several joined with '+' for convolutions that share grids.
+        With durations=True each entry is (label, [microseconds per device operation]), the
+        kernels' own device-stamped durations in that pass."""
         n = _check(lib().ogle_rt_launch_plan(self._h, 1 if with_detect else 0))
         out = []
         label, k = ctypes.c_char_p(), ctypes.c_int32()
+        us = (ctypes.c_float * 64)()
         for i in range(n):
-            _check(lib().ogle_rt_launch_plan_entry(self._h, i, ctypes.byref(label), ctypes.byref(k)))
-            out.append((label.value.decode(), int(k.value)))
+            _check(lib().ogle_rt_launch_plan_entry(self._h, i, ctypes.byref(label), ctypes.byref(k), us, 64))
+            out.append((label.value.decode(), [float(v) for v in us[:k.value]] if durations else int(k.value)))
         return out
 
     def tensor_shape(self, name):

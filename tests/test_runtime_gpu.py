@@ -660,3 +660,20 @@ def test_sibling_heads_fused_into_one_launch():
         assert np.abs(a - b).max() <= 2e-5 * np.abs(b).max(), n
     sess.compute(graph=True)
     np.testing.assert_array_equal(sess.get_output("cls_logits", "ANY"), runs[True][0]["cls_logits"])
+
+
+def test_launch_plan_names_every_dispatch_and_times_it():
+    """The launch plan of a pass: every call into the kernel library with its node label(s) and
+    the device-stamped duration of each kernel it became.  Positive durations, one entry per
+    node that launches something, and the same sequence on every pass."""
+    g, _ = models.separable_block(2, size=19, cin=64, cout=128)
+    x = rng(8100).uniform(0, 6, (2, 19, 19, 64)).astype(np.float32)
+    sess = session.Session()
+    sess.load_graph(g)
+    sess.run({"input": x})
+    want = sess.get_output("pw", "NHWC")
+    plan = sess.launch_plan(durations=True)
+    assert [l for l, _ in plan] == ["dw#Conv#", "pw#Conv#"]
+    assert all(len(us) >= 1 and all(0.5 < u < 1000.0 for u in us) for _, us in plan)
+    assert [l for l, k in sess.launch_plan()] == ["dw#Conv#", "pw#Conv#"]
+    np.testing.assert_array_equal(sess.get_output("pw", "NHWC"), want)
