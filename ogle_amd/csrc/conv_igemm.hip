@@ -319,16 +319,22 @@ __device__ __forceinline__ void igemm_tile(
   const int opitch = (g.o + 3) & ~3;
   const int o2 = g.o - o1;
   float* const pdst = partial != nullptr ? partial + (long)split * g.m_total * opitch : nullptr;
-  constexpr int SROW = WTN + 4;            // floats per staged row (padded)
-  constexpr bool STAGED = 4 * 32 * SROW * 4 <= 2 * STAGE;  // staging fits the K-loop LDS
+  // The staging region (reused K-loop LDS) takes JC 32-column blocks of a wave's tile at a
+  // time: as many as fit, so that a row segment a wave stores is as long as possible.
+  constexpr auto stage_fits = [](int jc) { return 4 * 32 * (jc * 32 + 4) * 4 <= 2 * STAGE; };
+  constexpr int JC = (TN % 4 == 0 && stage_fits(4)) ? 4 : (TN % 2 == 0 && stage_fits(2)) ? 2 : 1;
+  static_assert(stage_fits(JC), "epilogue staging exceeds the K-loop LDS");
+  constexpr int CW = JC * 32;              // columns staged at once
+  constexpr int SROW = CW + 4;             // floats per staged row (padded)
   float* const smw = reinterpret_cast<float*>(lds) + wave * 32 * SROW;
-  if constexpr (STAGED) {
-    if (pdst != nullptr || (sizeof(T) == 4 && (o1 & 3) == 0 && (o2 & 3) == 0)) {
-      constexpr int LPR = WTN / 4;             // lanes covering one staged row
-      constexpr int RPI = 64 / LPR;            // rows one store instruction covers
-      const int cv = lane % LPR;
-      const int rsub = lane / LPR;
-      const int col = n0 + wave_n * WTN + cv * 4;
+  if (pdst != nullptr || (sizeof(T) == 4 && (o1 & 3) == 0 && (o2 & 3) == 0)) {
+    constexpr int LPR = CW / 4;              // lanes covering one staged row
+    constexpr int RPI = 64 / LPR;            // rows one store instruction covers
+    const int cv = lane % LPR;
+    const int rsub = lane / LPR;
+#pragma unroll
+    for (int j0 = 0; j0 < TN; j0 += JC) {
+      const int col = n0 + wave_n * WTN + j0 * 32 + cv * 4;
       float4 bias4 = make_float4(0.f, 0.f, 0.f, 0.f);
       if (pdst == nullptr && bias != nullptr && col < g.o)
         bias4 = *reinterpret_cast<const float4*>(bias + col);
@@ -340,10 +346,10 @@ __device__ __forceinline__ void igemm_tile(
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
+        for (int j = 0; j < JC; ++j)
 #pragma unroll
           for (int r = 0; r < 16; ++r)
-            smw[((r >> 2) * 8 + lh * 4 + (r & 3)) * SROW + j * 32 + l32] = acc[i][j][r];
+            smw[((r >> 2) * 8 + lh * 4 + (r & 3)) * SROW + j * 32 + l32] = acc[i][j0 + j][r];
 #pragma unroll
         for (int it = 0; it < 32 / RPI; ++it) {
           const int row = it * RPI + rsub;
@@ -360,17 +366,20 @@ __device__ __forceinline__ void igemm_tile(
           }
         }
       }
-      return;
     }
-    if constexpr (sizeof(T) == 2) {
-      if ((g.o & 7) == 0 && y2 == nullptr) {
-        // fp16 output: the same staging, a lane then takes eight consecutive channels
-        // of a row and stores them as one 16-byte vector of halves
-        constexpr int LPR = WTN / 8;
-        constexpr int RPI = 64 / LPR;
-        const int cv = lane % LPR;
-        const int rsub = lane / LPR;
-        const int col = n0 + wave_n * WTN + cv * 8;
+    return;
+  }
+  if constexpr (sizeof(T) == 2) {
+    if ((g.o & 7) == 0 && y2 == nullptr) {
+      // fp16 output: the same staging, a lane then takes eight consecutive channels
+      // of a row and stores them as one 16-byte vector of halves
+      constexpr int LPR = CW / 8;
+      constexpr int RPI = 64 / LPR;
+      const int cv = lane % LPR;
+      const int rsub = lane / LPR;
+#pragma unroll
+      for (int j0 = 0; j0 < TN; j0 += JC) {
+        const int col = n0 + wave_n * WTN + j0 * 32 + cv * 8;
         float bias8[8];
 #pragma unroll
         for (int q = 0; q < 8; ++q) bias8[q] = 0.f;
@@ -383,10 +392,10 @@ __device__ __forceinline__ void igemm_tile(
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
 #pragma unroll
-          for (int j = 0; j < TN; ++j)
+          for (int j = 0; j < JC; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r)
-              smw[((r >> 2) * 8 + lh * 4 + (r & 3)) * SROW + j * 32 + l32] = acc[i][j][r];
+              smw[((r >> 2) * 8 + lh * 4 + (r & 3)) * SROW + j * 32 + l32] = acc[i][j0 + j][r];
 #pragma unroll
           for (int it = 0; it < 32 / RPI; ++it) {
             const int row = it * RPI + rsub;
@@ -405,8 +414,8 @@ __device__ __forceinline__ void igemm_tile(
             }
           }
         }
-        return;
       }
+      return;
     }
   }
 #pragma unroll
@@ -458,6 +467,19 @@ __global__ __launch_bounds__(256) void conv_igemm_kernel(IgemmProblem p) {
                                           static_cast<T*>(p.y), static_cast<T*>(p.y2), p.o1, p.ep,
                                           p.tiles_n, p.tiles, p.partial, p.slabs_per_split, p.splits,
                                           (int)blockIdx.x);
+}
+
+// The fp16 128x256 tile: 128 accumulator registers per lane, so the remaining registers
+// are capped to keep two waves per SIMD (one workgroup's barrier and LDS waits are then
+// covered by the other's MFMAs).
+template <bool PW>
+__global__ __launch_bounds__(256, 2) void conv_igemm_wide_f16_kernel(IgemmProblem p) {
+  __shared__ __attribute__((aligned(16))) unsigned char lds[igemm_lds_bytes<128, 256, 64>()];
+  igemm_tile<__half, 128, 256, 2, 2, 64, PW>(lds, p.g, static_cast<const __half*>(p.x),
+                                             static_cast<const __half*>(p.w), p.bias,
+                                             static_cast<__half*>(p.y), static_cast<__half*>(p.y2), p.o1,
+                                             p.ep, p.tiles_n, p.tiles, p.partial, p.slabs_per_split,
+                                             p.splits, (int)blockIdx.x);
 }
 
 // Several independent convolutions in one grid: blocks [first[i], first[i+1]) work
@@ -849,10 +871,12 @@ __global__ __launch_bounds__(256) void splitk_reduce_group_kernel(ReduceGroup gr
 // Tile configurations (BM, BN, waves along M, waves along N).
 enum TileCfg {
   CFG_128x128 = 0, CFG_128x64 = 1, CFG_64x64 = 2, CFG_128x32 = 3, CFG_WAVE32 = 4, CFG_WAVE16 = 5,
-  CFG_128x96 = 6, CFG_128x160 = 7  // all output channels of a narrow, long-K problem in one tile
+  CFG_128x96 = 6, CFG_128x160 = 7,  // all output channels of a narrow, long-K problem in one tile
+  CFG_128x256 = 8                    // fp16 storage: 64x128 per wave, 64-byte K slabs
 };
-constexpr int kCfgBM[] = {128, 128, 64, 128, 32, 16, 128, 128};
-constexpr int kCfgBN[] = {128, 64, 64, 32, 32, 16, 96, 160};
+constexpr int kCfgBM[] = {128, 128, 64, 128, 32, 16, 128, 128, 128};
+constexpr int kCfgBN[] = {128, 64, 64, 32, 32, 16, 96, 160, 256};
+constexpr int kRowBytesF16Wide = 64;  // K bytes per tile row per slab of CFG_128x256
 
 struct IgemmPlan {
   int cfg;
@@ -897,6 +921,18 @@ IgemmPlan plan_igemm(const OgleConvArgs& a, long m, bool allow_split) {
                            ((a.out_c > 64 && a.out_c <= 96) || (a.out_c > 128 && a.out_c <= 160));
   if (narrow_long) {
     p.cfg = a.out_c <= 96 ? CFG_128x96 : CFG_128x160;
+  } else if (a.dtype == OGLE_F16 && a.out_c >= 256 && tiles(CFG_128x256) >= 2 * kComputeUnits) {
+    // fp16 storage: one MFMA does sixteen times the work per operand byte, and a wave that
+    // owns 64x64 outputs reads its operands from LDS as fast as the MFMA pipe consumes them.
+    // A wave with 64x128 outputs reads a third less per MFMA and the tile pulls a quarter
+    // less from L2; 64-byte slabs keep two such workgroups per compute unit.  Measured on
+    // MI355X: M = 46208, K = N = 1024 gains 8 % (610 -> 662 TFLOP/s), but with fewer than two
+    // tiles per compute unit (M = 11552, N = 1024: 364 tiles) the second round is mostly
+    // empty and the 128x128 tile stays ahead (480 against 448 TFLOP/s).
+    p.cfg = CFG_128x256;
+    const int epr2 = kRowBytesF16Wide / esz;
+    p.cchunks = (a.in_c + epr2 - 1) / epr2;
+    p.ktiles = a.kernel_size * a.kernel_size * p.cchunks;
   } else if (a.out_c <= 32) {
     p.cfg = CFG_128x32;
   } else if (a.out_c > 64 && tiles(CFG_128x128) >= big_tiles_wanted) {
@@ -1118,6 +1154,16 @@ Prepared prepare(const OgleConvArgs& a, long m, const IgemmPlan& p) {
       break;                                                                                 \
   }
 
+// One problem, one grid of the LDS-tiled kernel.
+void launch_single(int dtype, int cfg, bool pw, unsigned grid, hipStream_t s, const IgemmProblem& prob) {
+  if (cfg == CFG_128x256) {  // fp16 storage only (plan_igemm)
+    if (pw) launch(conv_igemm_wide_f16_kernel<true>, dim3(grid), dim3(256), 0, s, prob);
+    else launch(conv_igemm_wide_f16_kernel<false>, dim3(grid), dim3(256), 0, s, prob);
+    return;
+  }
+  OGLE_IGEMM_DISPATCH(conv_igemm_kernel, dtype, cfg, pw, grid, s, prob);
+}
+
 void launch_wave(int dtype, bool pw, int cfg, const Prepared& pr, hipStream_t s) {
   const dim3 grid(pr.grid), block(256);
 #define OGLE_WAVE_LAUNCH(T, PW, TS) \
@@ -1166,7 +1212,7 @@ int32_t launch_conv_igemm(const OgleConvArgs& a, hipStream_t s) {
     launch_wave(a.dtype, pw, p.cfg, pr, s);
     return check_launch("conv_igemm_wave");
   }
-  OGLE_IGEMM_DISPATCH(conv_igemm_kernel, a.dtype, p.cfg, pw, pr.grid, s, pr.prob);
+  launch_single(a.dtype, p.cfg, pw, pr.grid, s, pr.prob);
   int32_t st = check_launch("conv_igemm");
   if (st != OGLE_OK || p.splits == 1) return st;
   if (a.dtype == OGLE_F16) launch_reduce_single<__half>(pr, s);
@@ -1214,7 +1260,8 @@ int32_t launch_conv_batch(const OgleConvArgs* args, int count, hipStream_t s,
     for (size_t b0 = a0; b0 < items.size() && grp.count < kMaxGroup; ++b0) {
       const Item& it = items[b0];
       if (done[b0] || it.dtype != head.dtype) continue;
-      const bool same = it.cfg == head.cfg && it.pw == head.pw;
+      const bool same = it.cfg == head.cfg && it.pw == head.pw && it.cfg != CFG_128x256;
+      if (b0 != a0 && (it.cfg == CFG_128x256 || head.cfg == CFG_128x256)) continue;  // fills the chip alone
       if (!same && !(mixable(head) && mixable(it))) continue;
       uniform = uniform && same;
       done[b0] = true;
@@ -1230,7 +1277,7 @@ int32_t launch_conv_batch(const OgleConvArgs* args, int count, hipStream_t s,
     if (grp.count == 1 && is_wave(head.cfg)) {
       launch_wave(head.dtype, head.pw, head.cfg, head.pr, s);
     } else if (grp.count == 1) {
-      OGLE_IGEMM_DISPATCH(conv_igemm_kernel, head.dtype, head.cfg, head.pw, grid, s, grp.p[0]);
+      launch_single(head.dtype, head.cfg, head.pw, grid, s, grp.p[0]);
     } else if (uniform && !is_wave(head.cfg)) {
       OGLE_IGEMM_DISPATCH(conv_igemm_group_kernel, head.dtype, head.cfg, head.pw, grid, s, grp);
     } else if (head.dtype == OGLE_F16) {

@@ -761,3 +761,162 @@ def test_kernels_against_committed_vectors():
         final = gpu_topk_nms(np.array([n], np.int32), ora["prior"][None], ora["cls"][None],
                              ora["score"][None], ora["rect"][None], 5, 0.45)
         np.testing.assert_array_equal(final[0]["prior"], ora["prior"][g["info%d_keep" % i]])
+
+
+def test_fp16_wide_tile_large_pointwise():
+    """fp16 storage with at least 512 tiles of 128x256 outputs takes the wide-tile kernel
+    (64x128 outputs per wave, 64-byte K slabs); ragged M, and K with a half-filled last slab."""
+    import torch
+    r = rng(2700)
+    n, h, w, c, o = 17, 32, 31, 72, 1024          # M = 16864 (not a multiple of 128), K = 72
+    x = r.uniform(0, 2, (n, h, w, c)).astype(np.float16).astype(np.float32)
+    wt = r.normal(0, np.sqrt(2 / c), (o, c, 1, 1)).astype(np.float16).astype(np.float32)
+    b = r.uniform(-0.1, 0.1, o).astype(np.float32)
+    got = gpu_conv(x, wt, b, act=H.ACT_RELU, variant=H.VARIANT_PW, dtype=H.F16)
+    a64 = x.reshape(-1, c).astype(np.float64)
+    w64 = wt.reshape(o, c).astype(np.float64)
+    ref = np.maximum(a64 @ w64.T + b, 0).astype(np.float32)
+    scale = np.abs(a64) @ np.abs(w64).T + np.abs(b)
+    half_ulp = 0.5 * 2.0 ** (np.floor(np.log2(np.maximum(np.abs(ref.astype(np.float64)), 2.0 ** -14))) - 10)
+    assert_conv_close(got.reshape(-1, o), ref, (scale + half_ulp / FP16_RTOL).astype(np.float32), FP16_RTOL,
+                      "fp16 wide tile")
+
+
+SPLIT_CASES = [
+    # n, h, w, c, o1, o2, k, s, p, dtype       (output channels [0,o1) -> y, [o1,o1+o2) -> y2)
+    (4, 19, 19, 128, 12, 63, 3, 1, 1, H.F32),      # SSD box + class head, 128x96 tile, element stores
+    (2, 10, 10, 256, 24, 126, 3, 1, 1, H.F32),     # 128x160 tile
+    (3, 9, 9, 64, 32, 64, 3, 1, 1, H.F32),         # both parts multiples of 4: 16-byte stores
+    (2, 7, 7, 96, 40, 24, 1, 1, 0, H.F32),         # pointwise, 64x64 tiles
+    (1, 3, 3, 128, 24, 126, 3, 1, 1, H.F32),       # tiny map: the wave-split kernel
+    (1, 1, 1, 128, 24, 126, 3, 1, 1, H.F32),       # one pixel
+    (2, 9, 9, 64, 16, 48, 3, 1, 1, H.F16),         # fp16 storage
+]
+
+
+@pytest.mark.parametrize("case", SPLIT_CASES)
+@pytest.mark.parametrize("workspace", [True, False])
+def test_conv_two_destinations(case, workspace):
+    """OgleConvArgs.output2_dev: one contraction over the concatenated filters writes each
+    part's channels to its own dense tensor; equal to the oracle run on each filter."""
+    import ctypes
+    import torch
+    from util import dev, pack_filter, stream_ptr
+    n, h, w, c, o1, o2, k, s, p, dtype = case
+    r = rng(2800 + SPLIT_CASES.index(case))
+    x = r.uniform(-1, 1, (n, h, w, c)).astype(np.float32)
+    wt = r.normal(0, 0.2, (o1 + o2, c, k, k)).astype(np.float32)
+    b = r.uniform(-0.1, 0.1, o1 + o2).astype(np.float32)
+    tdt = torch.float32
+    if dtype == H.F16:
+        x, wt = x.astype(np.float16).astype(np.float32), wt.astype(np.float16).astype(np.float32)
+        tdt = torch.float16
+    xd, bd, wd = dev(x, tdt), dev(b), pack_filter(wt, H.FILTER_OHWI, dtype)
+    oh, ow = H.out_size(h, k, s, p), H.out_size(w, k, s, p)
+    y1 = torch.full((n, oh, ow, o1), float("nan"), dtype=tdt, device="cuda")
+    y2 = torch.full((n, oh, ow, o2), float("nan"), dtype=tdt, device="cuda")
+    a = H.conv_args(xd.data_ptr(), wd.data_ptr(), bd.data_ptr(), y1.data_ptr(), n, h, w, c, o1 + o2, k, s, p,
+                    act=H.ACT_RELU, dtype=dtype)
+    a.output2_dev, a.out_c_split = y2.data_ptr(), o1
+    ws = None
+    if workspace:
+        need = H.lib().ogle_hip_conv_workspace_bytes(ctypes.byref(a))
+        if need:
+            ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+            a.workspace_dev, a.workspace_bytes = ws.data_ptr(), need
+    H.check(H.lib().ogle_hip_conv2d(ctypes.byref(a), stream_ptr()))
+    torch.cuda.synchronize()
+    rtol = FP16_RTOL if dtype == H.F16 else FP32_RTOL
+    for part, (lo, hi, y) in enumerate(((0, o1, y1), (o1, o1 + o2, y2))):
+        ref = O.conv2d(x, wt[lo:hi], b[lo:hi], s, p, 1, 1, O.ACT_RELU)
+        scale = O.conv2d_abs(x, wt[lo:hi], b[lo:hi], s, p, 1, 1)
+        if dtype == H.F16:
+            scale = scale + 2.0 ** -11 * np.abs(ref) / FP16_RTOL + 1e-3
+        assert_conv_close(y.float().cpu().numpy(), ref, scale, rtol, "two destinations part %d %s" % (part, case))
+
+
+def test_conv_two_destinations_errors():
+    import ctypes
+    import torch
+    from util import stream_ptr
+    x = torch.zeros((1, 4, 4, 6), device="cuda")      # C % 4 != 0: no MFMA path
+    w = torch.zeros((8 * 6 * 9,), device="cuda")
+    y1, y2 = torch.zeros((1, 4, 4, 3), device="cuda"), torch.zeros((1, 4, 4, 5), device="cuda")
+    a = H.conv_args(x.data_ptr(), w.data_ptr(), None, y1.data_ptr(), 1, 4, 4, 6, 8, 3, 1, 1)
+    a.output2_dev, a.out_c_split = y2.data_ptr(), 3
+    assert H.lib().ogle_hip_conv2d(ctypes.byref(a), stream_ptr()) == H.ERR_UNSUPPORTED
+    assert "MFMA" in H.last_error()
+    for bad in (0, 8, -1):
+        a.out_c_split = bad
+        assert H.lib().ogle_hip_conv2d(ctypes.byref(a), stream_ptr()) == H.ERR_INVALID_ARG
+    torch.cuda.synchronize()
+
+
+def test_conv_batch_begin_finish_equals_batch():
+    """ogle_hip_conv2d_batch_begin + _finish: the same outputs as ogle_hip_conv2d_batch, bit for
+    bit, with the reductions of every split-K plan launched once at the end."""
+    import ctypes
+    import torch
+    from util import pack_filter
+    r = rng(2900)
+    cases = [(4, 19, 19, 128, 12, 3, 1, 1), (4, 10, 10, 256, 126, 3, 1, 1), (2, 7, 7, 64, 96, 1, 1, 0),
+             (1, 5, 5, 512, 24, 3, 1, 1), (16, 19, 19, 64, 64, 1, 1, 0)]
+    args1, args2 = (H.ConvArgs * len(cases))(), (H.ConvArgs * len(cases))()
+    keep, outs = [], []
+    for i, (n, h, w, c, o, k, st, p) in enumerate(cases):
+        x = torch.from_numpy(r.uniform(-1, 1, (n, h, w, c)).astype(np.float32)).cuda()
+        wd = pack_filter(r.normal(0, 0.2, (o, c, k, k)).astype(np.float32), H.FILTER_OHWI)
+        b = torch.from_numpy(r.uniform(-.1, .1, o).astype(np.float32)).cuda()
+        oh, ow = H.out_size(h, k, st, p), H.out_size(w, k, st, p)
+        ya = torch.full((n, oh, ow, o), float("nan"), device="cuda")
+        yb = torch.full((n, oh, ow, o), float("nan"), device="cuda")
+        a = H.conv_args(x.data_ptr(), wd.data_ptr(), b.data_ptr(), ya.data_ptr(), n, h, w, c, o, k, st, p,
+                        1, 1, H.ACT_RELU)
+        need = H.lib().ogle_hip_conv_workspace_bytes(ctypes.byref(a))
+        wsa = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
+        wsb = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
+        if need:
+            a.workspace_dev, a.workspace_bytes = wsa.data_ptr(), need
+        args1[i] = a
+        a.output_dev = yb.data_ptr()
+        if need:
+            a.workspace_dev = wsb.data_ptr()
+        args2[i] = a
+        keep += [x, wd, b, wsa, wsb]
+        outs.append((ya, yb))
+    H.check(H.lib().ogle_hip_conv2d_batch(args1, len(cases), 0))
+    open_ = (ctypes.c_int32 * len(cases))()
+    before = H.lib().ogle_hip_launch_count()
+    H.check(H.lib().ogle_hip_conv2d_batch_begin(args2, len(cases), open_, 0))
+    assert sum(open_) >= 2                       # the long-K heads leave partial sums
+    torch.cuda.synchronize()
+    for (ya, yb), pending in zip(outs, open_):
+        if not pending:
+            assert torch.equal(ya, yb)
+    mid = H.lib().ogle_hip_launch_count()
+    H.check(H.lib().ogle_hip_conv2d_batch_finish(args2, len(cases), 0))
+    assert H.lib().ogle_hip_launch_count() - mid == 1     # one grid for every open reduction
+    assert mid > before
+    torch.cuda.synchronize()
+    for ya, yb in outs:
+        assert torch.equal(ya, yb)
+
+
+def test_kernel_timing_events():
+    """ogle_hip_kernel_timing_begin / _end: one device-stamped duration per launched kernel."""
+    import ctypes
+    import torch
+    x = torch.rand(4, 64, 64, 64, device="cuda")
+    y = torch.empty_like(x)
+    ua = H.UnaryArgs(x.data_ptr(), y.data_ptr(), x.numel(), H.UNARY_CLIP, 0.0, 0.5, H.F32)
+    torch.cuda.synchronize()
+    assert H.lib().ogle_hip_kernel_timing_begin() == 0
+    c0 = H.lib().ogle_hip_launch_count()
+    for _ in range(5):
+        H.check(H.lib().ogle_hip_unary(ctypes.byref(ua), 0))
+    buf = (ctypes.c_float * 8)()
+    n = H.lib().ogle_hip_kernel_timing_end(buf, 8)
+    assert n == 5 == H.lib().ogle_hip_launch_count() - c0
+    assert all(0.5 < buf[i] < 500.0 for i in range(5)), list(buf)
+    assert H.lib().ogle_hip_kernel_timing_end(buf, 8) == 0      # nothing recorded while off
+    assert torch.equal(y, x.clamp(0.0, 0.5))
