@@ -58,7 +58,7 @@ def family_of(nodes, layers):
     return " + ".join(sorted(fams))
 
 
-def per_family_roofline(sess, info, batch, passes):
+def per_family_roofline(sess, info, batch, passes, pass_us):
     """Kernel time per family from the kernels' own durations: every kernel of `passes` eager
     passes carries a start / stop HIP event pair that the device stamps with the kernel's begin
     and end (ogle_hip_kernel_timing_begin), the same quantity a rocprofv3 kernel trace reports,
@@ -85,17 +85,26 @@ def per_family_roofline(sess, info, batch, passes):
                             f["layers"] += 1
                             f["flops"] += layers[n]["flops_per_image"] * batch
                             f["bytes"] += layers[n]["act_bytes_per_image"] * batch + layers[n]["weight_bytes"]
+    # A kernel trace of the replayed pass takes a kernel's begin when its dispatch packet is picked
+    # up, i.e. at the previous kernel's end: its durations add up to the pass.  The events here
+    # bracket the kernel alone, so the pass's dispatch gaps (replayed pass - sum of kernel
+    # durations, shared equally among its dispatches) are added back before rates are formed.
+    kernel_sum = sum(f["us"] for f in fams.values())
+    gap_us = max(pass_us - kernel_sum, 0.0) / max(dispatches, 1)
     out = []
     for name, f in fams.items():
         bound = "mfma" if "MFMA implicit GEMM" in name else "hbm"
-        tflops, gbs = f["flops"] / f["us"] / 1e6, f["bytes"] / f["us"] / 1e3
-        out.append(dict(kernel=name, layers=f["layers"], launches=f["launches"], ms_per_step=round(f["us"] / 1e3, 4),
-                        avg_launch_us=round(f["us"] / max(f["launches"], 1), 2), bound=bound,
+        f["span_us"] = f["us"] + gap_us * f["launches"]
+        tflops, gbs = f["flops"] / f["span_us"] / 1e6, f["bytes"] / f["span_us"] / 1e3
+        out.append(dict(kernel=name, layers=f["layers"], launches=f["launches"],
+                        ms_per_step=round(f["span_us"] / 1e3, 4),
+                        avg_launch_us=round(f["span_us"] / max(f["launches"], 1), 2),
+                        avg_kernel_only_us=round(f["us"] / max(f["launches"], 1), 2), bound=bound,
                         tflops=round(tflops, 2), gbs=round(gbs, 1),
                         frac=round(gbs / HBM_PEAK_GBS if bound == "hbm" else tflops / MFMA_F32_PEAK_TFLOPS, 4),
                         flops_per_step=f["flops"], bytes_per_step=f["bytes"]))
     out.sort(key=lambda d: -d["ms_per_step"])
-    return out, sum(f["us"] for f in fams.values()) / 1e3, dispatches
+    return out, kernel_sum / 1e3, dispatches, gap_us
 
 
 def calibration_copy(megabytes=256, launches=3):
@@ -114,13 +123,21 @@ def calibration_copy(megabytes=256, launches=3):
     return n * 4
 
 
+# bench family -> family name in the summaries ogle_amd.profile_layers writes
+PROFILE_FAMILY = {"pointwise 1x1 backbone (MFMA implicit GEMM)": "pointwise",
+                  "SSD heads + extras chain (dense 3x3 and 1x1, MFMA implicit GEMM)": "heads+extras",
+                  "depthwise 3x3": "depthwise", "dense 3x3 stem (direct MFMA)": "stem"}
+
+
 def read_traffic_summary(kernel_family):
     """HBM bytes per launch of the dominant kernel from the committed counter summary
-    (profiles/bench_b16_pmc_traffic.txt, made from two rocprofv3 --pmc runs of this script)."""
-    path = os.path.join(ROOT, "profiles", "bench_b16_pmc_traffic.txt")
+    (profiles/bench_b16_per_layer_traffic.txt, made by ogle_amd.profile_layers from two
+    rocprofv3 --pmc runs of `bench.py --profile-layers ... --eager`)."""
+    path = os.path.join(ROOT, "profiles", "bench_b16_per_layer_traffic.txt")
+    key = "traffic_bytes_per_launch[%s]=" % PROFILE_FAMILY.get(kernel_family, kernel_family)
     try:
         for line in open(path):
-            if line.startswith("traffic_bytes_per_launch[%s]=" % kernel_family):
+            if line.startswith(key):
                 return float(line.split("=", 1)[1])
     except OSError:
         pass
@@ -338,15 +355,17 @@ def profile_layers_run(args):
     import torch
     sess, info = build_session(args.batch)
     plan = sess.launch_plan(with_detect=True)
-    sess.time_compute(args.warmup, args.steps, graph=True, with_detect=True)
+    copy_bytes = calibration_copy()
+    sess.time_compute(args.warmup, args.steps, graph=not args.eager, with_detect=True)
     sess.sync()
     torch.cuda.synchronize()
-    me = "python3 bench.py --profile-layers %s --steps %d --warmup %d --batch %d" % (
-        args.profile_layers, args.steps, args.warmup, args.batch)
-    doc = dict(workload="MobileNet-v1-SSD 300x300 fp32, batch %d, one session, hipGraph replay, "
-                        "network + decode/score filter + top-k/NMS" % args.batch,
+    me = "python3 bench.py --profile-layers %s --steps %d --warmup %d --batch %d%s" % (
+        args.profile_layers, args.steps, args.warmup, args.batch, " --eager" if args.eager else "")
+    doc = dict(workload="MobileNet-v1-SSD 300x300 fp32, batch %d, one session, %s, "
+                        "network + decode/score filter + top-k/NMS"
+                        % (args.batch, "kernel-by-kernel launches" if args.eager else "hipGraph replay"),
                batch=args.batch, replays=args.steps, dispatches_per_pass=sum(k for _, k in plan),
-               plan=plan,
+               plan=plan, calibration=dict(kernel="convert_kernel<float, float>", kib_per_launch=copy_bytes // 1024),
                layers={l["name"]: dict(kind=l["kind"], flops_per_image=l["flops_per_image"],
                                        act_bytes_per_image=l["act_bytes_per_image"],
                                        weight_bytes=l["weight_bytes"]) for l in info["layers"]},
@@ -354,7 +373,15 @@ def profile_layers_run(args):
                          "rocprofv3 --kernel-trace --output-format csv -d gpurun_out/layers -o b%d -- %s"
                          % (args.batch, me),
                          "python3 -m ogle_amd.profile_layers gpurun_out/layers/b%d_kernel_trace.csv %s"
-                         % (args.batch, args.profile_layers)])
+                         % (args.batch, args.profile_layers)] if not args.eager else
+               ["cd /tmp && export TMPDIR=/tmp && cd $GRAFT_REPO_ROOT",
+                "rocprofv3 --pmc FETCH_SIZE --output-format csv -d gpurun_out/layers -o fetch%d -- %s"
+                % (args.batch, me),
+                "rocprofv3 --pmc WRITE_SIZE --output-format csv -d gpurun_out/layers -o write%d -- %s"
+                % (args.batch, me),
+                "python3 -m ogle_amd.profile_layers --fetch gpurun_out/layers/fetch%d_counter_collection.csv "
+                "--write gpurun_out/layers/write%d_counter_collection.csv %s"
+                % (args.batch, args.batch, args.profile_layers)])
     with open(args.profile_layers, "w") as f:
         json.dump(doc, f)
     print(json.dumps(dict(profile_layers=args.profile_layers, dispatches_per_pass=doc["dispatches_per_pass"],
@@ -482,7 +509,8 @@ def main():
         for pb in pinned:
             pb.close()
 
-    fams, kernel_sum_ms, dispatches = per_family_roofline(sess, info, args.batch, passes=10)
+    fams, kernel_sum_ms, dispatches, gap_us = per_family_roofline(
+        sess, info, args.batch, passes=10, pass_us=single["event_ms_per_step"] * 1e3)
     dom = fams[0]
     roofline = dict(bound=dom["bound"], kernel=dom["kernel"],
                     achieved=dom["gbs"] if dom["bound"] == "hbm" else dom["tflops"],
@@ -490,8 +518,14 @@ def main():
                     unit="GB/s" if dom["bound"] == "hbm" else "TFLOP/s", frac=dom["frac"],
                     traffic=read_traffic_summary(dom["kernel"]), launches_per_step=dom["launches"],
                     avg_launch_us=dom["avg_launch_us"],
-                    measured="start / stop HIP events carried by every kernel of 10 eager passes (stamped "
-                             "by the device with the kernel's own begin and end), summed over the family",
+                    avg_kernel_only_us=dom["avg_kernel_only_us"],
+                    dispatch_gap_us=round(gap_us, 3),
+                    measured="avg_kernel_only_us: start / stop HIP events carried by every kernel of 10 eager "
+                             "passes, stamped by the device with the kernel's own begin and end, summed over "
+                             "the family; avg_launch_us (what frac uses) adds the replayed pass's mean dispatch "
+                             "gap (single-stream pass time - sum of kernel durations) / dispatches, because a "
+                             "rocprofv3 kernel trace of the replayed pass counts a kernel from the previous "
+                             "kernel's end",
                     algorithmic_per_step=dom["flops_per_step"] if dom["bound"] == "mfma" else dom["bytes_per_step"])
 
     # batch-1 latency: each pass waits for the previous one

@@ -1,6 +1,12 @@
 """Per-layer summary of a rocprofv3 kernel trace of replayed passes.
 
     python -m ogle_amd.profile_layers KERNEL_TRACE.csv PLAN.json [-o SUMMARY.txt]
+    python -m ogle_amd.profile_layers --fetch FETCH.csv --write WRITE.csv PLAN.json [-o SUMMARY.txt]
+
+The second form reads the counter_collection CSVs of two `rocprofv3 --pmc` runs of the same
+command (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch) instead of a kernel trace and gives HBM
+bytes per launch next to the algorithmic bytes.  Each counter is scaled by what it reads for the
+plain copy of known size that `bench.py --profile-layers` launches before the replays.
 
 PLAN.json is what `bench.py --profile-layers PLAN.json` writes: the dispatch sequence of one
 pass (Session.launch_plan: which node(s) every call into the kernel library was made for and
@@ -98,6 +104,93 @@ def summarize(trace_path, plan):
     return out, fam, pos, sum(spans) / reps
 
 
+def _dispatch_rows(path, counter):
+    csv.field_size_limit(1 << 30)
+    rows = [r for r in csv.DictReader(open(path)) if r["Counter_Name"] == counter]
+    rows.sort(key=lambda r: int(r["Dispatch_Id"]))
+    return rows
+
+
+def _scaled_tail(path, counter, plan):
+    """Per position of the pass: (kernel, bytes per launch) from one counter run, averaged over the
+    replays and scaled by the calibration copy's reading."""
+    rows = _dispatch_rows(path, counter)
+    cal = plan["calibration"]
+    seen = [float(r["Counter_Value"]) for r in rows if cal["kernel"] in r["Kernel_Name"]]
+    if not seen:
+        raise SystemExit("%s: no dispatch of the calibration kernel %s" % (path, cal["kernel"]))
+    scale = cal["kib_per_launch"] / (sum(seen) / len(seen))
+    n, reps = plan["dispatches_per_pass"], plan["replays"]
+    if len(rows) < n * reps:
+        raise SystemExit("%s holds %d dispatches, fewer than %d replays x %d" % (path, len(rows), reps, n))
+    tail = rows[-n * reps:]
+    pos = []
+    for j in range(n):
+        names = {short_kernel(tail[r * n + j]["Kernel_Name"]) for r in range(reps)}
+        if len(names) != 1:
+            raise SystemExit("position %d of the pass is not the same kernel in every replay: %s" % (j, names))
+        kib = sum(float(tail[r * n + j]["Counter_Value"]) for r in range(reps)) / reps
+        pos.append((names.pop(), kib * scale * 1024.0))
+    return pos, scale, sum(seen) / len(seen)
+
+
+def render_traffic(fetch_path, write_path, plan):
+    fetch, fscale, fraw = _scaled_tail(fetch_path, "FETCH_SIZE", plan)
+    write, wscale, wraw = _scaled_tail(write_path, "WRITE_SIZE", plan)
+    layers, batch = plan["layers"], plan["batch"]
+    lines = []
+    w = lines.append
+    w("# HBM traffic per launch of the pass (rocprofv3 counters): %s" % plan["workload"])
+    w("")
+    w("commands (run from the repository root on one MI355X, one counter per run):")
+    for c in plan["commands"]:
+        w("    " + c)
+    w("")
+    cal = plan["calibration"]
+    w("Counters are KiB per dispatch.  Before the passes the script launches a plain copy of %d KiB"
+      % cal["kib_per_launch"])
+    w("(%s: reads and writes that much), which calibrates them:" % cal["kernel"])
+    w("    FETCH_SIZE read %.1f KiB for the copy -> scale %.4f" % (fraw, fscale))
+    w("    WRITE_SIZE read %.1f KiB for the copy -> scale %.4f" % (wraw, wscale))
+    w("Values below are scaled and averaged over %d passes; algorithmic = input + weights + bias + output"
+      % plan["replays"])
+    w("once each (0 for reductions, concat and the detector tail, whose bytes are all overhead here).")
+    w("")
+    w("%-44s %-46s %10s %10s %10s %7s" % ("node(s)", "kernel", "fetch MB", "write MB", "algo MB", "ratio"))
+    fam, at = {}, 0
+    for label, k in plan["plan"]:
+        is_reduce = label.startswith("reduce:")
+        nodes = [m[0] for m in re.findall(r"([^#+\[\]:]+)#([A-Za-z0-9_]+)#", label)]
+        algo = 0 if is_reduce else sum(layers[x]["act_bytes_per_image"] * batch + layers[x]["weight_bytes"]
+                                       for x in nodes if x in layers)
+        f = family_of(nodes, layers)
+        name = ("reduce:" if is_reduce else "") + "+".join(nodes)
+        if len(name) > 43:
+            name = name[:40] + "..."
+        fb = sum(b for _, b in fetch[at:at + k])
+        wb = sum(b for _, b in write[at:at + k])
+        for i in range(k):
+            w("%-44s %-46s %10.2f %10.2f %10s %7s" % (
+                name if i == 0 else "  (same call)", fetch[at + i][0][:46], fetch[at + i][1] / 1e6,
+                write[at + i][1] / 1e6, ("%.2f" % (algo / 1e6)) if i == 0 else "",
+                ("%.2f" % ((fb + wb) / algo)) if i == 0 and algo else ""))
+        at += k
+        a = fam.setdefault(f, dict(traffic=0.0, algo=0.0, launches=0))
+        a["traffic"] += fb + wb
+        a["algo"] += algo
+        a["launches"] += k
+    w("")
+    w("per family (traffic of the family's launches incl. its split-K reductions; per launch = / launches):")
+    w("%-28s %9s %12s %12s %7s" % ("family", "launches", "traffic MB", "algo MB", "ratio"))
+    for f, a in sorted(fam.items(), key=lambda kv: -kv[1]["traffic"]):
+        w("%-28s %9d %12.2f %12.2f %7s" % (f, a["launches"], a["traffic"] / 1e6, a["algo"] / 1e6,
+                                            ("%.2f" % (a["traffic"] / a["algo"])) if a["algo"] else ""))
+    w("")
+    for f, a in sorted(fam.items()):
+        w("traffic_bytes_per_launch[%s]=%d" % (f, round(a["traffic"] / a["launches"])))
+    return "\n".join(lines) + "\n"
+
+
 def render(out, fam, pos, span, plan):
     lines = []
     w = lines.append
@@ -148,13 +241,22 @@ def render(out, fam, pos, span, plan):
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("trace")
+    ap.add_argument("trace", nargs="?")
     ap.add_argument("plan")
+    ap.add_argument("--fetch", help="counter_collection CSV of a --pmc FETCH_SIZE run")
+    ap.add_argument("--write", help="counter_collection CSV of a --pmc WRITE_SIZE run")
     ap.add_argument("-o", "--out")
     args = ap.parse_args()
     plan = json.load(open(args.plan))
-    out, fam, pos, span = summarize(args.trace, plan)
-    text = render(out, fam, pos, span, plan)
+    if args.fetch or args.write:
+        if not (args.fetch and args.write) or args.trace:
+            ap.error("give --fetch and --write together, without a kernel trace")
+        text = render_traffic(args.fetch, args.write, plan)
+    else:
+        if not args.trace:
+            ap.error("a kernel trace or --fetch/--write is needed")
+        out, fam, pos, span = summarize(args.trace, plan)
+        text = render(out, fam, pos, span, plan)
     if args.out:
         with open(args.out, "w") as f:
             f.write(text)
