@@ -120,8 +120,21 @@ __device__ __forceinline__ void igemm_tile(
   // tiles sharing a band of A rows run on one XCD and, when K is split, an XCD owns
   // a fixed subset of the K ranges: the filter and input slabs of one K range are
   // then fetched into one L2 only instead of all eight.
+  // When K is split and the input is the larger operand (a 3x3 head on a big map), the
+  // other layout is used instead (splits < 0 marks it): tile rows are dealt to the XCDs and
+  // all K ranges of a tile row run on the same XCD, so each band of input rows (with the
+  // halo its taps share) is fetched into one L2 only, and the filter into all eight.
   int pid, split;
-  {
+  if (splits < 0) {
+    splits = -splits;
+    const int xcd = bid & 7, j = bid >> 3;
+    const int per_row = tiles_n * splits;
+    const int r = (j / per_row) * 8 + xcd;
+    const int rem = j % per_row;
+    pid = r * tiles_n + rem / splits;
+    split = rem % splits;
+    if (pid >= tiles) return;
+  } else {
     const int xcd = bid & 7, j = bid >> 3;
     if (splits == 1) {
       // tile row r (the tiles_n tiles that share one band of A rows) goes to XCD
@@ -881,6 +894,7 @@ constexpr int kRowBytesF16Wide = 64;  // K bytes per tile row per slab of CFG_12
 struct IgemmPlan {
   int cfg;
   int splits;
+  bool rows_on_xcd;  // split-K work layout: tile rows, not K ranges, pinned to an XCD
   int slabs_per_split;
   int ktiles;
   int cchunks;
@@ -891,6 +905,7 @@ constexpr long kComputeUnits = 256;
 constexpr int kRowBytesF32 = 64;   // bytes of K per tile row per slab, fp32
 
 bool is_pointwise(const OgleConvArgs& a);
+bool is_wave(int cfg);
 
 // Picks the output tile and the K split.  Problems with few output
 // tiles but a long contraction (the SSD heads, the small feature maps) are split
@@ -1018,6 +1033,18 @@ IgemmPlan plan_igemm(const OgleConvArgs& a, long m, bool allow_split) {
   // partial sums are kept in rows of the channel count rounded up to four
   p.workspace_bytes =
       p.splits > 1 ? (size_t)p.splits * (size_t)m * ((a.out_c + 3) & ~3) * sizeof(float) : 0;
+  // Which operand an XCD's L2 should keep to itself: with K ranges pinned to XCDs the input is
+  // fetched by all eight L2s and the filter by one, with tile rows pinned it is the other way
+  // round (the rocprofv3 FETCH_SIZE of the 19x19x512 class head fell from 8.5x its input to
+  // about the input plus eight filters).
+  {
+    const long x_bytes = (long)a.n * a.in_h * a.in_w * a.in_c * esz;
+    const long w_bytes = (long)a.out_c * a.kernel_size * a.kernel_size * a.in_c * esz;
+    // whole tile rows per XCD: only when they spread evenly (within a tenth) over the eight
+    const long tiles_m = (m + kCfgBM[p.cfg] - 1) / kCfgBM[p.cfg];
+    const bool even = ((tiles_m + 7) / 8) * 8 * 10 <= tiles_m * 11;
+    p.rows_on_xcd = p.splits > 1 && !is_wave(p.cfg) && x_bytes > w_bytes && even;
+  }
   return p;
 }
 
@@ -1029,6 +1056,7 @@ int tile_bn(int cfg) { return kCfgBN[cfg]; }
 unsigned grid_blocks(const IgemmPlan& p, int tiles_m, int tiles_n) {
   const int tiles = tiles_m * tiles_n;
   if (p.splits == 1) return 8u * (unsigned)((tiles_m + 7) / 8) * (unsigned)tiles_n;
+  if (p.rows_on_xcd) return 8u * (unsigned)((tiles_m + 7) / 8) * (unsigned)tiles_n * (unsigned)p.splits;
   if (p.splits != 2 && p.splits != 4) return (unsigned)tiles * (unsigned)p.splits;
   const int xpz = 8 / p.splits;
   return 8u * (unsigned)((tiles + xpz - 1) / xpz);
@@ -1094,7 +1122,7 @@ Prepared prepare(const OgleConvArgs& a, long m, const IgemmPlan& p) {
   out.prob.tiles = tiles_m * tiles_n;
   out.prob.partial = p.splits > 1 ? static_cast<float*>(a.workspace_dev) : nullptr;
   out.prob.slabs_per_split = p.slabs_per_split;
-  out.prob.splits = p.splits;
+  out.prob.splits = p.rows_on_xcd ? -p.splits : p.splits;
   out.prob.variant = (p.cfg == CFG_WAVE32 ? 4 : p.cfg == CFG_WAVE16 ? 6 : p.cfg == CFG_128x32 ? 2 : 0) +
                      (is_pointwise(a) ? 1 : 0);
   if (is_wave(p.cfg)) {
@@ -1268,7 +1296,7 @@ int32_t launch_conv_batch(const OgleConvArgs* args, int count, hipStream_t s,
       const Prepared& pr = it.pr;
       grp.first[grp.count + 1] = grp.first[grp.count] + (int)pr.grid;
       grp.p[grp.count++] = pr.prob;
-      if (pr.prob.splits > 1) {
+      if (pr.prob.splits > 1 || pr.prob.splits < -1) {
         red.first[red.count + 1] = red.first[red.count] + (int)pr.reduce_grid;
         red.p[red.count++] = pr.red;
       }
