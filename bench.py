@@ -218,6 +218,17 @@ def kernel_table(iters=50, warm=5):
     conv_row("pointwise GEMM @C3 fp16 storage, fp32 accumulate", "ogle_hip_pwconv_gemm", "mfma",
              32, 19, 19, 512, 1024, 1, 1, 0, dtype=H.F16, peak=2500.0)
 
+    # yardstick for the two rows above: the vendor library's GEMM (torch.matmul -> hipBLASLt /
+    # rocBLAS) on the same shape and types; a comparison figure, not part of the path
+    for dt, tag in ((torch.float32, "fp32"), (torch.float16, "fp16")):
+        ga = torch.randn(11552, 512, device="cuda", dtype=dt)
+        gb = torch.randn(1024, 512, device="cuda", dtype=dt)
+        gc = torch.empty(11552, 1024, device="cuda", dtype=dt)
+        row("vendor library GEMM on the C3 shape, %s (yardstick)" % tag,
+            timed(lambda: torch.matmul(ga, gb.t(), out=gc)), 2.0 * 11552 * 512 * 1024,
+            ga.element_size() * (ga.numel() + gb.numel() + gc.numel()), "mfma",
+            MFMA_F32_PEAK_TFLOPS if dt == torch.float32 else 2500.0)
+
     # C4: the twelve SSD head convolutions of 64 images in one grouped call
     maps = [(19, 512, 3), (10, 1024, 6), (5, 512, 6), (3, 256, 6), (2, 256, 6), (1, 128, 6)]
     probs = []

@@ -164,10 +164,10 @@ int64_t ogle_rt_model_debug_string(const void* data, size_t size, char* out, int
 int32_t ogle_rt_num_kernels(OgleSession* s);
 
 /*
- * Issue order.  The reference runs nodes in file order (fbo_session.cc:140-153);
- * here a convolution whose result is not needed at once may be issued earlier, next
- * to another one, so that both share a grid.  ogle_rt_set_reorder(s, 0) before the
- * first run keeps strict file order.  ogle_rt_issue_order_name returns the name of
+ * Issue order.  The reference runs nodes in file order (fbo_session.cc:140-153), and so
+ * does a session here unless ogle_rt_set_reorder(s, 1) is called before the first run:
+ * then a convolution whose result is not needed at once may be issued earlier, next
+ * to another one, so that both share a grid (same results).  ogle_rt_issue_order_name returns the name of
  * the i-th node a pass issues (valid after the first run; NULL past the end).
  */
 int32_t ogle_rt_set_reorder(OgleSession* s, int32_t on);

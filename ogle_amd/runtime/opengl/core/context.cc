@@ -103,13 +103,18 @@ bool Context::Conflicts(const OgleConvArgs* pending, int n_pending, const MemRan
   return false;
 }
 
+// A convolution that needs a deferred one's result (or overwrites what it reads) only
+// forces out the deferred ones it conflicts with: it is deferred itself, and the others
+// may still share its grid.  Any other kind of launch goes to the stream at once and
+// takes everything deferred with it (BeforeLaunch).
 void Context::BeforeConv(const OgleConvArgs& args) {
   if (pending_.empty() && unreduced_.empty()) return;
   MemRange reads[3], writes[3];
   ConvRanges(args, reads, writes);
-  if (pending_.size() >= 16 ||
-      Conflicts(pending_.data(), static_cast<int>(pending_.size()), reads, 3, writes, 3))
+  if (pending_.size() >= 16)
     LaunchPending();
+  else
+    LaunchPendingThatConflict(reads, 3, writes, 3);
   FinishReductions(reads, 3, writes, 3, false);
 }
 
@@ -220,6 +225,25 @@ void Context::LaunchPending() {
   batch.swap(pending_);
   std::vector<std::string> labels;
   labels.swap(pending_labels_);
+  LaunchBatch(batch, labels);
+}
+
+void Context::LaunchPendingThatConflict(const MemRange* reads, int n_reads, const MemRange* writes,
+                                        int n_writes) {
+  std::vector<OgleConvArgs> batch, keep;
+  std::vector<std::string> labels, keep_labels;
+  for (size_t i = 0; i < pending_.size(); ++i) {
+    const bool hit = Conflicts(&pending_[i], 1, reads, n_reads, writes, n_writes);
+    (hit ? batch : keep).push_back(pending_[i]);
+    (hit ? labels : keep_labels).push_back(pending_labels_[i]);
+  }
+  if (batch.empty()) return;
+  pending_.swap(keep);
+  pending_labels_.swap(keep_labels);
+  LaunchBatch(batch, labels);
+}
+
+void Context::LaunchBatch(std::vector<OgleConvArgs>& batch, std::vector<std::string>& labels) {
   // launches the running node made itself before this point belong to that node
   if (!current_label_.empty()) LogLaunches(current_label_, node_count_before_);
   const int64_t before = ogle_hip_launch_count();
@@ -241,7 +265,7 @@ void Context::LaunchPending() {
       unreduced_.push_back(batch[i]);
       unreduced_labels_.push_back(labels[i]);
     }
-  if (unreduced_.empty()) workspace_used_ = 0;
+  if (pending_.empty() && unreduced_.empty()) workspace_used_ = 0;
 }
 
 void Context::Flush() {

@@ -117,8 +117,14 @@ class Context {
   // unreduced_: their reduction is only launched when something touches their output,
   // bias or workspace (FinishReductions with those ranges) or at Flush, so that all
   // reductions still open at that point share one grid.  Workspace slices are recycled
-  // once nothing is pending or unreduced.
+  // once nothing is pending or unreduced.  LaunchPendingThatConflict launches only the
+  // deferred convolutions that touch the given ranges: deferred convolutions never depend
+  // on each other (one that would is only queued after the ones it conflicts with have
+  // been launched), so the rest can wait for more company.
   void LaunchPending();
+  void LaunchPendingThatConflict(const MemRange* reads, int n_reads, const MemRange* writes,
+                                 int n_writes);
+  void LaunchBatch(std::vector<OgleConvArgs>& batch, std::vector<std::string>& labels);
   void FinishReductions(const MemRange* reads, int n_reads, const MemRange* writes, int n_writes,
                         bool all);
   std::vector<OgleConvArgs> pending_;

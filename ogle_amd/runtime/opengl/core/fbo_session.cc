@@ -24,8 +24,8 @@ namespace opengl {
 
 FBOSession::FBOSession(Context* context) : context_(context) {
   context_->Reset();
-  const char* env = std::getenv("OGLE_FILE_ORDER");
-  if (env != nullptr && env[0] != '\0' && env[0] != '0') reorder_ = false;
+  const char* env = std::getenv("OGLE_REORDER");
+  if (env != nullptr && env[0] != '\0' && env[0] != '0') reorder_ = true;
   env = std::getenv("OGLE_SIBLING_FUSION");
   if (env != nullptr && env[0] != '\0' && env[0] != '0') fuse_siblings_ = true;
 }
@@ -269,12 +269,12 @@ void FBOSession::PlaceInputsInOutputs() {
   }
 }
 
-// Issue order of a pass.  The context defers convolutions and launches the
-// deferred ones as one grid when something needs a result; in file order the SSD
-// heads all come last and fill the chip by themselves while the chain of small
-// feature-extractor convolutions before them runs one under-filled launch after
+// Issue order of a pass: file order, unless reordering was asked for.  The context defers
+// convolutions and launches the deferred ones as one grid when something needs a result; in
+// file order the SSD heads all come last and fill the chip by themselves while the chain of
+// small feature-extractor convolutions before them runs one under-filled launch after
 // another.  A head only needs its feature map, so it may be issued any time between
-// that map's launch and its own place in the file.  This pass simulates the
+// that map's launch and its own place in the file.  With reordering this pass simulates the
 // context's flush rule over the file order to find the launch groups, then moves
 // each convolution that has such slack to the group (within its window) where it
 // adds least to the estimated pass time: a group costs max(launch floor, work /

@@ -7,11 +7,12 @@
 // subgraphs are computed once during Setup (the ready_ flags), only the first Run
 // allocates.  Additions for a launch-bound GPU: Compute() replays the kernels
 // without re-uploading inputs, RunProfiled() brackets every node with HIP events,
-// CaptureGraph()/LaunchGraph() replay the whole run as one hipGraph, and the
-// convolutions whose results are not needed at once (the SSD heads) are issued
-// earlier than their place in the file, next to a convolution of the serial chain,
-// so that the two share one grid (set_reorder(false) or OGLE_FILE_ORDER=1 keeps
-// strict file order; results are the same either way).
+// CaptureGraph()/LaunchGraph() replay the whole run as one hipGraph.  On request
+// (set_reorder(true) or OGLE_REORDER=1) the convolutions whose results are not needed at
+// once (the SSD heads) are issued earlier than their place in the file, next to a
+// convolution of the serial chain, so that the two share one grid; results are the same
+// either way, and with the present kernels file order is the faster one (all heads in
+// one grid), so it is the default.
 #ifndef OPENGL_CORE_FBO_SESSION_H_
 #define OPENGL_CORE_FBO_SESSION_H_
 
@@ -104,7 +105,7 @@ class FBOSession {
   NamedIndex tensor_name_index_;
   std::vector<bool> ready_;
   bool allow_resized_ = false;
-  bool reorder_ = true;
+  bool reorder_ = false;
   bool fuse_siblings_ = false;
   std::vector<Kernel*> order_;  // the per-pass kernels in issue order (not owned)
   IntList default_input_sizes_;
