@@ -7,6 +7,8 @@
 // Semantics follow conv2d.glsl:29-92 / conv2d_grp.glsl:30-123: accumulator
 // starts at the bias, taps outside the image are skipped, then the fused
 // activation.  Accumulation order is ky, kx, input channel ascending.
+#include <algorithm>
+#include <type_traits>
 #include "common.h"
 
 namespace ogle {
@@ -88,6 +90,7 @@ __global__ __launch_bounds__(256) void conv_direct_small_k(
 // vector cache), all loads of a tile in flight before the first MFMA.  Rows past
 // the end, taps outside the image and the odd K tail contribute zeros.
 typedef float stem_acc_t __attribute__((ext_vector_type(16)));
+typedef unsigned int stem_u32x2 __attribute__((ext_vector_type(2)));
 
 // 32-bit element offset that no operand reaches (they are kept below 2^31 bytes):
 // a buffer access at it reads zero / is dropped.
@@ -148,26 +151,34 @@ __global__ __launch_bounds__(256) void conv_stem_mfma(
       bval[s] = (col < o && kidx < ktot) ? to_f32(w[(long)col * ktot + kidx]) : 0.f;
     }
     const float bias_v = (bias != nullptr && col < o) ? bias[col] : 0.f;
-    for (int tile = wave; tile < tiles_m; tile += waves) {
+    // the taps of a tile, all issued at once; a tile past the end reads zeros without touching memory
+    auto gather = [&](int tile, float (&dst)[KS]) {
       const int m = tile * 32 + l32;
       const int ox = m % ow;
       const int t = m / ow;
       const int oy = t % oh;
       const int b = t / oh;
       const int iy0 = oy * stride, ix0 = ox * stride;
-      const int base = m < m_total ? ((b * h + iy0) * wd + ix0) * c : -0x40000000;
-      float a[KS];
+      const int base = (tile < tiles_m && m < m_total) ? ((b * h + iy0) * wd + ix0) * c : -0x40000000;
 #pragma unroll
       for (int s = 0; s < KS; ++s) {
         const bool in = (unsigned)(iy0 + tap_dy[s]) < (unsigned)h &&
                         (unsigned)(ix0 + tap_dx[s]) < (unsigned)wd && base >= 0;
-        a[s] = stem_load<T>(rx, in ? (unsigned)(base + tap_off[s]) * ESZ : kStemOutOfRange);
+        dst[s] = stem_load<T>(rx, in ? (unsigned)(base + tap_off[s]) * ESZ : kStemOutOfRange);
       }
+    };
+    float a[KS], a_next[KS];
+    gather(wave, a);
+    for (int tile = wave; tile < tiles_m; tile += waves) {
+      // the next tile's taps are in flight while this tile is multiplied and stored
+      gather(tile + waves, a_next);
       stem_acc_t acc;
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[r] = 0.f;
 #pragma unroll
       for (int s = 0; s < KS; ++s) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], bval[s], acc, 0, 0, 0);
+#pragma unroll
+      for (int s = 0; s < KS; ++s) a[s] = a_next[s];
       // register r of lane l: pixel 8*(r/4) + 4*(l/32) + r%4 of the tile, channel l%32
       const int row0 = tile * 32 + lh * 4;
       const unsigned off0 = (unsigned)(row0 * o + col);
@@ -177,6 +188,103 @@ __global__ __launch_bounds__(256) void conv_stem_mfma(
         const bool ok = row0 + dr < m_total && col < o;
         stem_store<T>(ry, ok ? (off0 + (unsigned)(dr * o)) * ESZ : kStemOutOfRange,
                       apply_epilogue(acc[r] + bias_v, ep));
+      }
+    }
+  }
+}
+
+// The RGB stem (3x3 taps on 3 channels, fp32, even stride, padding 1, even width, output
+// channels a multiple of 32): the nine values one filter row needs for a pixel are nine
+// consecutive floats of an input row, so instead of 27 scalar gathers (a counter run showed 32
+// vector-cache accesses per such load instruction and the kernel bound by them) a lane fetches
+// its share of K as runs of 8-byte pairs.  With an even stride and padding 1 a pixel's run starts
+// at an odd float of its row, so the pair that starts one float earlier is 8-byte aligned.  The
+// lower half of the wave takes filter row 0 and the first five values of row 1, the upper half
+// the last four values of row 1 (plus one zero) and row 2: five pairs for the 9-run and three
+// for the rest, eight load instructions instead of fourteen, each twice as wide.  The
+// contraction order is permuted to match (the filter values a lane keeps are picked
+// accordingly).  Values that fall into padding columns are cleared with a per-lane test, and
+// so are padding rows, rows past the end and pairs outside the tensor.
+template <int UNUSED = 0>
+__global__ __launch_bounds__(256) void conv_stem_rgb_mfma(
+    const float* __restrict__ x, const float* __restrict__ w, const float* __restrict__ bias,
+    float* __restrict__ y, int h, int wd, int oh, int ow, int o, int stride, Epilogue ep,
+    int m_total, int tiles_m, unsigned x_bytes, unsigned y_bytes) {
+  constexpr int KS = 14;
+  const int lane = threadIdx.x & 63;
+  const int l32 = lane & 31, lh = lane >> 5;
+  const int wave = (int)(blockIdx.x * 4 + (threadIdx.x >> 6));
+  const int waves = (int)(gridDim.x * 4);
+  const __amdgpu_buffer_rsrc_t rx =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(x), 0, (int)x_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t ry = __builtin_amdgcn_make_buffer_rsrc(y, 0, (int)y_bytes, 0x00020000);
+  const int row_floats = wd * 3;
+  const unsigned total_floats = x_bytes / 4u;
+  const int run0_ky = lh ? 2 : 0;
+  const int run1_count = lh ? 4 : 5;
+  for (int n0 = 0; n0 < o; n0 += 32) {
+    const int col = n0 + l32;
+    float bval[KS];
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      const int k = s < 9 ? run0_ky * 9 + s : 9 + (lh ? 5 : 0) + (s - 9);
+      bval[s] = (s < 9 || s - 9 < run1_count) ? w[(long)col * 27 + k] : 0.f;
+    }
+    const float bias_v = bias != nullptr ? bias[col] : 0.f;
+    for (int tile = wave; tile < tiles_m; tile += waves) {
+      const int m = tile * 32 + l32;
+      const int ox = m % ow;
+      const int t = m / ow;
+      const int oy = t % oh;
+      const int b = t / oh;
+      const int iy0 = oy * stride - 1;
+      const int f0 = (ox * stride - 1) * 3;  // first float of a pixel's 9-run within an input row (odd)
+      // PAIRS 8-byte pairs of input row iy from float f (even) on.  Plain 8-byte loads (the
+      // 8-byte buffer load builtin compiles to a one-dword load with this toolchain); a pair
+      // outside the tensor, or of a row that does not exist, is read from the tensor's start
+      // instead and its values are cleared.
+      auto fetch = [&](int iy, int f, float* v, auto pairs) {
+        const bool row_ok = m < m_total && (unsigned)iy < (unsigned)h;
+        const int first = (b * h + iy) * row_floats + f;  // may be negative in the first row
+#pragma unroll
+        for (int i = 0; i < decltype(pairs)::value; ++i) {
+          const int at = first + 2 * i;
+          const bool ok = row_ok && (unsigned)at + 1u < total_floats;
+          const unsigned byte_off = ok ? (unsigned)at * 4u : 0u;
+          const float2 q = *reinterpret_cast<const float2*>(reinterpret_cast<const char*>(x) + byte_off);
+          v[2 * i] = ok ? q.x : 0.f;
+          v[2 * i + 1] = ok ? q.y : 0.f;
+        }
+      };
+      float v0[10], v1[6];
+      fetch(iy0 + run0_ky, f0 - 1, v0, std::integral_constant<int, 5>());
+      // filter row 1: floats [f0, f0 + 5) for the lower half, [f0 + 5, f0 + 9) for the upper
+      const int f1 = lh ? f0 + 5 : f0 - 1;
+      fetch(iy0 + 1, f1, v1, std::integral_constant<int, 3>());
+      float a[KS];
+#pragma unroll
+      for (int j = 0; j < 9; ++j)
+        a[j] = (unsigned)(f0 + j) < (unsigned)row_floats ? v0[j + 1] : 0.f;
+#pragma unroll
+      for (int j = 0; j < 5; ++j) {
+        const int f = lh ? f0 + 5 + j : f0 + j;
+        const float val = lh ? v1[j] : v1[j + 1];
+        a[9 + j] = ((unsigned)f < (unsigned)row_floats && j < run1_count) ? val : 0.f;
+      }
+      stem_acc_t acc;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+#pragma unroll
+      for (int s = 0; s < KS; ++s) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], bval[s], acc, 0, 0, 0);
+      // register r of lane l: pixel 8*(r/4) + 4*(l/32) + r%4 of the tile, channel l%32; rows
+      // past the end lie past the end of the buffer and are dropped by the range check
+      const unsigned off0 = (unsigned)((tile * 32 + lh * 4) * o + col) * 4u;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int dr = (r >> 2) * 8 + (r & 3);
+        __builtin_amdgcn_raw_buffer_store_b32(
+            __builtin_bit_cast(unsigned, apply_epilogue(acc[r] + bias_v, ep)), ry,
+            (int)(off0 + (unsigned)(dr * o) * 4u), 0, 0);
       }
     }
   }
@@ -246,6 +354,17 @@ int32_t run_direct(const OgleConvArgs& a, hipStream_t s) {
       taps.dx[kidx] = (tap % a.kernel_size) * a.dilation - a.padding;
       taps.off[kidx] = (taps.dy[kidx] * a.in_w + taps.dx[kidx]) * a.in_c + ci;
       if (kidx >= ktot) taps.dy[kidx] = -0x40000000;
+    }
+    if (sizeof(T) == 4 && a.kernel_size == 3 && a.in_c == 3 && a.dilation == 1 && a.padding == 1 &&
+        a.stride % 2 == 0 && a.in_w % 2 == 0 && a.out_c % 32 == 0 &&
+        reinterpret_cast<uintptr_t>(x) % 8 == 0) {
+      // four workgroups per compute unit measured best for this one (17.3 against 18.3 us at batch 16)
+      const int rgb_blocks = std::min((tiles_m + 3) / 4, 256 * 4);
+      launch((conv_stem_rgb_mfma<0>), dim3(rgb_blocks), dim3(256), 0, s,
+             reinterpret_cast<const float*>(x), reinterpret_cast<const float*>(w), a.bias_dev,
+             reinterpret_cast<float*>(y), a.in_h, a.in_w, a.out_h, a.out_w, a.out_c, a.stride, ep,
+             (int)pixels_all, tiles_m, (unsigned)x_bytes, (unsigned)y_bytes);
+      return check_launch("conv_stem_rgb_mfma");
     }
 #define OGLE_STEM_CASE(KS)                                                                        \
   launch((conv_stem_mfma<T, KS>), dim3(blocks), dim3(256), 0, s, x, w, a.bias_dev, y,  \

@@ -106,7 +106,13 @@ def test_conv_shape_sweep_dense_and_depthwise():
 
 STEM_CASES = [
     # n, h, w, c, o, k, s, p, d   (K = k*k*c <= 32 and >= 4096 output pixels: the MFMA stem kernel)
-    (2, 96, 96, 3, 32, 3, 2, 1, 1),     # the RGB stem shape
+    (2, 96, 96, 3, 32, 3, 2, 1, 1),     # the RGB stem shape (pair loads: even stride, padding 1, even width)
+    (3, 75, 78, 3, 64, 3, 2, 1, 1),     # RGB pair loads, odd height, ragged last tile, two channel tiles
+    (2, 50, 90, 3, 32, 3, 4, 1, 1),     # RGB pair loads, stride 4, the right edge is padding
+    (3, 75, 77, 3, 32, 3, 2, 1, 1),     # RGB, odd width: the general kernel
+    (2, 66, 65, 3, 64, 3, 1, 1, 1),     # RGB, stride 1, two channel tiles
+    (2, 71, 70, 3, 32, 3, 2, 0, 1),     # RGB, no padding
+    (1, 131, 67, 3, 96, 3, 3, 1, 1),    # RGB, stride 3
     (1, 70, 67, 3, 20, 3, 1, 1, 1),     # ragged pixel count, fewer channels than a tile
     (1, 65, 66, 1, 40, 3, 1, 0, 1),     # one input channel, two channel tiles, no padding
     (1, 80, 80, 2, 33, 3, 1, 2, 2),     # dilation 2
