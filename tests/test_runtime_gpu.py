@@ -677,3 +677,45 @@ def test_launch_plan_names_every_dispatch_and_times_it():
     assert all(len(us) >= 1 and all(0.5 < u < 1000.0 for u in us) for _, us in plan)
     assert [l for l, k in sess.launch_plan()] == ["dw#Conv#", "pw#Conv#"]
     np.testing.assert_array_equal(sess.get_output("pw", "NHWC"), want)
+
+
+def test_convolution_only_forces_out_what_it_conflicts_with():
+    """Deferred convolutions never depend on each other, so one that needs a deferred result
+    launches only the convolutions it conflicts with and joins the rest: a -> c with b
+    independent of both goes out as [a], then [b + c] in one grid; a launch of any other kind
+    (the pool) takes the whole queue.  Outputs equal the oracle's, eager and replayed."""
+    r = rng(8200)
+    gb = dlx.GraphBuilder()
+    x = gb.add_input("input", [2, 16, 12, 12])
+    ws = {}
+    for name, cin, cout, k in (("a", 16, 32, 3), ("b", 16, 24, 1), ("c", 32, 16, 1)):
+        ws[name] = (r.normal(0, 0.2, (cout, cin, k, k)).astype(np.float32),
+                    r.normal(0, 0.1, cout).astype(np.float32))
+    def conv(name, src, k, pad):
+        w, b = ws[name]
+        return gb.add_conv(name, src, gb.add_filter(name + ".w", w), gb.add_const(name + ".b", b),
+                           kernel=k, pad=pad, activation_type="Relu")
+    a = conv("a", x, 3, 1)
+    b = conv("b", x, 1, 0)
+    c = conv("c", a, 1, 0)
+    gb.add_pool("pool", b, "MaxPool", 2, 2, 0)
+    xin = r.uniform(-1, 1, (2, 12, 12, 16)).astype(np.float32)
+    sess = session.Session()
+    sess.load_graph(gb)
+    sess.run({"input": xin})
+    plan = [l for l, _ in sess.launch_plan()]
+    assert plan == ["a#Conv#", "b#Conv#+c#Conv#", "pool#MaxPool#"], plan
+    ra = O.conv2d(xin, *ws["a"], 1, 1, 1, 1, O.ACT_RELU)
+    rb = O.conv2d(xin, *ws["b"], 1, 0, 1, 1, O.ACT_RELU)
+    da = sess.get_output("a", "NHWC")
+    assert_conv_close(da, ra, O.conv2d_abs(xin, *ws["a"], 1, 1), FP32_RTOL, "a")
+    assert_conv_close(sess.get_output("b", "NHWC"), rb, O.conv2d_abs(xin, *ws["b"], 1, 0), FP32_RTOL, "b")
+    assert_conv_close(sess.get_output("c", "NHWC"), O.conv2d(da, *ws["c"], 1, 0, 1, 1, O.ACT_RELU),
+                      O.conv2d_abs(da, *ws["c"], 1, 0), FP32_RTOL, "c")
+    np.testing.assert_array_equal(sess.get_output("pool", "NHWC"),
+                                  O.pool2d(sess.get_output("b", "NHWC"), 2, 2, 0, O.POOL_MAX))
+    eager = {n: sess.get_output(n, "NHWC") for n in ("a", "b", "c", "pool")}
+    sess.compute(graph=True)
+    sess.compute(graph=True)
+    for n, v in eager.items():
+        np.testing.assert_array_equal(sess.get_output(n, "NHWC"), v)
