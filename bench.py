@@ -229,6 +229,18 @@ def kernel_table(iters=50, warm=5):
             ga.element_size() * (ga.numel() + gb.numel() + gc.numel()), "mfma",
             MFMA_F32_PEAK_TFLOPS if dt == torch.float32 else 2500.0)
 
+    # yardstick for the bandwidth-bound rows: a plain copy too large for the 256 MB last-level
+    # cache (1 GiB in, 1 GiB out), i.e. what HBM itself delivers to a streaming kernel here
+    big = 1 << 28
+    gsrc = torch.ones(big, dtype=torch.float32, device="cuda")
+    gdst = torch.empty_like(gsrc)
+    row("plain copy 1 GiB -> 1 GiB, library copy kernel (HBM yardstick)",
+        timed(lambda: H.check(L.ogle_hip_convert(gsrc.data_ptr(), H.F32, gdst.data_ptr(), H.F32, big, st)),
+              ), 0.0, 8.0 * big, "hbm")
+    row("plain copy 1 GiB -> 1 GiB, torch copy_ (HBM yardstick)", timed(lambda: gdst.copy_(gsrc)), 0.0,
+        8.0 * big, "hbm")
+    del gsrc, gdst
+
     # C4: the twelve SSD head convolutions of 64 images in one grouped call
     maps = [(19, 512, 3), (10, 1024, 6), (5, 512, 6), (3, 256, 6), (2, 256, 6), (1, 128, 6)]
     probs = []
