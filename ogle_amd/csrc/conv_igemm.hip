@@ -1001,9 +1001,9 @@ IgemmPlan plan_igemm(const OgleConvArgs& a, long m, bool allow_split) {
   // launch), whether or not a workspace was offered.  Measured on MI355X against
   // split-K + reduce: the 32x32 form wins once its tiles cover half the chip, for
   // K <= 1024 pointwise and K <= 512 otherwise; the 16x16 form wins for pointwise
-  // K <= 1024 while its tiles stay under two per compute unit, and for K <= 1536 on the
-  // very small maps; a longer K per wave is a serial chain of MFMAs and loses to the
-  // split across workgroups.
+  // K <= 1024 while its tiles stay under two per compute unit, and for K <= 1536 while they
+  // stay under one per unit (3x3x256 <- 5x5x128 at batch 16: 7.0 against 9.5 us); a longer K
+  // per wave is a serial chain of MFMAs and loses to the split across workgroups.
   {
     const long k_total = (long)a.kernel_size * a.kernel_size * a.in_c;
     const bool pw = is_pointwise(a);
@@ -1011,10 +1011,13 @@ IgemmPlan plan_igemm(const OgleConvArgs& a, long m, bool allow_split) {
                              (t < 8 * kComputeUnits && p.ktiles >= 128);
     const long t32 = tiles(CFG_WAVE32), t16 = tiles(CFG_WAVE16);
     const bool small16 = (pw && k_total <= 1024 && t16 <= 2 * kComputeUnits) ||
-                         (k_total <= 1536 && t16 <= kComputeUnits / 2);
+                         (k_total <= 1536 && t16 <= kComputeUnits);
+    // other than pointwise: K <= 512, or up to 2304 while every 32x32 tile has a compute unit
+    // to itself (5x5x512 <- 10x10x256, 3x3 stride 2, at batch 16: 19.8 against 21.6 us)
+    const long k32cap = t32 <= kComputeUnits ? 2304 : 512;
     if (narrow_long) {
       // stays on the wide tile
-    } else if (would_split && !small16 && k_total <= (pw ? 1024 : 512) && t32 >= kComputeUnits / 2 &&
+    } else if (would_split && !small16 && k_total <= (pw ? 1024 : k32cap) && t32 >= kComputeUnits / 2 &&
         t32 <= 4 * kComputeUnits) {
       p.cfg = CFG_WAVE32;
       p.splits = 1;
