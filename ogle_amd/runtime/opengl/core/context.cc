@@ -133,22 +133,21 @@ void Context::BeforeLaunch(const MemRange* reads, int n_reads, const MemRange* w
 void Context::FinishReductions(const MemRange* reads, int n_reads, const MemRange* writes,
                                int n_writes, bool all) {
   if (unreduced_.empty()) return;
-  std::vector<OgleConvArgs> now, keep;
-  std::vector<std::string> now_labels, keep_labels;
-  for (size_t i = 0; i < unreduced_.size(); ++i) {
-    bool hit = all;
-    if (!hit) {
-      OgleConvArgs c = unreduced_[i];
-      c.input_dev = nullptr;   // no longer read
-      c.filter_dev = nullptr;
-      hit = Conflicts(&c, 1, reads, n_reads, writes, n_writes);
-    }
-    (hit ? now : keep).push_back(unreduced_[i]);
-    (hit ? now_labels : keep_labels).push_back(unreduced_labels_[i]);
+  // One reduction that is needed takes every open one with it: they share the grid, and the
+  // others' results are wanted soon after (the box concat asks for six head reductions, the
+  // class concat for the other six a launch later).
+  bool any = all;
+  for (size_t i = 0; i < unreduced_.size() && !any; ++i) {
+    OgleConvArgs c = unreduced_[i];
+    c.input_dev = nullptr;   // no longer read
+    c.filter_dev = nullptr;
+    any = Conflicts(&c, 1, reads, n_reads, writes, n_writes);
   }
-  if (now.empty()) return;
-  unreduced_.swap(keep);
-  unreduced_labels_.swap(keep_labels);
+  if (!any) return;
+  std::vector<OgleConvArgs> now;
+  std::vector<std::string> now_labels;
+  now.swap(unreduced_);
+  now_labels.swap(unreduced_labels_);
   if (!current_label_.empty()) LogLaunches(current_label_, node_count_before_);
   const int64_t before = ogle_hip_launch_count();
   const int32_t st = ogle_hip_conv2d_batch_finish(now.data(), static_cast<int32_t>(now.size()), stream());
