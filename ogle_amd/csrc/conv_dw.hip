@@ -273,7 +273,18 @@ int32_t launch_rows(const OgleConvArgs& a, hipStream_t s, const Epilogue& ep, in
 // and below, where the number of waves, not the re-read rows, decides the time.
 template <typename T, int S>
 int32_t pick_rows(const OgleConvArgs& a, hipStream_t s, const Epilogue& ep) {
-  const int seg_rows = (S == 1 && a.out_h > 40) ? 13 : 4;
+  int seg_rows = (S == 1 && a.out_h > 40) ? 13 : 4;
+  // Few images: with fewer than one workgroup per compute unit the launch is a handful of
+  // long serial walks (150x150x32 at batch 1: 28 workgroups of 13-row walks, 7.6 us); shorter
+  // segments make more of them (the rows a segment re-reads do not matter at this size).
+  {
+    constexpr int V = Vec<T>::N;
+    const int q = (S == 1 && a.out_w >= 2) ? 2 : 1;
+    auto workgroups = [&](int rows) {
+      return ((long)a.n * ((a.out_h + rows - 1) / rows) * ((a.out_w + q - 1) / q) * (a.in_c / V) + 255) / 256;
+    };
+    while (seg_rows > 2 && workgroups(seg_rows) < 256) seg_rows = seg_rows > 4 ? 4 : 2;
+  }
   if (S == 1 && a.out_w >= 2) return launch_rows<T, S, 2, 1>(a, s, ep, seg_rows);
   return launch_rows<T, S, 1, 1>(a, s, ep, seg_rows);
 }
