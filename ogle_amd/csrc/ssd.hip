@@ -410,9 +410,9 @@ __global__ __launch_bounds__(kNmsThreads) void ssd_topk_nms_kernel(NmsParams p) 
   unsigned prefix = 0, mask = 0;
   int remaining = m;  // how many of the entries matching `prefix` are still wanted
   if (nv > p.topk) {
+    if (tid < 256) hist[tid] = 0;
+    __syncthreads();
     for (int shift = 24; shift >= 0; shift -= 8) {
-      if (tid < 256) hist[tid] = 0;
-      __syncthreads();
       for (int i = tid; i < n; i += kNmsThreads) {
         const unsigned k = keys[i];
         // (empty slots stay out: they would all hit one counter, and cannot be chosen)
@@ -420,8 +420,10 @@ __global__ __launch_bounds__(kNmsThreads) void ssd_topk_nms_kernel(NmsParams p) 
       }
       __syncthreads();
       // thread t < 256: entries whose digit is above t, and at or above t (suffix sums
-      // of the histogram: a shuffle scan inside each wave plus the totals of later waves)
+      // of the histogram: a shuffle scan inside each wave plus the totals of later waves);
+      // it also clears its counter for the next pass
       const int mine = tid < 256 ? hist[tid] : 0;
+      if (tid < 256) hist[tid] = 0;
       int sfx = mine;
 #pragma unroll
       for (int d = 1; d < 64; d <<= 1) {
@@ -440,34 +442,56 @@ __global__ __launch_bounds__(kNmsThreads) void ssd_topk_nms_kernel(NmsParams p) 
         }
       }
       __syncthreads();
+      // (the chosen digit is next written two barriers from here, the wave totals one)
       prefix |= (unsigned)misc[kNmsWaves] << shift;
       mask |= 255u << shift;
       remaining -= misc[kNmsWaves + 1];
-      __syncthreads();  // misc and hist are rewritten by the next pass
     }
+    __syncthreads();  // misc is reused by the compaction
   }
   // now: take every key above `prefix`, and the first `remaining` equal to it
   // (nv <= topk: every entry is taken)
 
-  // 2. ordered compaction of the selected entries
+  // 2. ordered compaction of the selected entries.  A thread takes a contiguous run of slots
+  // and counts, in one packed word, its entries above the k-th key and its entries equal to
+  // it; one scan over the workgroup gives both counts for everything before the run, and an
+  // entry's place follows from them: (above before it) + min(equal before it, remaining).
   {
-    int taken = 0, equal_seen = 0;
-    for (int start = 0; start < n; start += kNmsThreads) {
-      const int i = start + tid;
+    const int per = (n + kNmsThreads - 1) / kNmsThreads;
+    const int first = tid * per;
+    unsigned mine = 0;  // above | equal << 16  (n < 65536: the keys fit in LDS)
+    for (int e = 0; e < per; ++e) {
+      const int i = first + e;
+      const unsigned k = i < n ? keys[i] : 0u;
+      const bool live = i < n && (!SPARSE || k != 0u);
+      if (live && (nv <= p.topk || k > prefix)) mine += 1u;
+      if (live && nv > p.topk && k == prefix) mine += 65536u;
+    }
+    unsigned incl = mine;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const unsigned v = __shfl_up(incl, d, 64);
+      if (lane >= d) incl += v;
+    }
+    unsigned* wave_total = reinterpret_cast<unsigned*>(misc);
+    if (lane == 63) wave_total[wave] = incl;
+    __syncthreads();
+    unsigned before = incl - mine;
+    for (int wv = 0; wv < wave; ++wv) before += wave_total[wv];
+    int above = (int)(before & 0xffffu), equal = (int)(before >> 16);
+    for (int e = 0; e < per; ++e) {
+      const int i = first + e;
       const unsigned k = i < n ? keys[i] : 0u;
       const bool live = i < n && (!SPARSE || k != 0u);
       const bool gt = live && (nv <= p.topk || k > prefix);
       const bool eq = live && nv > p.topk && k == prefix;
-      int eq_total, total;
-      const int eq_before = equal_seen + block_rank(eq, misc, lane, wave, &eq_total);
-      const bool take = gt || (eq && eq_before < remaining);
-      const int before = taken + block_rank(take, misc, lane, wave, &total);
-      if (take) {
-        cand_key[before] = k;
-        cand_idx[before] = i;
+      if (gt || (eq && equal < remaining)) {
+        const int at = above + (equal < remaining ? equal : remaining);
+        cand_key[at] = k;
+        cand_idx[at] = i;
       }
-      taken += total;
-      equal_seen += eq_total;
+      above += gt ? 1 : 0;
+      equal += eq ? 1 : 0;
     }
   }
   for (int r = m + tid; r < ((m + 3) & ~3); r += kNmsThreads) cand_key[r] = 0u;  // padding ranks last
@@ -508,16 +532,29 @@ __global__ __launch_bounds__(kNmsThreads) void ssd_topk_nms_kernel(NmsParams p) 
   // 4. NMS: all (i, j) pairs with i < j are spread over the workgroup; a pair that
   // overlaps by more than the threshold marks j (every writer stores the same value)
   if (m > 1) {
-    // pair number t = i * m + j, advanced by the thread count per step without dividing
-    const int step_i = kNmsThreads / m, step_j = kNmsThreads - step_i * m;
-    int i = tid / m, j = tid - i * m;
-    for (; i < m; i += step_i, j += step_j) {
-      if (j >= m) {
-        j -= m;
-        ++i;
-        if (i >= m) break;
+    // Only the pairs with i < j are visited: they are laid out as rows of equal length (row a
+    // holds the pairs (a, j > a) and fills up with those of the row that mirrors it), and a
+    // thread steps through them by the thread count without dividing.
+    const bool odd = (m & 1) != 0;
+    const int len = odd ? m : m - 1;
+    const int rows = odd ? (m - 1) / 2 : m / 2;
+    const int step_a = kNmsThreads / len, step_b = kNmsThreads - step_a * len;
+    int a = tid / len, b = tid - a * len;
+    for (; a < rows; a += step_a, b += step_b) {
+      if (b >= len) {
+        b -= len;
+        ++a;
+        if (a >= rows) break;
       }
-      if (i < j && corner_iou(frects[i], frects[j]) > p.threshold) dropped[j] = 1;
+      int i, j;
+      if (odd) {
+        i = b > a ? a : m - 2 - a;
+        j = b > a ? b : m - 1 - b;
+      } else {
+        i = b >= a ? a : m - 1 - a;
+        j = b >= a ? b + 1 : m - 1 - b;
+      }
+      if (corner_iou(frects[i], frects[j]) > p.threshold) dropped[j] = 1;
     }
   }
   __syncthreads();
