@@ -276,3 +276,37 @@ def test_residual_graph_onnx_to_device():
     assert_conv_close(folded.get_output("c1.act", "NHWC"), ref1, O.conv2d_abs(x, wf, bf, 1, 1), FP32_RTOL,
                       "onnx c1")
     assert len(folded.issue_order()) == 5
+
+
+@pytest.mark.gpu
+def test_classifier_tail_onnx_to_device():
+    """GlobalAveragePool -> Flatten -> Gemm (transB = 1, the Linear form) from ONNX: the converters
+    of the ops that close a MobileNet classifier, end to end."""
+    from ogle_amd import session
+    w = WRITERS["proto2"]
+    r = rng(31020)
+    batch, c, classes = 3, 256, 40
+    wt = r.normal(0, 0.05, (classes, c)).astype(np.float32)
+    b = r.normal(0, 0.1, classes).astype(np.float32)
+    nodes = [w.node("GlobalAveragePool", ["input"], ["pool"]),
+             w.node("Flatten", ["pool"], ["flat"], axis=1),
+             w.node("Gemm", ["flat", "fc.w", "fc.b"], ["logits"], alpha=1.0, beta=1.0, transB=1)]
+    blob = w.model(nodes, [w.value_info("input", [batch, c, 7, 7])], [w.value_info("logits", [batch, classes])],
+                   [w.tensor("fc.w", wt), w.tensor("fc.b", b, raw=True)])
+    model = onnx.convert(blob)
+    by = {n["name"]: n for n in dlx.decode_model(model)["graph"]["nodes"]}
+    assert [by[n]["type"] for n in ("pool", "flat", "fc.w", "fc.b", "logits")] == \
+        ["GlobalAveragePool", "Flatten", "Const", "Const", "Gemm"]
+    gemm = dict((f, v) for f, _, v in dlx._fields(by["logits"]["attr"][dlx.ATTR_GEMM]))
+    assert struct.unpack("<f", gemm[1])[0] == 1.0 and struct.unpack("<f", gemm[2])[0] == 1.0 and gemm[3] == 1
+    x = r.uniform(0, 6, (batch, 7, 7, c)).astype(np.float32)
+    sess = session.Session()
+    sess.load_graph(model)
+    sess.run({"input": x})
+    pooled = sess.get_output("flat", "ANY")
+    np.testing.assert_allclose(pooled, O.pool2d(x, 7, 1, 0, O.POOL_GLOBAL_AVG).reshape(batch, c), rtol=1e-6, atol=1e-6)
+    ref = O.gemm(pooled, wt, b, 1.0, 1.0, True)
+    scale = np.abs(pooled).astype(np.float64) @ np.abs(wt).astype(np.float64).T + np.abs(b)
+    got = sess.get_output("logits", "ANY")
+    assert got.shape == (batch, classes)
+    assert np.all(np.abs(got - ref) <= 1e-5 * scale)
