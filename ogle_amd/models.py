@@ -58,23 +58,30 @@ def mobilenet_v1_ssd(batch, seed=20240005, num_classes=21, image=300, head_std=0
     the extras, concatenated to box_preds (N, 1917, 4) and cls_logits (N, 1917, classes).
     BN (gamma~U(.5,1.5), beta, mean~N(0,.1), var~U(.5,1.5)) is folded; activation ReLU6 as
     Clip(0, 6).  Returns (GraphBuilder, info) where info lists every conv layer
-    (name, kind, shapes) and, if with_weights, the folded weights for an oracle run."""
+    (name, kind, shapes) and, if with_weights, the folded weights for an oracle run plus, under
+    "unfolded", what they were folded from: name -> (w, gamma, beta, mean, var), or (w,) for a
+    head."""
     r = np.random.Generator(np.random.PCG64(seed))
     g = dlx.GraphBuilder()
     x = g.add_input("input", [batch, 3, image, image])
     layers = []
     weights = {}
+    unfolded = {}
 
     def conv_bn(name, x, cin, cout, k, stride, pad, group=1, bn=True, act=True, std=None):
         fan_in = (cin // group) * k * k
         std = np.sqrt(2.0 / fan_in) if std is None else std
         w = r.normal(0, std, (cout, cin // group, k, k)).astype(np.float32)
         b = None
+        if with_weights:
+            unfolded[name] = (w,)
         if bn:
             gamma = r.uniform(0.5, 1.5, cout).astype(np.float32)
             beta = r.normal(0, 0.1, cout).astype(np.float32)
             mean = r.normal(0, 0.1, cout).astype(np.float32)
             var = r.uniform(0.5, 1.5, cout).astype(np.float32)
+            if with_weights:
+                unfolded[name] = (w, gamma, beta, mean, var)
             w, b = fold_batchnorm(w, None, gamma, beta, mean, var)
         wi = g.add_filter(name + ".weight", w)
         bi = g.add_const(name + ".bias", b) if b is not None else None
@@ -141,7 +148,7 @@ def mobilenet_v1_ssd(batch, seed=20240005, num_classes=21, image=300, head_std=0
         l["weight_bytes"] = 4 * (w_elems + (l["cout"] if l["name"].find("head") < 0 else 0))
         l["act_bytes_per_image"] = 4 * (l["in_size"] ** 2 * l["cin"] + out_size ** 2 * l["cout"])
     info = dict(layers=layers, priors=priors, num_classes=num_classes, weights=weights,
-                anchors=anchors, seed=seed)
+                unfolded=unfolded, anchors=anchors, seed=seed)
     return g, info
 
 

@@ -310,3 +310,99 @@ def test_classifier_tail_onnx_to_device():
     got = sess.get_output("logits", "ANY")
     assert got.shape == (batch, classes)
     assert np.all(np.abs(got - ref) <= 1e-5 * scale)
+
+
+def ssd_onnx(w, info, batch, image=300):
+    """MobileNet-v1-SSD as an exporter writes it before constant folding: every backbone and
+    extra layer Conv -> BatchNormalization -> Clip(0, 6), every head Conv -> Transpose(0,2,3,1)
+    -> Reshape (shape from a Constant node) and the two Concat nodes over axis 1, with the
+    weights of models.mobilenet_v1_ssd(with_weights=True) before their folding."""
+    nodes, inits = [], []
+    taps = {"block11.pw": 0, "block13.pw": 1, "extra1.conv": 2, "extra2.conv": 3, "extra3.conv": 4,
+            "extra4.conv": 5}
+    maps, cur = {}, "input"
+    locs, confs = [], []
+    for l in info["layers"]:
+        name, un = l["name"], info["unfolded"][l["name"]]
+        head = name.startswith("head")
+        src = maps[int(name[4:name.index(".")])] if head else cur
+        inits.append(w.tensor(name + ".w", un[0], raw=True))
+        nodes.append(w.node("Conv", [src, name + ".w"], [name if head else name + ".conv"],
+                            kernel_shape=[l["k"]] * 2, strides=[l["stride"]] * 2, pads=[l["pad"]] * 4,
+                            dilations=[1, 1], group=l["group"]))
+        if head:
+            last = 4 if name.endswith(".loc") else info["num_classes"]
+            nodes.append(w.node("Transpose", [name], [name + ".permute"], perm=[0, 2, 3, 1]))
+            nodes.append(w.node("Constant", [], [name + ".shape"],
+                                value=w.tensor("", np.array([batch, -1, last], np.int64))))
+            nodes.append(w.node("Reshape", [name + ".permute", name + ".shape"], [name + ".view"]))
+            (locs if last == 4 else confs).append(name + ".view")
+            continue
+        inits += [w.tensor("%s.%s" % (name, t), v) for t, v in zip("gbmv", un[1:])]
+        nodes.append(w.node("BatchNormalization", [name + ".conv"] + ["%s.%s" % (name, t) for t in "gbmv"],
+                            [name + ".bn"], epsilon=1e-5, momentum=0.9))
+        nodes.append(w.node("Clip", [name + ".bn"], [name], min=0.0, max=6.0))
+        cur = name
+        if name in taps:
+            maps[taps[name]] = name
+    nodes.append(w.node("Concat", locs, ["box_preds"], axis=1))
+    nodes.append(w.node("Concat", confs, ["cls_logits"], axis=1))
+    nodes.append(w.node("Constant", [], ["anchors"], value=w.tensor("", info["anchors"], raw=True)))
+    outs = [w.value_info("cls_logits", [batch, info["priors"], info["num_classes"]]),
+            w.value_info("box_preds", [batch, info["priors"], 4]),
+            w.value_info("anchors", [info["priors"], 4])]
+    return w.model(nodes, [w.value_info("input", [batch, 3, image, image])], outs, inits)
+
+
+def test_whole_detector_converts_and_folds():
+    """47 convolutions, 35 of them with BatchNormalization and Clip behind them: after conversion
+    and the remapper, what is left is the graph models.mobilenet_v1_ssd builds directly, with the
+    same folded weights."""
+    from ogle_amd import models
+    g, info = models.mobilenet_v1_ssd(1, with_weights=True)
+    blob = ssd_onnx(WRITERS["proto3"], info, 1)
+    plain = dlx.decode_model(onnx.convert(blob))["graph"]["nodes"]
+    kinds = [n["type"] for n in plain]
+    assert kinds.count("Conv") == 47 and kinds.count("BatchNormalization") == 35 and kinds.count("Clip") == 35
+    folded, n_bn, n_act = onnx.convert_and_fold(blob)
+    assert (n_bn, n_act) == (35, 35)
+    model = dlx.decode_model(folded)
+    nodes, names = model["graph"]["nodes"], model["graph"]["tensor_names"]
+    kinds = [n["type"] for n in nodes]
+    assert kinds.count("Conv") == 47 and "BatchNormalization" not in kinds and "Clip" not in kinds
+    assert kinds.count("Concat") == 2 and kinds.count("Reshape") == 12 and kinds.count("Transpose") == 12
+    direct = {n["name"]: n for n in dlx.decode_model(g.serialize())["graph"]["nodes"]}
+    by = {n["name"]: n for n in nodes}
+    for name in ("conv0", "block7.dw", "block13.pw", "extra2.conv"):
+        conv = by[name]
+        wf, bf = info["weights"][name]
+        got_w = const_of(model, names[conv["input_index"][1]])
+        got_b = const_of(model, names[conv["input_index"][2]])
+        assert got_w["dims"] == list(wf.shape)
+        np.testing.assert_allclose(got_w["float_data"].reshape(wf.shape), wf, rtol=2e-6, atol=1e-7)
+        np.testing.assert_allclose(got_b["float_data"], bf, rtol=2e-6, atol=1e-7)
+        assert dlx.decode_conv2d_attr(conv["attr"][dlx.ATTR_CONV2D]) == \
+            dlx.decode_conv2d_attr(direct[name]["attr"][dlx.ATTR_CONV2D])
+
+
+@pytest.mark.gpu
+def test_whole_detector_onnx_to_device():
+    """The detector's ONNX form, converted and folded, gives the outputs of the directly built
+    graph on the device (both run the same kernels; the folded weights may differ in the last
+    bit, so outputs agree to a small multiple of the fp32 unit against their scale)."""
+    from ogle_amd import models, session
+    batch = 2
+    g, info = models.mobilenet_v1_ssd(batch, with_weights=True)
+    folded = onnx.convert_and_fold(ssd_onnx(WRITERS["proto2"], info, batch))[0]
+    x = rng(31030).uniform(-1, 1, (batch, 300, 300, 3)).astype(np.float32)
+    outs = {}
+    for tag, blob in (("direct", g.serialize()), ("onnx", folded)):
+        sess = session.Session()
+        sess.load_graph(blob)
+        sess.run({"input": x})
+        outs[tag] = {n: sess.get_output(n, "ANY") for n in ("cls_logits", "box_preds", "anchors")}
+    np.testing.assert_array_equal(outs["onnx"]["anchors"], outs["direct"]["anchors"])
+    for name in ("cls_logits", "box_preds"):
+        a, b = outs["onnx"][name], outs["direct"][name]
+        assert a.shape == b.shape
+        assert np.abs(a - b).max() <= 1e-4 * np.abs(b).max(), name
