@@ -218,7 +218,7 @@ REL_FLOOR = 1e-2
 FP16_REL_FLOOR = 5e-2
 
 # what -> (worst normwise ratio err/scale, worst relative error where test (2) applies):
-# the achieved figures, written to gpurun_out/parity_achieved.json at the end of a GPU session.
+# the achieved figures, written as parity_achieved.json at the end of a GPU session (conftest.py).
 PARITY_LOG = {}
 
 
