@@ -181,7 +181,22 @@ typedef struct OgleConvArgs {
    * fp16 storage: in_c % 8 == 0): otherwise OGLE_ERR_UNSUPPORTED. */
   void* output2_dev;
   int32_t out_c_split;
+  /* Optional distance, in elements, between the first outputs of consecutive images in
+   * output_dev (0: the images follow each other, out_h * out_w * out_c apart).  A larger
+   * value leaves a gap after every image: each image's out_h * out_w * out_c outputs stay
+   * contiguous, and image b starts at output_dev + b * out_image_stride.  This is how a
+   * convolution writes straight into its place inside the output of a Concat over axis 1
+   * (the SSD box and class heads at batch > 1), which then has nothing left to copy; the
+   * reference draws the head, then copies it (concat.cc:49-99).  Must be 0 or at least
+   * out_h * out_w * out_c, and cannot be combined with output2_dev.  Only the MFMA
+   * implicit-GEMM path takes it (ogle_hip_conv_takes_image_stride): otherwise
+   * OGLE_ERR_UNSUPPORTED. */
+  int64_t out_image_stride;
 } OgleConvArgs;
+
+/* 1 if a convolution of this geometry and dtype runs on a path that honours
+ * out_image_stride, 0 if not (pointers are not looked at). */
+int32_t ogle_hip_conv_takes_image_stride(const OgleConvArgs* args);
 
 /* Bytes of workspace the fastest plan for `args` would use (0 if it needs none). */
 size_t ogle_hip_conv_workspace_bytes(const OgleConvArgs* args);

@@ -68,6 +68,13 @@ int32_t ogle_rt_hazard_conflicts(const OgleConvArgs* pending, int32_t n_pending,
                                  int32_t n_reads, const void* const* write_ptrs,
                                  const size_t* write_bytes, int32_t n_writes);
 
+/* The same rule for a convolution as the next launch: what `next` reads (input, filter,
+ * bias) and writes (output(s), workspace; with out_image_stride one range per image, so
+ * that convolutions whose images interleave inside one tensor do not count as
+ * overlapping) against the `n_pending` deferred ones. */
+int32_t ogle_rt_conv_hazard_conflicts(const OgleConvArgs* pending, int32_t n_pending,
+                                      const OgleConvArgs* next);
+
 /*
  * Times `iters` passes (after `warmup` untimed ones) with HIP events recorded on
  * the session's stream; inputs stay resident.  use_graph selects ogle_rt_compute
@@ -138,7 +145,9 @@ int32_t ogle_rt_launch_plan_entry(OgleSession* s, int32_t i, const char** label,
 int32_t ogle_rt_tensor_shape(OgleSession* s, const char* name, int32_t* dims);
 /* Layout tag of a tensor as a TensorProto.DataFormat value (dlxnet.proto:7-30), or negative. */
 int32_t ogle_rt_tensor_dformat(OgleSession* s, const char* name);
-/* Device address of a tensor's first element (for zero-copy consumers), or NULL. */
+/* Device address of a tensor's first element (for zero-copy consumers), or NULL; NULL too
+ * for a tensor that is not dense on the device (a convolution output produced in its place
+ * inside a concatenation's output at batch > 1: read it with ogle_rt_get_output). */
 void* ogle_rt_tensor_device_ptr(OgleSession* s, const char* name);
 /* The session's hipStream_t. */
 void* ogle_rt_stream(OgleSession* s);

@@ -102,32 +102,71 @@ constexpr int kRegistrySize = sizeof(kRegistry) / sizeof(kRegistry[0]);
 bool positive(int v) { return v > 0; }
 
 const char kSplitNeedsMfma[] =
-    "a second destination (output2_dev) is only supported by the MFMA implicit-GEMM kernels: "
+    "a second destination (output2_dev) and an image stride (out_image_stride) are only "
+    "supported by the MFMA implicit-GEMM kernels: "
     "group 1, in_c % 4 == 0 (fp16: % 8), kernel_size^2 * in_c >= 32";
 
-// launch_conv_direct for the batch entry point: it cannot divide the output.
+// True for arguments only the implicit-GEMM kernels can serve.
+bool needs_mfma(const OgleConvArgs& a) {
+  return a.output2_dev != nullptr ||
+         (a.out_image_stride != 0 && a.out_image_stride != (int64_t)a.out_h * a.out_w * a.out_c);
+}
+
+// launch_conv_direct for the batch entry point: it writes one dense output.
 int32_t direct_no_split(const OgleConvArgs& a, hipStream_t s) {
-  if (a.output2_dev != nullptr) return fail(OGLE_ERR_UNSUPPORTED, kSplitNeedsMfma);
+  if (needs_mfma(a)) return fail(OGLE_ERR_UNSUPPORTED, kSplitNeedsMfma);
   return launch_conv_direct(a, s);
 }
 
-// Byte extents of a convolution's tensors, and interval overlap of two device ranges.
+// Byte extents of a convolution's tensors.  A span is `count` runs of `run` bytes whose
+// starts lie `stride` bytes apart (count 1: one plain range); an output written with
+// out_image_stride is one run per image.
+struct Span {
+  const void* ptr;
+  size_t run, stride;
+  long count;
+};
 size_t elem_bytes(const OgleConvArgs& a) { return a.dtype == OGLE_F16 ? 2 : 4; }
-size_t input_bytes(const OgleConvArgs& a) {
-  return (size_t)a.n * a.in_h * a.in_w * a.in_c * elem_bytes(a);
+Span plain(const void* p, size_t bytes) { return Span{p, bytes, 0, 1}; }
+Span input_span(const OgleConvArgs& a) {
+  return plain(a.input_dev, (size_t)a.n * a.in_h * a.in_w * a.in_c * elem_bytes(a));
 }
-size_t output_bytes(const OgleConvArgs& a) {
+Span output_span(const OgleConvArgs& a) {
   const int c = a.output2_dev != nullptr ? a.out_c_split : a.out_c;
-  return (size_t)a.n * a.out_h * a.out_w * c * elem_bytes(a);
+  const size_t image = (size_t)a.out_h * a.out_w * c * elem_bytes(a);
+  if (a.out_image_stride == 0 || a.n == 1 || (size_t)a.out_image_stride * elem_bytes(a) == image)
+    return plain(a.output_dev, image * a.n);
+  return Span{a.output_dev, image, (size_t)a.out_image_stride * elem_bytes(a), a.n};
 }
-size_t output2_bytes(const OgleConvArgs& a) {
-  if (a.output2_dev == nullptr) return 0;
-  return (size_t)a.n * a.out_h * a.out_w * (a.out_c - a.out_c_split) * elem_bytes(a);
+Span output2_span(const OgleConvArgs& a) {
+  if (a.output2_dev == nullptr) return plain(nullptr, 0);
+  return plain(a.output2_dev,
+               (size_t)a.n * a.out_h * a.out_w * (a.out_c - a.out_c_split) * elem_bytes(a));
 }
-bool overlap(const void* a, size_t a_bytes, const void* b, size_t b_bytes) {
-  if (a == nullptr || b == nullptr || a_bytes == 0 || b_bytes == 0) return false;
-  const uintptr_t a0 = reinterpret_cast<uintptr_t>(a), b0 = reinterpret_cast<uintptr_t>(b);
-  return a0 < b0 + b_bytes && b0 < a0 + a_bytes;
+Span workspace_span(const OgleConvArgs& a) { return plain(a.workspace_dev, a.workspace_bytes); }
+// True if the two spans share a byte.  Two spans of the same stride are compared by where
+// their runs lie inside one period (exact when both cover the same images, otherwise on
+// the safe side); other strided pairs run by run.
+bool overlap(const Span& a, const Span& b) {
+  if (a.ptr == nullptr || b.ptr == nullptr || a.run == 0 || b.run == 0) return false;
+  const uintptr_t a0 = reinterpret_cast<uintptr_t>(a.ptr), b0 = reinterpret_cast<uintptr_t>(b.ptr);
+  const uintptr_t a1 = a0 + (size_t)(a.count - 1) * a.stride + a.run;
+  const uintptr_t b1 = b0 + (size_t)(b.count - 1) * b.stride + b.run;
+  if (!(a0 < b1 && b0 < a1)) return false;
+  if (a.count == 1 && b.count == 1) return true;
+  if (a.count > 1 && b.count > 1) {
+    if (a.stride != b.stride || a.run > a.stride || b.run > b.stride) return true;
+    const size_t d = b0 >= a0 ? (b0 - a0) % a.stride : (a.stride - (a0 - b0) % a.stride) % a.stride;
+    return d < a.run || d + b.run > a.stride;
+  }
+  const Span& many = a.count > 1 ? a : b;
+  const Span& one = a.count > 1 ? b : a;
+  const uintptr_t m0 = reinterpret_cast<uintptr_t>(many.ptr), o0 = reinterpret_cast<uintptr_t>(one.ptr);
+  for (long i = 0; i < many.count; ++i) {
+    const uintptr_t r0 = m0 + (size_t)i * many.stride;
+    if (r0 < o0 + one.run && o0 < r0 + many.run) return true;
+  }
+  return false;
 }
 
 int32_t validate_conv(const OgleConvArgs* a, const char* who) {
@@ -168,6 +207,17 @@ int32_t validate_conv(const OgleConvArgs* a, const char* who) {
     set_error("%s: out_c_split %d must lie strictly between 0 and out_c %d", who, a->out_c_split,
               a->out_c);
     return OGLE_ERR_INVALID_ARG;
+  }
+  if (a->out_image_stride != 0) {
+    if (a->out_image_stride < (int64_t)a->out_h * a->out_w * a->out_c) {
+      set_error("%s: out_image_stride %lld is less than one image's %d x %d x %d outputs", who,
+                (long long)a->out_image_stride, a->out_h, a->out_w, a->out_c);
+      return OGLE_ERR_INVALID_ARG;
+    }
+    if (a->output2_dev != nullptr) {
+      set_error("%s: out_image_stride cannot be combined with output2_dev", who);
+      return OGLE_ERR_INVALID_ARG;
+    }
   }
   if (a->in_c % a->group != 0 || a->out_c % a->group != 0) {
     set_error("%s: channels %d -> %d not divisible by group %d", who, a->in_c, a->out_c, a->group);
@@ -308,6 +358,20 @@ size_t ogle_hip_conv_workspace_bytes(const OgleConvArgs* a) {
   return conv_igemm_workspace_bytes(q);
 }
 
+int32_t ogle_hip_conv_takes_image_stride(const OgleConvArgs* a) {
+  if (a == nullptr) return 0;
+  OgleConvArgs q = *a;  // pointers are not looked at: only shapes are validated
+  static char dummy;
+  q.input_dev = q.filter_dev = &dummy;
+  q.output_dev = &dummy;
+  q.output2_dev = nullptr;
+  q.out_image_stride = 0;
+  q.workspace_dev = nullptr;
+  q.workspace_bytes = 0;
+  if (validate_conv(&q, "conv_takes_image_stride") != OGLE_OK) return 0;
+  return conv_igemm_takes(q) ? 1 : 0;
+}
+
 int32_t ogle_hip_conv2d(const OgleConvArgs* a, ogle_stream_t stream) {
   int32_t st = validate_conv(a, "conv2d");
   if (st != OGLE_OK) return st;
@@ -315,7 +379,7 @@ int32_t ogle_hip_conv2d(const OgleConvArgs* a, ogle_stream_t stream) {
     st = launch_conv_igemm(*a, as_stream(stream));
     if (st != OGLE_ERR_UNSUPPORTED) return st;
   }
-  if (a->output2_dev != nullptr) return fail(OGLE_ERR_UNSUPPORTED, kSplitNeedsMfma);
+  if (needs_mfma(*a)) return fail(OGLE_ERR_UNSUPPORTED, kSplitNeedsMfma);
   return launch_conv_direct(*a, as_stream(stream));
 }
 
@@ -329,7 +393,7 @@ int32_t ogle_hip_conv2d_noalloc(const OgleConvArgs* a, ogle_stream_t stream) {
     st = launch_conv_igemm_static_scratch(*a, as_stream(stream));
     if (st != OGLE_ERR_UNSUPPORTED) return st;
   }
-  if (a->output2_dev != nullptr) return fail(OGLE_ERR_UNSUPPORTED, kSplitNeedsMfma);
+  if (needs_mfma(*a)) return fail(OGLE_ERR_UNSUPPORTED, kSplitNeedsMfma);
   return launch_conv_direct(*a, as_stream(stream));
 }
 
@@ -369,22 +433,17 @@ int32_t conv2d_batch_impl(const OgleConvArgs* args, int32_t count, int32_t* redu
     if (st != OGLE_OK) return st;
     for (int j = 0; j < i; ++j) {
       const OgleConvArgs &p = args[i], &q = args[j];
-      if (overlap(p.input_dev, input_bytes(p), q.output_dev, output_bytes(q)) ||
-          overlap(q.input_dev, input_bytes(q), p.output_dev, output_bytes(p)) ||
-          overlap(p.output_dev, output_bytes(p), q.output_dev, output_bytes(q)))
+      if (overlap(input_span(p), output_span(q)) || overlap(input_span(q), output_span(p)) ||
+          overlap(output_span(p), output_span(q)))
         return fail(OGLE_ERR_INVALID_ARG, "conv2d_batch: the convolutions depend on each other");
-      if (overlap(p.output2_dev, output2_bytes(p), q.input_dev, input_bytes(q)) ||
-          overlap(q.output2_dev, output2_bytes(q), p.input_dev, input_bytes(p)) ||
-          overlap(p.output2_dev, output2_bytes(p), q.output_dev, output_bytes(q)) ||
-          overlap(q.output2_dev, output2_bytes(q), p.output_dev, output_bytes(p)) ||
-          overlap(p.output2_dev, output2_bytes(p), q.output2_dev, output2_bytes(q)))
+      if (overlap(output2_span(p), input_span(q)) || overlap(output2_span(q), input_span(p)) ||
+          overlap(output2_span(p), output_span(q)) || overlap(output2_span(q), output_span(p)) ||
+          overlap(output2_span(p), output2_span(q)))
         return fail(OGLE_ERR_INVALID_ARG, "conv2d_batch: the convolutions depend on each other");
-      if (overlap(p.workspace_dev, p.workspace_bytes, q.workspace_dev, q.workspace_bytes))
+      if (overlap(workspace_span(p), workspace_span(q)))
         return fail(OGLE_ERR_INVALID_ARG, "conv2d_batch: two convolutions share one workspace");
-      if (overlap(p.workspace_dev, p.workspace_bytes, q.output_dev, output_bytes(q)) ||
-          overlap(q.workspace_dev, q.workspace_bytes, p.output_dev, output_bytes(p)) ||
-          overlap(p.workspace_dev, p.workspace_bytes, q.input_dev, input_bytes(q)) ||
-          overlap(q.workspace_dev, q.workspace_bytes, p.input_dev, input_bytes(p)))
+      if (overlap(workspace_span(p), output_span(q)) || overlap(workspace_span(q), output_span(p)) ||
+          overlap(workspace_span(p), input_span(q)) || overlap(workspace_span(q), input_span(p)))
         return fail(OGLE_ERR_INVALID_ARG,
                     "conv2d_batch: a workspace overlaps another convolution's tensor");
     }
@@ -401,7 +460,7 @@ int32_t ogle_hip_dwconv2d(const OgleConvArgs* a, ogle_stream_t stream) {
     set_error("dwconv2d: group %d must equal in_c %d and out_c %d", a->group, a->in_c, a->out_c);
     return OGLE_ERR_INVALID_ARG;
   }
-  if (a->output2_dev != nullptr) return fail(OGLE_ERR_UNSUPPORTED, kSplitNeedsMfma);
+  if (needs_mfma(*a)) return fail(OGLE_ERR_UNSUPPORTED, kSplitNeedsMfma);
   return launch_conv_dw(*a, as_stream(stream));
 }
 
@@ -416,7 +475,7 @@ int32_t ogle_hip_pwconv_gemm(const OgleConvArgs* a, ogle_stream_t stream) {
   }
   st = launch_conv_igemm(*a, as_stream(stream));
   if (st != OGLE_ERR_UNSUPPORTED) return st;
-  if (a->output2_dev != nullptr) return fail(OGLE_ERR_UNSUPPORTED, kSplitNeedsMfma);
+  if (needs_mfma(*a)) return fail(OGLE_ERR_UNSUPPORTED, kSplitNeedsMfma);
   return launch_conv_direct(*a, as_stream(stream));
 }
 

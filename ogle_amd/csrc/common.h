@@ -103,6 +103,7 @@ __device__ __forceinline__ int xcd_swizzle(int pid, int grid) {
 // Launchers implemented in the .hip files (host side).
 int32_t launch_conv_igemm(const OgleConvArgs& a, hipStream_t s);   // returns OGLE_ERR_UNSUPPORTED if shape not eligible
 size_t conv_igemm_workspace_bytes(const OgleConvArgs& a);
+bool conv_igemm_takes(const OgleConvArgs& a);  // launch_conv_igemm would not return OGLE_ERR_UNSUPPORTED
 int32_t launch_conv_igemm_static_scratch(const OgleConvArgs& a, hipStream_t s);
 // reduce_pending != nullptr: split-K reductions are not launched; reduce_pending[i] says
 // whether convolution i still needs launch_conv_reduce.

@@ -47,7 +47,17 @@ struct ConvGeom {
   int ktiles;    // taps * cchunks
   unsigned x_bytes;  // size of the input tensor (buffer-load range)
   unsigned w_bytes;  // size of the packed filter
+  long oimg;         // elements between the outputs of consecutive images; 0: dense
 };
+
+// Element offset of output row `row` (= (image, oy, ox) flattened) whose channels are
+// `pitch` apart per row: dense, or with a gap after every image's oh * ow rows.
+__device__ __forceinline__ long out_row_offset(const ConvGeom& g, int row, int pitch) {
+  if (g.oimg == 0) return (long)row * pitch;
+  const int hw = g.oh * g.ow;
+  const int b = row / hw;
+  return (long)b * g.oimg + (long)(row - b * hw) * pitch;
+}
 
 template <typename T>
 struct Mma;
@@ -340,7 +350,7 @@ __device__ __forceinline__ void igemm_tile(
   constexpr int CW = JC * 32;              // columns staged at once
   constexpr int SROW = CW + 4;             // floats per staged row (padded)
   float* const smw = reinterpret_cast<float*>(lds) + wave * 32 * SROW;
-  if (pdst != nullptr || (sizeof(T) == 4 && (o1 & 3) == 0 && (o2 & 3) == 0)) {
+  if (pdst != nullptr || (sizeof(T) == 4 && (o1 & 3) == 0 && (o2 & 3) == 0 && (g.oimg & 3) == 0)) {
     constexpr int LPR = CW / 4;              // lanes covering one staged row
     constexpr int RPI = 64 / LPR;            // rows one store instruction covers
     const int cv = lane % LPR;
@@ -375,7 +385,8 @@ __device__ __forceinline__ void igemm_tile(
               v.z = apply_epilogue(v.z + bias4.z, ep);
               v.w = apply_epilogue(v.w + bias4.w, ep);
             }
-            *reinterpret_cast<float4*>(dbase + (long)grow * dpitch + dcol) = v;
+            const long at = pdst != nullptr ? (long)grow * dpitch : out_row_offset(g, grow, dpitch);
+            *reinterpret_cast<float4*>(dbase + at + dcol) = v;
           }
         }
       }
@@ -383,7 +394,7 @@ __device__ __forceinline__ void igemm_tile(
     return;
   }
   if constexpr (sizeof(T) == 2) {
-    if ((g.o & 7) == 0 && y2 == nullptr) {
+    if ((g.o & 7) == 0 && y2 == nullptr && (g.oimg & 7) == 0) {
       // fp16 output: the same staging, a lane then takes eight consecutive channels
       // of a row and stores them as one 16-byte vector of halves
       constexpr int LPR = CW / 8;
@@ -423,7 +434,7 @@ __device__ __forceinline__ void igemm_tile(
               for (int q = 0; q < 4; ++q)
                 h[q] = __floats2half2_rn(apply_epilogue(f[2 * q] + bias8[2 * q], ep),
                                          apply_epilogue(f[2 * q + 1] + bias8[2 * q + 1], ep));
-              *reinterpret_cast<uint4*>(reinterpret_cast<__half*>(y) + (long)grow * g.o + col) = packed;
+              *reinterpret_cast<uint4*>(reinterpret_cast<__half*>(y) + out_row_offset(g, grow, g.o) + col) = packed;
             }
           }
         }
@@ -449,7 +460,7 @@ __device__ __forceinline__ void igemm_tile(
         if (pdst != nullptr) {
           pdst[(long)row * opitch + col] = acc[i][j][r];
         } else {
-          dst[(long)row * dpitch] = from_f32<T>(apply_epilogue(acc[i][j][r] + bv, ep));
+          dst[out_row_offset(g, row, dpitch)] = from_f32<T>(apply_epilogue(acc[i][j][r] + bv, ep));
         }
       }
     }
@@ -789,8 +800,8 @@ __device__ __forceinline__ void igemm_wave_tile(
     }
     return;
   }
-  T* dst = y + (long)grow * g.o + gcol;
-  if ((g.o & 3) == 0) {
+  T* dst = y + out_row_offset(g, grow, g.o) + gcol;
+  if ((g.o & 3) == 0 && (g.oimg & 3) == 0) {
     if constexpr (sizeof(T) == 4) {
       *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
     } else {
@@ -824,6 +835,8 @@ struct ReduceProblem {
   int o, o1, opitch, splits;
   Epilogue ep;
   int lanes;  // lanes per output element (1, 2, 4 or 8)
+  long oimg;  // elements between the outputs of consecutive images in y; 0: dense
+  int hw;     // output rows per image
 };
 struct ReduceGroup {
   int count;
@@ -855,7 +868,10 @@ __device__ __forceinline__ void splitk_reduce_block(const ReduceProblem& r, int 
   if (live && q == 0) {
     if (r.bias != nullptr) acc += r.bias[col];
     const T out = from_f32<T>(apply_epilogue(acc, r.ep));
-    if (col < r.o1) static_cast<T*>(r.y)[row * r.o1 + col] = out;
+    if (r.oimg != 0) {
+      const long b = row / r.hw;
+      static_cast<T*>(r.y)[b * r.oimg + (row - b * r.hw) * r.o + col] = out;
+    } else if (col < r.o1) static_cast<T*>(r.y)[row * r.o1 + col] = out;
     else static_cast<T*>(r.y2)[row * (r.o - r.o1) + (col - r.o1)] = out;
   }
 }
@@ -1112,6 +1128,7 @@ Prepared prepare(const OgleConvArgs& a, long m, const IgemmPlan& p) {
   const long esz = a.dtype == OGLE_F16 ? 2 : 4;
   g.x_bytes = (unsigned)((long)a.n * a.in_h * a.in_w * a.in_c * esz);
   g.w_bytes = (unsigned)((long)a.out_c * a.kernel_size * a.kernel_size * a.in_c * esz);
+  g.oimg = a.out_image_stride == (long)a.out_h * a.out_w * a.out_c ? 0 : a.out_image_stride;
   const int tiles_m = (g.m_total + tile_bm(p.cfg) - 1) / tile_bm(p.cfg);
   const int tiles_n = (g.o + tile_bn(p.cfg) - 1) / tile_bn(p.cfg);
   out.prob.x = a.input_dev;
@@ -1139,7 +1156,8 @@ Prepared prepare(const OgleConvArgs& a, long m, const IgemmPlan& p) {
     int lanes = 1;
     while (lanes < 8 && lanes * 2 <= p.splits && mn * lanes < 64L * 1024) lanes *= 2;
     out.red = ReduceProblem{out.prob.partial, a.bias_dev, a.output_dev, a.output2_dev, mn, g.o,
-                            out.prob.o1, (g.o + 3) & ~3, p.splits, out.prob.ep, lanes};
+                            out.prob.o1, (g.o + 3) & ~3, p.splits, out.prob.ep, lanes, g.oimg,
+                            g.oh * g.ow};
     out.reduce_lanes = lanes;
     out.reduce_grid = (unsigned)((mn * lanes + 255) / 256);
   }
@@ -1226,6 +1244,11 @@ void launch_reduce_single(const Prepared& pr, hipStream_t s) {
 }
 
 }  // namespace
+
+bool conv_igemm_takes(const OgleConvArgs& a) {
+  long m = 0;
+  return igemm_eligible(a, &m);
+}
 
 size_t conv_igemm_workspace_bytes(const OgleConvArgs& a) {
   long m = 0;

@@ -31,6 +31,7 @@ SYMBOLS = [
     "ogle_hip_conv2d_noalloc", "ogle_hip_launch_count",
     "ogle_hip_conv2d_batch_begin", "ogle_hip_conv2d_batch_finish",
     "ogle_hip_kernel_timing_begin", "ogle_hip_kernel_timing_end",
+    "ogle_hip_conv_takes_image_stride",
 ]
 CONV_NOALLOC_SCRATCH_BYTES = 16 << 20
 UNARY_RELU, UNARY_CLIP = 0, 1
@@ -55,6 +56,7 @@ class ConvArgs(ctypes.Structure):
         ("act_variant", ctypes.c_int32), ("dtype", ctypes.c_int32),
         ("workspace_dev", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
         ("output2_dev", ctypes.c_void_p), ("out_c_split", ctypes.c_int32),
+        ("out_image_stride", ctypes.c_int64),
     ]
 
 
@@ -190,6 +192,7 @@ def lib():
         l.ogle_hip_conv2d_batch_finish.argtypes = [ctypes.POINTER(ConvArgs), ctypes.c_int32, ctypes.c_void_p]
         l.ogle_hip_conv_workspace_bytes.argtypes = [ctypes.POINTER(ConvArgs)]
         l.ogle_hip_conv_workspace_bytes.restype = ctypes.c_size_t
+        l.ogle_hip_conv_takes_image_stride.argtypes = [ctypes.POINTER(ConvArgs)]
         l.ogle_hip_gemm_workspace_bytes.argtypes = [ctypes.POINTER(GemmArgs)]
         l.ogle_hip_gemm_workspace_bytes.restype = ctypes.c_size_t
         l.ogle_hip_expf.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64,
@@ -230,4 +233,4 @@ def conv_args(x_ptr, w_ptr, b_ptr, y_ptr, n, h, w, c, o, k, stride=1, pad=0, dil
               act=ACT_NONE, minv=0.0, maxv=0.0, variant=VARIANT_NHWC4, dtype=F32):
     return ConvArgs(x_ptr, w_ptr, b_ptr, y_ptr, n, h, w, c,
                     out_size(h, k, stride, pad, dilation), out_size(w, k, stride, pad, dilation), o,
-                    k, stride, pad, dilation, group, act, minv, maxv, variant, dtype, None, 0, None, 0)
+                    k, stride, pad, dilation, group, act, minv, maxv, variant, dtype, None, 0, None, 0, 0)

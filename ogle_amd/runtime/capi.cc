@@ -120,6 +120,14 @@ int32_t ogle_rt_hazard_conflicts(const OgleConvArgs* pending, int32_t n_pending,
              : 0;
 }
 
+int32_t ogle_rt_conv_hazard_conflicts(const OgleConvArgs* pending, int32_t n_pending,
+                                      const OgleConvArgs* next) {
+  if (n_pending < 0 || next == nullptr || (n_pending > 0 && pending == nullptr)) return -1;
+  opengl::MemRange reads[3], writes[3];
+  opengl::Context::ConvRanges(*next, reads, writes);
+  return opengl::Context::Conflicts(pending, n_pending, reads, 3, writes, 3) ? 1 : 0;
+}
+
 int32_t ogle_rt_run(OgleSession* s, int32_t n_inputs, const char* const* names,
                     const float* const* data, const int32_t* const* dims, const int32_t* ranks,
                     const char* const* dformats) {
@@ -373,7 +381,7 @@ void* ogle_rt_tensor_device_ptr(OgleSession* s, const char* name) {
   void* p = nullptr;
   Guard([&]() -> int64_t {
     Tensor* t = s->session->FindTensorByName(name);
-    p = t ? t->device_ptr() : nullptr;
+    p = t && t->outer_stride_bytes() == 0 ? t->device_ptr() : nullptr;
     return 0;
   });
   return p;

@@ -62,10 +62,29 @@ void* Context::Workspace(size_t bytes) {
 
 namespace {
 size_t ElemBytes(const OgleConvArgs& a) { return a.dtype == OGLE_F16 ? 2 : 4; }
+// True if the two ranges share a byte.  Two strided ranges of the same stride are compared
+// by where their runs lie inside one period (exact when both cover the same slices, on the
+// safe side otherwise), any other strided pair run by run.
 bool Overlap(const MemRange& a, const MemRange& b) {
   if (a.ptr == nullptr || b.ptr == nullptr || a.bytes == 0 || b.bytes == 0) return false;
   const uintptr_t a0 = reinterpret_cast<uintptr_t>(a.ptr), b0 = reinterpret_cast<uintptr_t>(b.ptr);
-  return a0 < b0 + b.bytes && b0 < a0 + a.bytes;
+  const uintptr_t a1 = a0 + (a.count - 1) * a.stride + a.bytes;
+  const uintptr_t b1 = b0 + (b.count - 1) * b.stride + b.bytes;
+  if (!(a0 < b1 && b0 < a1)) return false;
+  if (a.count <= 1 && b.count <= 1) return true;
+  if (a.count > 1 && b.count > 1) {
+    if (a.stride != b.stride || a.bytes > a.stride || b.bytes > b.stride) return true;
+    const size_t d = b0 >= a0 ? (b0 - a0) % a.stride : (a.stride - (a0 - b0) % a.stride) % a.stride;
+    return d < a.bytes || d + b.bytes > a.stride;
+  }
+  const MemRange& many = a.count > 1 ? a : b;
+  const MemRange& one = a.count > 1 ? b : a;
+  const uintptr_t m0 = reinterpret_cast<uintptr_t>(many.ptr), o0 = reinterpret_cast<uintptr_t>(one.ptr);
+  for (size_t i = 0; i < many.count; ++i) {
+    const uintptr_t r0 = m0 + i * many.stride;
+    if (r0 < o0 + one.bytes && o0 < r0 + many.bytes) return true;
+  }
+  return false;
 }
 }  // namespace
 
@@ -79,6 +98,10 @@ void Context::ConvRanges(const OgleConvArgs& c, MemRange reads[3], MemRange writ
   const size_t pixels = static_cast<size_t>(c.n) * c.out_h * c.out_w;
   const int first = c.output2_dev != nullptr ? c.out_c_split : c.out_c;
   writes[0] = {c.output_dev, pixels * first * esz};
+  const size_t image = static_cast<size_t>(c.out_h) * c.out_w * first * esz;
+  if (c.out_image_stride != 0 && c.n > 1 && static_cast<size_t>(c.out_image_stride) * esz != image)
+    writes[0] = {c.output_dev, image, static_cast<size_t>(c.out_image_stride) * esz,
+                 static_cast<size_t>(c.n)};
   writes[1] = {c.workspace_dev, c.workspace_dev != nullptr ? c.workspace_bytes : 0};
   writes[2] = {c.output2_dev, c.output2_dev != nullptr ? pixels * (c.out_c - first) * esz : 0};
 }
@@ -349,6 +372,7 @@ void Context::CopyCPUTensorToDevice(const Tensor* cpu, Tensor* dev) {
   CHECK(cpu->is_host()) << "source must be a host tensor";
   CHECK(dev->mem_type() != Tensor::HOST_MEMORY) << "destination must be a device tensor";
   CHECK_EQ(cpu->num_elements(), dev->num_elements());
+  CHECK_EQ(dev->outer_stride_bytes(), 0u) << "upload into a tensor that lies inside another one";
   const size_t bytes = cpu->num_elements() * sizeof(float);
   if (bytes == 0) return;
   Flush();
@@ -368,6 +392,22 @@ void Context::CopyCPUTensorToDevice(const Tensor* cpu, Tensor* dev) {
   OGLE_HIP_CALL(hipStreamSynchronize(s));
   dev->set_initialized(true);
 }
+
+namespace {
+// Device -> host copy of a tensor's elements in dense order, whether or not its runs lie
+// apart on the device.
+void ReadDense(const Tensor* dev, void* dst, hipStream_t s) {
+  const size_t bytes = dev->num_elements() * sizeof(float);
+  const size_t stride = dev->outer_stride_bytes();
+  if (stride == 0) {
+    OGLE_HIP_CALL(hipMemcpyAsync(dst, dev->device_ptr(), bytes, hipMemcpyDeviceToHost, s));
+    return;
+  }
+  const size_t run = bytes / dev->outer_count();
+  OGLE_HIP_CALL(hipMemcpy2DAsync(dst, run, dev->device_ptr(), stride, run, dev->outer_count(),
+                                 hipMemcpyDeviceToHost, s));
+}
+}  // namespace
 
 void Context::CopyDeviceTensorToCPU(const Tensor* dev, Tensor* cpu) {
   CHECK(cpu->is_host()) << "destination must be a host tensor";
@@ -389,18 +429,18 @@ void Context::CopyDeviceTensorToCPU(const Tensor* dev, Tensor* cpu) {
       CHECK(dev->dformat() == dlxnet::TensorProto::HWN4C4)
           << "HWN4C4 readback of a tensor that is not a filter (" << FormatToStr(dev->dformat()) << ")";
     std::vector<float> dense(dev->num_elements());
-    OGLE_HIP_CALL(hipMemcpyAsync(dense.data(), dev->device_ptr(), bytes, hipMemcpyDeviceToHost, s));
+    ReadDense(dev, dense.data(), s);
     OGLE_HIP_CALL(hipStreamSynchronize(s));
     std::memset(cpu->host(), 0, cpu->AllocatedSize());
     PaddedIndexWalk(dev->shape(), cpu->dformat(), dense.data(), cpu->host<float>(), true);
   } else if (cpu->dformat() == dlxnet::TensorProto::NCHW && IsImageTag(dev->dformat())) {
     CHECK_EQ(dev->dims_size(), 4);
     std::vector<float> tmp(dev->num_elements());
-    OGLE_HIP_CALL(hipMemcpyAsync(tmp.data(), dev->device_ptr(), bytes, hipMemcpyDeviceToHost, s));
+    ReadDense(dev, tmp.data(), s);
     OGLE_HIP_CALL(hipStreamSynchronize(s));
     Permute4(tmp.data(), cpu->host<float>(), dev->shape(), false);
   } else {
-    OGLE_HIP_CALL(hipMemcpyAsync(cpu->host(), dev->device_ptr(), bytes, hipMemcpyDeviceToHost, s));
+    ReadDense(dev, cpu->host(), s);
     OGLE_HIP_CALL(hipStreamSynchronize(s));
   }
   cpu->set_initialized(true);

@@ -14,10 +14,14 @@
 
 namespace opengl {
 
-// A byte range of device memory, [ptr, ptr + bytes).
+// A byte range of device memory, [ptr, ptr + bytes); with count > 1, that many ranges of
+// `bytes` whose starts lie `stride` bytes apart (a convolution output written one image at
+// a time into a larger tensor).
 struct MemRange {
   const void* ptr;
   size_t bytes;
+  size_t stride = 0;
+  size_t count = 1;
 };
 
 class Context {

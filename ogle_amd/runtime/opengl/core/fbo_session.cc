@@ -181,15 +181,20 @@ void FBOSession::FuseSiblings() {
   }
 }
 
-// Where a node's output is nothing but its inputs back to back (a Concat with a single
-// slice before its axis: the SSD box and class concats at batch 1), the producers of
-// those inputs are pointed at their places inside the output, so that the node has
-// nothing left to copy (ogle_hip_concat then launches nothing).  An input qualifies if,
-// looking through nodes that only re-interpret memory, it is the whole output of a live
-// node with its own allocation that has not been placed already; its place must be
-// 16-byte aligned unless the producer is a convolution whose channel count is not a
-// multiple of four (those store element by element).  All inputs of the node must
-// qualify.  Every tensor that aliases a moved allocation is re-pointed with it.
+// Where a node's output is nothing but its inputs side by side (Kernel::
+// InputPlacementInOutput: a Concat), the producers of those inputs are pointed at their
+// places inside the output, so that the node has nothing left to copy.  With a single
+// slice before the concat axis (the SSD box and class concats at batch 1) an input's place
+// is one dense range; with several (the same concats at batch > 1) it is one run per
+// slice, the runs a whole output slice apart, and the producer must be able to write its
+// images that far apart (Kernel::CanWriteOuterSlicesApart: a convolution on the MFMA
+// path) and be read by nothing but this node, since every other kernel assumes dense
+// inputs.  An input qualifies if, looking through nodes that only re-interpret memory, it
+// is the whole output of a live node with its own allocation that has not been placed
+// already; its place (and the distance between runs) must be 16-byte aligned unless the
+// producer is a convolution whose channel count is not a multiple of four (those store
+// element by element).  All inputs of the node must qualify.  Every tensor that aliases
+// a moved allocation is re-pointed with it.
 void FBOSession::PlaceInputsInOutputs() {
   std::map<int, std::pair<Kernel*, int>> producer;  // tensor index -> (kernel, output slot)
   for (auto& k : kernels_)
@@ -223,10 +228,12 @@ void FBOSession::PlaceInputsInOutputs() {
   for (auto& kp : kernels_) {
     Kernel* k = kp.get();
     if (CheckKernelReady(k)) continue;
-    const std::vector<size_t> offsets = k->InputOffsetsInOutput();
+    const Kernel::Placement pl = k->InputPlacementInOutput();
+    const std::vector<size_t>& offsets = pl.offsets;
     if (offsets.empty() || offsets.size() != k->input_tensor_indexes_.size()) continue;
     Tensor* out = k->output_tensors_[0];
     if (!out->owns_device_buffer()) continue;
+    const bool apart = pl.outer_count > 1;
     std::vector<int> roots;
     bool ok = true;
     for (size_t i = 0; i < offsets.size() && ok; ++i) {
@@ -246,12 +253,14 @@ void FBOSession::PlaceInputsInOutputs() {
       // A place that is only 4-byte aligned suits a convolution that stores element by
       // element, but every other kernel reads 16-byte vectors from the tensor's start:
       // the exception holds only if this node is the allocation's sole reader.
-      const bool by_element = pk->kernel_type() == "Conv" && root->shape().back() % 4 != 0 &&
-                              !has_other_reader(idx, k);
+      const bool sole = !has_other_reader(idx, k);
+      const bool by_element = pk->kernel_type() == "Conv" && root->shape().back() % 4 != 0 && sole;
+      const bool aligned = place % 16 == 0 && (!apart || pl.outer_stride % 16 == 0);
       ok = !CheckKernelReady(pk) && root->owns_device_buffer() && placed.count(idx) == 0 &&
            std::find(roots.begin(), roots.end(), idx) == roots.end() &&
            root->num_elements() == k->input_tensors_[i]->num_elements() &&
-           (place % 16 == 0 || (by_element && place % 4 == 0));
+           (aligned || (by_element && place % 4 == 0 && pl.outer_stride % 4 == 0)) &&
+           (!apart || (sole && pk->CanWriteOuterSlicesApart(pl.outer_count)));
       roots.push_back(idx);
     }
     if (!ok) continue;
@@ -262,10 +271,11 @@ void FBOSession::PlaceInputsInOutputs() {
       for (auto& t : total_tensors_)
         if (t && t.get() != root && t->mem_type() == Tensor::DEVICE_BUFFER &&
             !t->owns_device_buffer() && t->device_ptr() == old)
-          t->Rebind(place);
-      root->Rebind(place);
+          t->Rebind(place, pl.outer_count, pl.outer_stride);
+      root->Rebind(place, pl.outer_count, pl.outer_stride);
       placed.insert(roots[i]);
     }
+    k->set_inputs_in_place(true);
   }
 }
 

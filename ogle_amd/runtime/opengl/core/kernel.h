@@ -61,14 +61,33 @@ class Kernel {
   // re-interpretation of dense memory), or -1.  Not in the reference, where every
   // layout change is a draw call; with linear NHWC buffers Reshape and an identity
   // Transpose move no data.  Consulted by the executor after InferOutputShape.
-// If output 0 is nothing but the inputs placed back to back, the byte offset of
-  // every input inside it (the session may then have the inputs produced in place);
-  // empty otherwise.  Valid after InferOutputShape.
-  virtual std::vector<size_t> InputOffsetsInOutput() const { return {}; }
-    virtual int OutputAliasesInput(int i) const {
+  virtual int OutputAliasesInput(int i) const {
     (void)i;
     return -1;
   }
+
+  // If output 0 is nothing but the inputs placed side by side, where every input lies
+  // inside it (the session may then have the inputs produced in place, and the node has
+  // nothing left to copy); `offsets` empty otherwise.  The output is `outer_count` slices
+  // of `outer_stride` bytes, and input i fills bytes [offsets[i], offsets[i] + its size /
+  // outer_count) of every slice: one slice for a concatenation over the first axis that
+  // is not 1, one per image for the SSD concatenations over axis 1 at batch > 1.  Valid
+  // after InferOutputShape.
+  struct Placement {
+    std::vector<size_t> offsets;
+    size_t outer_count = 1;
+    size_t outer_stride = 0;
+  };
+  virtual Placement InputPlacementInOutput() const { return {}; }
+  // True if this node can write output 0 as `count` equal runs whose starts lie further
+  // apart than a run is long (Tensor::outer_stride_bytes) instead of densely.
+  virtual bool CanWriteOuterSlicesApart(size_t count) const {
+    (void)count;
+    return false;
+  }
+  // Set by the session once every input has been placed inside output 0.
+  void set_inputs_in_place(bool v) { inputs_in_place_ = v; }
+  bool inputs_in_place() const { return inputs_in_place_; }
 
   // Sibling fusion, not in the reference: two nodes that read the same tensor with the
   // same attributes may run as one launch that fetches the input once (the box and the
@@ -108,6 +127,7 @@ class Kernel {
   std::string build_options_;
   FBOSession* session_ = nullptr;
   Kernel* absorbed_by_ = nullptr;  // the sibling that does this node's work, if any
+  bool inputs_in_place_ = false;
 };
 
 }  // namespace opengl

@@ -86,12 +86,15 @@ Tensor::Tensor(const Tensor* other, IntList shape, DataFormat dformat)
   allocated_size_ = other->AllocatedSize();
 }
 
-void Tensor::Rebind(void* ptr) {
+void Tensor::Rebind(void* ptr, size_t outer_count, size_t outer_stride) {
   CHECK(mem_type_ != HOST_MEMORY && device_ != nullptr) << "only device tensors can be rebound";
   DeviceBuffer* buf = device<DeviceBuffer>();
   if (buf->owned && buf->ptr != nullptr) (void)hipFree(buf->ptr);
   buf->ptr = ptr;
   buf->owned = false;
+  const bool apart = outer_count > 1 && outer_stride * outer_count != num_elements() * sizeof(float);
+  buf->outer_count = apart ? outer_count : 1;
+  buf->outer_stride = apart ? outer_stride : 0;
 }
 
 Tensor::~Tensor() {

@@ -23,6 +23,12 @@ struct DeviceBuffer {
   void* ptr = nullptr;
   size_t bytes = 0;
   bool owned = true;  // false for a view that aliases another tensor's buffer
+  // Dense unless outer_count > 1: then the tensor's elements are outer_count equal runs
+  // (one per index of the first dimension) whose starts lie outer_stride bytes apart,
+  // i.e. the tensor sits inside a larger one (a convolution output produced in its place
+  // inside a concatenation's output).
+  size_t outer_count = 1;
+  size_t outer_stride = 0;
 };
 
 class Tensor {
@@ -70,8 +76,14 @@ class Tensor {
   // True when this tensor's device memory is its own allocation (not a view).
   bool owns_device_buffer() const { return device_ != nullptr && device<DeviceBuffer>()->owned; }
   // Makes this device tensor a view of memory owned elsewhere, starting at `ptr`
-  // (its own allocation, if any, is released).  The contents are not moved.
-  void Rebind(void* ptr);
+  // (its own allocation, if any, is released).  The contents are not moved.  With
+  // outer_count > 1 the view is that many equal runs, outer_stride bytes apart.
+  void Rebind(void* ptr, size_t outer_count = 1, size_t outer_stride = 0);
+  // 0 for a dense tensor, else the distance between the runs (see DeviceBuffer).
+  size_t outer_stride_bytes() const {
+    return device_ && device<DeviceBuffer>()->outer_count > 1 ? device<DeviceBuffer>()->outer_stride : 0;
+  }
+  size_t outer_count() const { return device_ ? device<DeviceBuffer>()->outer_count : 1; }
 
   const IntList& shape() const { return shape_; }
   size_t num_elements() const;

@@ -41,23 +41,28 @@ void ConcatKernel::InferOutputShape(const TensorList& input_tensors, TensorShape
   }
 }
 
-// With a single slice before the axis (batch 1 on axis 1, or axis 0) the output is the
-// inputs back to back.
-std::vector<size_t> ConcatKernel::InputOffsetsInOutput() const {
-  if (input_tensors_.empty() || output_tensors_.empty()) return {};
+// The output is outer (product of the dimensions before the axis) slices, each the
+// inputs' slices back to back.
+Kernel::Placement ConcatKernel::InputPlacementInOutput() const {
+  Placement pl;
+  if (input_tensors_.empty() || output_tensors_.empty()) return pl;
   const IntList& out = output_tensors_[0]->shape();
-  for (int d = 0; d < axis_; ++d)
-    if (out[d] != 1) return {};
-  std::vector<size_t> offsets;
+  size_t outer = 1, inner = sizeof(float);
+  for (int d = 0; d < axis_; ++d) outer *= out[d];
+  for (size_t d = axis_ + 1; d < out.size(); ++d) inner *= out[d];
+  if (outer == 0) return pl;
   size_t at = 0;
   for (const Tensor* t : input_tensors_) {
-    offsets.push_back(at);
-    at += t->num_elements() * sizeof(float);
+    pl.offsets.push_back(at);
+    at += static_cast<size_t>(t->shape()[axis_]) * inner;
   }
-  return offsets;
+  pl.outer_count = outer;
+  pl.outer_stride = outer > 1 ? at : 0;
+  return pl;
 }
 
 void ConcatKernel::Compute(TensorList& inputs, TensorList& outputs) {
+  if (inputs_in_place()) return;  // every producer wrote straight into the output
   program_->Activate();
   const IntList& out = outputs[0]->shape();
   OgleConcatArgs a{};

@@ -14,7 +14,7 @@ class ConcatKernel : public Kernel {
   void InferOutputShape(TensorShapeList&, TensorShapeList&) override {}
   void SetupAttr(const dlxnet::Attribute& attr) override;
   void SelectKernel(const TensorList& inputs) override;
-  std::vector<size_t> InputOffsetsInOutput() const override;
+  Placement InputPlacementInOutput() const override;
 
  private:
   int axis_ = 0;

@@ -206,6 +206,18 @@ size_t Conv2DKernel::ScratchBytes() const {
   return static_cast<size_t>(workspace_need_);
 }
 
+// One run per image (OgleConvArgs.out_image_stride): only the kernels the library says
+// take it, and not a pair of fused siblings (two destinations).
+bool Conv2DKernel::CanWriteOuterSlicesApart(size_t count) const {
+  if (input_tensors_.empty() || output_tensors_.empty() || sibling_ != nullptr || absorbed()) return false;
+  if (variant_ == kDepthwise) return false;
+  const IntList& out = output_tensors_[0]->shape();
+  if (out.size() != 4 || static_cast<size_t>(out[0]) != count) return false;
+  OgleConvArgs a{};
+  FillGeometry(input_tensors_[0], output_tensors_[0], &a);
+  return ogle_hip_conv_takes_image_stride(&a) == 1;
+}
+
 double Conv2DKernel::WorkEstimate() const {
   if (input_tensors_.empty() || output_tensors_.empty() || absorbed()) return 0.0;
   const IntList& in = input_tensors_[0]->shape();
@@ -229,6 +241,7 @@ void Conv2DKernel::Compute(TensorList& inputs, TensorList& outputs) {
   a.filter_dev = packed_filter_->device_ptr();
   a.bias_dev = inputs.size() > 2 ? static_cast<const float*>(inputs[2]->device_ptr()) : nullptr;
   a.output_dev = outputs[0]->device_ptr();
+  a.out_image_stride = static_cast<int64_t>(outputs[0]->outer_stride_bytes() / sizeof(float));
   if (sibling_ != nullptr) {
     a.output2_dev = sibling_->output_tensors_[0]->device_ptr();
     if (fused_bias_) a.bias_dev = static_cast<const float*>(fused_bias_->device_ptr());

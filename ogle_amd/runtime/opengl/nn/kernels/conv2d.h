@@ -23,6 +23,7 @@ class Conv2DKernel : public Kernel {
   bool TryAbsorb(Kernel* other) override;
   double WorkEstimate() const override;
   size_t ScratchBytes() const override;
+  bool CanWriteOuterSlicesApart(size_t count) const override;
 
  private:
   enum Variant { kDense, kDepthwise, kPointwise, kGrouped };

@@ -26,6 +26,7 @@ SYMBOLS = [
     "ogle_rt_set_reorder", "ogle_rt_issue_order_name", "ogle_rt_set_device_nms",
     "ogle_rt_detect_results", "ogle_rt_graph_captured", "ogle_rt_hazard_conflicts",
     "ogle_rt_set_fuse_siblings", "ogle_rt_launch_plan", "ogle_rt_launch_plan_entry",
+    "ogle_rt_conv_hazard_conflicts",
 ]
 
 
@@ -66,6 +67,8 @@ def lib():
         l.ogle_rt_hazard_conflicts.argtypes = [
             ctypes.POINTER(_hip.ConvArgs), i32, ctypes.POINTER(vp), ctypes.POINTER(ctypes.c_size_t),
             i32, ctypes.POINTER(vp), ctypes.POINTER(ctypes.c_size_t), i32]
+        l.ogle_rt_conv_hazard_conflicts.argtypes = [ctypes.POINTER(_hip.ConvArgs), i32,
+                                                    ctypes.POINTER(_hip.ConvArgs)]
         l.ogle_rt_time_compute.argtypes = [vp, i32, i32, i32, i32, i32,
                                            ctypes.POINTER(ctypes.c_float),
                                            ctypes.POINTER(ctypes.c_float)]
@@ -148,6 +151,12 @@ def hazard_conflicts(pending, reads, writes):
     wp, wb = split(writes)
     return bool(_check(lib().ogle_rt_hazard_conflicts(arr, len(pending), rp, rb, len(reads), wp, wb,
                                                       len(writes))))
+
+
+def conv_hazard_conflicts(pending, nxt):
+    """The same rule with a convolution (hip.ConvArgs) as the next launch."""
+    arr = (_hip.ConvArgs * max(1, len(pending)))(*pending)
+    return bool(_check(lib().ogle_rt_conv_hazard_conflicts(arr, len(pending), ctypes.byref(nxt))))
 
 
 def registered_kernels():

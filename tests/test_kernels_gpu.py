@@ -175,6 +175,60 @@ def test_conv_wave_split_kernel(case, dtype):
         assert_conv_close(got, ref, scale, FP16_RTOL if dtype == H.F16 else FP32_RTOL, str(case))
 
 
+# (n, h, w, c, o, k, stride, pad, image stride beyond the image's own outputs, lead)
+IMAGE_STRIDE_CASES = [
+    (16, 19, 19, 512, 12, 3, 1, 1, 2000, 0),     # box head: split-K + reduce, 16-byte rows
+    (16, 19, 19, 512, 63, 3, 1, 1, 40257 - 22743, 0),   # class head: odd stride, stores by element
+    (4, 10, 10, 256, 24, 3, 1, 1, 36, 24),       # small map: wave-split kernel or short split
+    (3, 5, 5, 64, 126, 3, 1, 1, 1, 7),           # 16x16 tiles, everything unaligned
+    (2, 38, 38, 128, 64, 1, 1, 0, 64, 128),      # pointwise, no split: the tile kernel's row stores
+    (64, 10, 10, 256, 24, 3, 1, 1, 5064, 0),     # batch 64: tile kernel without a split
+    (5, 7, 9, 32, 40, 3, 2, 1, 0, 0),            # stride equal to the image: the dense case
+]
+
+
+@pytest.mark.parametrize("case", IMAGE_STRIDE_CASES)
+@pytest.mark.parametrize("dtype", [H.F32, H.F16])
+@pytest.mark.parametrize("workspace", [True, False])
+def test_conv_out_image_stride(case, dtype, workspace):
+    """OgleConvArgs.out_image_stride: every image's outputs equal the dense launch's bit for bit,
+    land at lead + b * stride, and nothing between the images is written."""
+    n, h, w, c, o, k, s, p, extra, lead = case
+    r = rng(1800 + IMAGE_STRIDE_CASES.index(case))
+    x = r.uniform(-1, 1, (n, h, w, c)).astype(np.float32)
+    wt = r.normal(0, 0.2, (o, c, k, k)).astype(np.float32)
+    b = r.uniform(-0.1, 0.1, o).astype(np.float32)
+    variant = H.VARIANT_PW if (k == 1 and s == 1 and p == 0) else H.VARIANT_NHWC4
+    dense = gpu_conv(x, wt, b, s, p, 1, 1, H.ACT_RELU, 0.0, 0.0, variant, dtype, None, workspace)
+    image = dense[0].size
+    stride = image + extra
+    flat = gpu_conv(x, wt, b, s, p, 1, 1, H.ACT_RELU, 0.0, 0.0, variant, dtype, None, workspace,
+                    image_stride=stride, lead=lead)
+    assert flat.size == lead + n * stride
+    assert np.isnan(flat[:lead]).all()
+    rows = flat[lead:].reshape(n, stride)
+    np.testing.assert_array_equal(rows[:, :image].reshape(dense.shape), dense)
+    assert np.isnan(rows[:, image:]).all()
+    if dtype == H.F32:
+        ref = O.conv2d(x, wt, b, s, p, 1, 1, O.ACT_RELU, 0.0, 0.0, variant)
+        assert_conv_close(dense, ref, O.conv2d_abs(x, wt, b, s, p, 1, 1), FP32_RTOL, "stride " + str(case))
+
+
+def test_conv_out_image_stride_is_refused_off_the_mfma_path():
+    r = rng(1850)
+    x = r.uniform(-1, 1, (2, 6, 6, 3)).astype(np.float32)
+    wt = r.normal(0, 0.2, (8, 3, 3, 3)).astype(np.float32)
+    with pytest.raises(H.OgleError, match="out_image_stride"):
+        gpu_conv(x, wt, None, 1, 1, image_stride=6 * 6 * 8 + 8)
+    xd = r.uniform(-1, 1, (2, 6, 6, 16)).astype(np.float32)
+    wd = r.normal(0, 0.2, (16, 1, 3, 3)).astype(np.float32)
+    with pytest.raises(H.OgleError, match="out_image_stride"):
+        gpu_conv(xd, wd, None, 1, 1, groups=16, image_stride=6 * 6 * 16 + 16)
+    wt2 = r.normal(0, 0.2, (8, 16, 3, 3)).astype(np.float32)
+    with pytest.raises(H.OgleError, match="less than one image"):
+        gpu_conv(xd, wt2, None, 1, 1, image_stride=6 * 6 * 8 - 1)
+
+
 def test_conv_shape_sweep_mfma_path():
     """Channel counts that take the implicit-GEMM kernel, ragged in every dimension."""
     r = rng(2100)
@@ -395,6 +449,62 @@ def test_config4_heads_batch64_single_and_grouped_calls():
             what = "C4 b64 head %dx%d o%d %s" % (m, m, o, tag)
             assert_conv_close(got, ref.astype(np.float32), scale, FP32_RTOL, what)
             assert_conv_close(got[:1], ora, scale[:1], FP32_RTOL, what + " vs oracle")
+
+
+@pytest.mark.parametrize("batch", [2, 16])
+def test_heads_written_in_place_of_the_concat(batch):
+    """The twelve SSD heads as one ogle_hip_conv2d_batch call (and as begin + finish) with
+    out_image_stride set so that every head writes its images straight into box_preds /
+    cls_logits: the two buffers equal the concatenation of the heads launched one by one, bit
+    for bit, and the call still refuses two heads whose places overlap."""
+    import ctypes
+    import torch
+    from util import pack_filter
+    r = rng(20240016)
+    priors = sum(m * m * a for m, _, a in C4_MAPS)
+    outs = {4: torch.full((batch, priors, 4), float("nan"), device="cuda"),
+            21: torch.full((batch, priors, 21), float("nan"), device="cuda")}
+    outs2 = {k: torch.full_like(v, float("nan")) for k, v in outs.items()}
+    args = (H.ConvArgs * 12)()
+    args2 = (H.ConvArgs * 12)()
+    keep, singles = [], {4: [], 21: []}
+    at = 0
+    for mi, (m, c, a) in enumerate(C4_MAPS):
+        f = r.uniform(0, 6, (batch, m, m, c)).astype(np.float32)
+        fd = torch.from_numpy(f).cuda()
+        for hi, last in enumerate((4, 21)):
+            o = a * last
+            wt = r.normal(0, 0.01, (o, c, 3, 3)).astype(np.float32)
+            b = r.uniform(-0.1, 0.1, o).astype(np.float32)
+            singles[last].append(gpu_conv(f, wt, b, 1, 1).reshape(batch, m * m * a, last))
+            wd = pack_filter(wt, H.FILTER_OHWI)
+            bd = torch.from_numpy(b).cuda()
+            for arr, dst in ((args, outs), (args2, outs2)):
+                ar = H.conv_args(fd.data_ptr(), wd.data_ptr(), bd.data_ptr(),
+                                 dst[last].data_ptr() + at * last * 4, batch, m, m, c, o, 3, 1, 1)
+                ar.out_image_stride = priors * last
+                need = H.lib().ogle_hip_conv_workspace_bytes(ctypes.byref(ar))
+                if need:
+                    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+                    ar.workspace_dev, ar.workspace_bytes = ws.data_ptr(), need
+                    keep.append(ws)
+                arr[mi * 2 + hi] = ar
+            keep += [fd, wd, bd]
+        at += m * m * a
+    H.check(H.lib().ogle_hip_conv2d_batch(args, 12, 0))
+    open_ = (ctypes.c_int32 * 12)()
+    H.check(H.lib().ogle_hip_conv2d_batch_begin(args2, 12, open_, 0))
+    H.check(H.lib().ogle_hip_conv2d_batch_finish(args2, 12, 0))
+    torch.cuda.synchronize()
+    for last in (4, 21):
+        ref = np.concatenate(singles[last], axis=1)
+        np.testing.assert_array_equal(outs[last].cpu().numpy(), ref)
+        np.testing.assert_array_equal(outs2[last].cpu().numpy(), ref)
+    # the second map's box head moved one element into the first one's place
+    args[2].output_dev -= 4
+    assert H.lib().ogle_hip_conv2d_batch(args, 12, 0) == H.ERR_INVALID_ARG
+    assert "depend on each other" in H.last_error()
+    torch.cuda.synchronize()
 
 
 def test_fp16_storage_depthwise_and_pool():

@@ -257,6 +257,48 @@ def test_hazard_rule_is_interval_overlap():
     assert not C([], [(big, 4096)], [(big, 4096)])
 
 
+def test_hazard_rule_with_images_written_apart():
+    """Convolutions that write their images into interleaved places of one tensor (heads
+    produced inside a concat's output at batch > 1): image b of head i lies at base + b * stride
+    + offset_i.  Heads whose places differ do not conflict although their hulls overlap; a
+    reader of the enclosing tensor, of one image's slice, or a head on the same place does."""
+    base, n = 0x1000000, 4
+    img = 4 * 4 * 16 * 4                 # one image of a 4x4x16 head, 1 KiB
+    stride = 3 * img + 256               # three heads and a gap per output slice
+
+    def head(slot, inp=0x5000000, **kw):
+        a = _fake_conv(inp, base + slot * img, n=n, **kw)
+        a.out_image_stride = stride // 4
+        return a
+    C, CC = session.hazard_conflicts, session.conv_hazard_conflicts
+    pend = [head(0), head(1)]
+    assert not CC(pend, head(2))                          # its own place in every slice
+    assert CC(pend, head(1))                              # the same place: write after write
+    half = head(0)
+    half.output_dev = base + img // 2                     # straddles heads 0 and 1
+    assert CC(pend, half)
+    later = head(0)
+    later.output_dev = base + n * stride                  # the next tensor: past the last image
+    assert not CC(pend, later)
+    assert CC(pend, head(2, inp=base + stride))           # reads what head 0 writes (image 1)
+    gap = head(2)
+    gap.input_dev = base + 3 * img                        # an input that fits in the 256-byte gap
+    gap.in_h, gap.in_w, gap.in_c, gap.n = 1, 1, 8, 1
+    assert not CC(pend, gap)
+    dense = _fake_conv(0x5000000, base, n=n)              # dense writer over the same hull
+    assert CC(pend, dense)
+    # plain ranges against the strided writes
+    assert C(pend, [(base, n * stride)], [])              # the enclosing tensor (a detector read)
+    assert C(pend, [(base + 2 * stride + img, 4)], [])    # image 2 of head 1
+    assert not C(pend, [(base + 2 * img, img + 256)], []) # head 2's place and the gap in slice 0
+    assert not C(pend, [], [(base + stride + 2 * img, img)])
+    assert C(pend, [], [(base + 3 * stride + img - 4, 8)])
+    # one image: the stride means nothing
+    one = _fake_conv(0x5000000, base, n=1)
+    one.out_image_stride = stride // 4
+    assert C([one], [(base + img - 4, 4)], []) and not C([one], [(base + img, 4)], [])
+
+
 def test_reloading_a_graph_resets_the_session():
     """LoadGraph on a session that already holds a graph starts from scratch: kernel count
     follows the new graph and no recorded pass survives (checked on the device as well)."""

@@ -272,7 +272,7 @@ def test_concat_inputs_are_produced_in_place_at_batch1():
     concat outputs: every head output sits at its running offset inside box_preds / cls_logits
     (the class heads at offsets that are only 4-byte aligned: 63 and 126 channels are stored
     element by element), the concat has nothing to copy, and a replay after new input still gives
-    the concatenation.  At batch 2 the outputs interleave per image and nothing is placed."""
+    the concatenation."""
     sess, info, x = _run_ssd(1)
     for out_name, suffix, last in (("box_preds", "loc", 4), ("cls_logits", "conf", 21)):
         base = sess.tensor_device_ptr(out_name)
@@ -287,13 +287,95 @@ def test_concat_inputs_are_produced_in_place_at_batch1():
     for out_name, suffix, last in (("box_preds", "loc", 4), ("cls_logits", "conf", 21)):
         parts = [sess.get_output("head%d.%s" % (i, suffix), "NHWC").reshape(1, -1, last) for i in range(6)]
         np.testing.assert_array_equal(sess.get_output(out_name, "ANY"), np.concatenate(parts, 1))
-    # the same network at batch 1 and as image 0 of a batch of 2 (nothing placed there)
+    # the same network at batch 1 and as image 0 of a batch of 2
     sess2, _, xb = _run_ssd(2)
-    assert sess2.tensor_device_ptr("head0.loc") != sess2.tensor_device_ptr("box_preds")
     sess.run({"input": xb[:1]})
     for name in ("box_preds", "cls_logits"):
         a, b = sess.get_output(name, "ANY"), sess2.get_output(name, "ANY")[:1]
         assert np.all(np.abs(a - b) <= 1e-4 * (np.abs(b) + 1.0)), name
+
+
+def test_concat_inputs_are_produced_in_place_at_batch3():
+    """With several slices before the concat axis (batch > 1) the heads write their images
+    one output slice apart (OgleConvArgs.out_image_stride), straight into box_preds /
+    cls_logits: no Concat launch is left in the pass, a head's tensor is no longer dense on
+    the device (no device pointer; reading it back gathers its images), every head still
+    matches the oracle on the device's own feature map, the concat outputs are exactly the
+    heads side by side, and a replayed hipGraph gives the same."""
+    batch = 3
+    g, info = models.mobilenet_v1_ssd(batch, seed=20240005, with_weights=True)
+    x = rng(79).uniform(-1, 1, (batch, 300, 300, 3)).astype(np.float32)
+    sess = session.Session()
+    sess.load_graph(g)
+    sess.run({"input": x})
+    labels = [l for l, _ in sess.launch_plan()]
+    assert not any("#Concat#" in l for l in labels), labels
+    assert any("head0.loc#Conv#" in l for l in labels)
+    feats = ["block11.pw", "block13.pw", "extra1.conv", "extra2.conv", "extra3.conv", "extra4.conv"]
+    for out_name, suffix, last in (("box_preds", "loc", 4), ("cls_logits", "conf", 21)):
+        assert sess.tensor_device_ptr(out_name) is not None
+        parts = []
+        for i, feat in enumerate(feats):
+            name = "head%d.%s" % (i, suffix)
+            assert sess.tensor_device_ptr(name) is None and sess.tensor_device_ptr(name + ".view") is None
+            got = sess.get_output(name, "NHWC")
+            xin = sess.get_output(feat, "NHWC")
+            w, b = info["weights"][name]
+            assert_conv_close(got, O.conv2d(xin, w, b, 1, 1), O.conv2d_abs(xin, w, b, 1, 1), FP32_RTOL,
+                              "in place " + name)
+            np.testing.assert_array_equal(sess.get_output(name + ".view", "ANY"), got.reshape(batch, -1, last))
+            # NCHW readback of a tensor whose images lie apart
+            np.testing.assert_array_equal(sess.get_output(name, "NCHW"), got.transpose(0, 3, 1, 2))
+            parts.append(got.reshape(batch, -1, last))
+        whole = sess.get_output(out_name, "ANY")
+        assert whole.shape == (batch, 1917, last)
+        np.testing.assert_array_equal(whole, np.concatenate(parts, 1))
+        sess.compute(graph=True)
+        np.testing.assert_array_equal(sess.get_output(out_name, "ANY"), whole)
+        sess.compute(graph=False)
+        np.testing.assert_array_equal(sess.get_output(out_name, "ANY"), whole)
+
+
+def test_concat_at_batch2_copies_what_cannot_be_produced_in_place():
+    """Batch 2, concat over axis 1: a pooling output cannot be written with its images apart and
+    a convolution with a second reader must stay dense, so the concat copies; two convolutions
+    read by nothing else are placed.  Same values either way."""
+    r = rng(7995)
+    x = r.uniform(-1, 1, (2, 6, 6, 16)).astype(np.float32)
+    wa = r.normal(0, 0.3, (8, 16, 3, 3)).astype(np.float32)
+    wb = r.normal(0, 0.3, (8, 16, 3, 3)).astype(np.float32)
+    ra, rb = O.conv2d(x, wa, None, 1, 1), O.conv2d(x, wb, None, 1, 1)
+    for kind in ("placed", "pool", "second_reader"):
+        gb = dlx.GraphBuilder()
+        xi = gb.add_input("input", [2, 16, 6, 6])
+        a = gb.add_conv("a", xi, gb.add_filter("a.weight", wa), None, 3, 1, 1)
+        b = gb.add_conv("b", xi, gb.add_filter("b.weight", wb), None, 3, 1, 1)
+        second = b
+        if kind == "pool":
+            second = gb.add_pool("b.pool", b, "MaxPool", 1, 1, 0)     # a copy of b made by another kernel
+        if kind == "second_reader":
+            gb.add_relu("b.relu", b)
+        outs = []
+        for name, y in (("a", a), ("b", second)):
+            t = gb.add_transpose(name + ".permute", y, [0, 2, 3, 1])
+            shp = gb.add_const(name + ".shape", np.array([2, -1, 4], np.float32))
+            outs.append(gb.add_reshape(name + ".view", t, shp))
+        gb.add_concat("cat", outs, 1)
+        sess = session.Session()
+        sess.load_graph(gb)
+        sess.run({"input": x})
+        cat = sess.get_output("cat", "ANY")
+        ref = np.concatenate([ra.reshape(2, -1, 4), rb.reshape(2, -1, 4)], 1)
+        assert cat.shape == ref.shape
+        np.testing.assert_allclose(cat, ref, rtol=0, atol=1e-4)
+        labels = " ".join(l for l, _ in sess.launch_plan())
+        if kind == "placed":
+            assert "#Concat#" not in labels and sess.tensor_device_ptr("a") is None
+        else:
+            assert "cat#Concat#" in labels and sess.tensor_device_ptr("a") is not None
+        if kind == "second_reader":
+            np.testing.assert_array_equal(sess.get_output("b.relu", "NHWC"), np.maximum(sess.get_output("b", "NHWC"), 0))
+        np.testing.assert_array_equal(sess.get_output("a", "NHWC").reshape(2, -1, 4), cat[:, :72])
 
 
 def test_graph_replay_equals_eager_batch2():

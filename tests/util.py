@@ -42,9 +42,13 @@ def pack_filter(w_oihw, layout, dtype=H.F32):
 
 
 def gpu_conv(x, w, b=None, stride=1, pad=0, dilation=1, groups=1, act=H.ACT_NONE, minv=0.0,
-             maxv=0.0, variant=H.VARIANT_NHWC4, dtype=H.F32, entry=None, workspace=True):
+             maxv=0.0, variant=H.VARIANT_NHWC4, dtype=H.F32, entry=None, workspace=True,
+             image_stride=0, lead=0):
     """x NHWC numpy, w OIHW numpy.  Returns NHWC numpy fp32.  With workspace=True the launch gets
-    the scratch buffer ogle_hip_conv_workspace_bytes asks for (enables the split-K plans)."""
+    the scratch buffer ogle_hip_conv_workspace_bytes asks for (enables the split-K plans).
+    With image_stride (elements) the output goes into a NaN-filled buffer of `lead` +
+    n * image_stride elements, image b at lead + b * image_stride, and the whole buffer is
+    returned flat (fp32)."""
     torch = _torch()
     tdt = torch.float16 if dtype == H.F16 else torch.float32
     n, h, wd, c = x.shape
@@ -62,10 +66,14 @@ def gpu_conv(x, w, b=None, stride=1, pad=0, dilation=1, groups=1, act=H.ACT_NONE
     wdv = pack_filter(w, layout, dtype)
     bd = dev(b.astype(np.float32)) if b is not None else None
     oh, ow = H.out_size(h, k, stride, pad, dilation), H.out_size(wd, k, stride, pad, dilation)
-    y = torch.full((n, oh, ow, o), float("nan"), dtype=tdt, device="cuda")
+    if image_stride:
+        y = torch.full((lead + n * image_stride,), float("nan"), dtype=tdt, device="cuda")
+    else:
+        y = torch.full((n, oh, ow, o), float("nan"), dtype=tdt, device="cuda")
     args = H.conv_args(xd.data_ptr(), wdv.data_ptr(), bd.data_ptr() if bd is not None else None,
-                       y.data_ptr(), n, h, wd, c, o, k, stride, pad, dilation, groups, act, minv,
-                       maxv, variant, dtype)
+                       y.data_ptr() + lead * y.element_size(), n, h, wd, c, o, k, stride, pad, dilation,
+                       groups, act, minv, maxv, variant, dtype)
+    args.out_image_stride = image_stride
     ws = None
     if workspace:
         need = H.lib().ogle_hip_conv_workspace_bytes(ctypes.byref(args))
