@@ -844,35 +844,60 @@ struct ReduceGroup {
   ReduceProblem p[kMaxGroup];
 };
 
-// Sums the split-K partials, then bias and activation.  LANES consecutive lanes
-// share one output element: lane q adds splits q, q+LANES, ... in ascending order and
-// the LANES partial sums are then combined in a fixed butterfly order, so the result
-// depends on neither timing nor grid shape.  Spreading the splits over lanes keeps
-// many loads in flight when there are few outputs but many splits.
+// Sums the split-K partials, then bias and activation.  A work item is four consecutive
+// channels of one output row (the partial rows are padded to a multiple of four floats,
+// so it is one 16-byte load per split), shared by LANES consecutive lanes: lane q adds
+// splits q, q+LANES, ... in ascending order and the LANES partial sums are then combined
+// in a fixed butterfly order, so the result depends on neither timing nor grid shape.
+// Spreading the splits over lanes keeps many loads in flight when there are few outputs
+// but many splits.
 template <typename T, int LANES>
 __device__ __forceinline__ void splitk_reduce_block(const ReduceProblem& r, int bid) {
   const int q = threadIdx.x % LANES;
+  const int gpr = r.opitch >> 2;       // four-channel groups per row
+  const long rows = r.mn / r.o;
   const long idx = (long)bid * (blockDim.x / LANES) + threadIdx.x / LANES;
-  const bool live = idx < r.mn;  // dead lanes still take part in the shuffles
-  float acc = 0.f;
-  const long row = idx / r.o;
-  const int col = (int)(idx - row * r.o);
+  const bool live = idx < rows * gpr;  // dead lanes still take part in the shuffles
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  const long row = idx / gpr;
+  const int col = (int)(idx - row * gpr) * 4;
   if (live) {
-    const long src = row * r.opitch + col;
-    const long zstride = (r.mn / r.o) * r.opitch;
+    const float* src = r.partial + row * r.opitch + col;
+    const long zstride = rows * r.opitch;
 #pragma unroll 4
-    for (int z = q; z < r.splits; z += LANES) acc += r.partial[(long)z * zstride + src];
+    for (int z = q; z < r.splits; z += LANES) {
+      const float4 t = *reinterpret_cast<const float4*>(src + (long)z * zstride);
+      acc.x += t.x; acc.y += t.y; acc.z += t.z; acc.w += t.w;
+    }
   }
 #pragma unroll
-  for (int d = 1; d < LANES; d <<= 1) acc += __shfl_xor(acc, d, 64);
-  if (live && q == 0) {
-    if (r.bias != nullptr) acc += r.bias[col];
-    const T out = from_f32<T>(apply_epilogue(acc, r.ep));
-    if (r.oimg != 0) {
-      const long b = row / r.hw;
-      static_cast<T*>(r.y)[b * r.oimg + (row - b * r.hw) * r.o + col] = out;
-    } else if (col < r.o1) static_cast<T*>(r.y)[row * r.o1 + col] = out;
-    else static_cast<T*>(r.y2)[row * (r.o - r.o1) + (col - r.o1)] = out;
+  for (int d = 1; d < LANES; d <<= 1) {
+    acc.x += __shfl_xor(acc.x, d, 64);
+    acc.y += __shfl_xor(acc.y, d, 64);
+    acc.z += __shfl_xor(acc.z, d, 64);
+    acc.w += __shfl_xor(acc.w, d, 64);
+  }
+  if (!live || q != 0) return;
+  float v[4] = {acc.x, acc.y, acc.z, acc.w};
+#pragma unroll
+  for (int e = 0; e < 4; ++e)
+    if (col + e < r.o) v[e] = apply_epilogue(v[e] + (r.bias != nullptr ? r.bias[col + e] : 0.f), r.ep);
+  // where this row's channels start in y
+  long at = row * r.o1;
+  if (r.oimg != 0) {
+    const long b = row / r.hw;
+    at = b * r.oimg + (row - b * r.hw) * r.o;
+  }
+  if (sizeof(T) == 4 && r.y2 == nullptr && (r.o & 3) == 0 && (r.oimg & 3) == 0) {
+    *reinterpret_cast<float4*>(static_cast<float*>(r.y) + at + col) = make_float4(v[0], v[1], v[2], v[3]);
+    return;
+  }
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int c = col + e;
+    if (c >= r.o) continue;
+    if (c < r.o1) static_cast<T*>(r.y)[at + c] = from_f32<T>(v[e]);
+    else static_cast<T*>(r.y2)[row * (r.o - r.o1) + (c - r.o1)] = from_f32<T>(v[e]);
   }
 }
 
@@ -1153,13 +1178,14 @@ Prepared prepare(const OgleConvArgs& a, long m, const IgemmPlan& p) {
   if (p.splits > 1) {
     const long mn = (long)g.m_total * g.o;
     // enough lanes per output that the grid still has about a thousand waves
+    const long items = (long)g.m_total * (((g.o + 3) & ~3) / 4);  // four channels each
     int lanes = 1;
-    while (lanes < 8 && lanes * 2 <= p.splits && mn * lanes < 64L * 1024) lanes *= 2;
+    while (lanes < 8 && lanes * 2 <= p.splits && items * lanes < 64L * 1024) lanes *= 2;
     out.red = ReduceProblem{out.prob.partial, a.bias_dev, a.output_dev, a.output2_dev, mn, g.o,
                             out.prob.o1, (g.o + 3) & ~3, p.splits, out.prob.ep, lanes, g.oimg,
                             g.oh * g.ow};
     out.reduce_lanes = lanes;
-    out.reduce_grid = (unsigned)((mn * lanes + 255) / 256);
+    out.reduce_grid = (unsigned)((items * lanes + 255) / 256);
   }
   return out;
 }
