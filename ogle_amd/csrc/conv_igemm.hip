@@ -59,27 +59,6 @@ __device__ __forceinline__ long out_row_offset(const ConvGeom& g, int row, int p
   return (long)b * g.oimg + (long)(row - b * hw) * pitch;
 }
 
-template <typename T>
-struct Mma;
-template <>
-struct Mma<float> {
-  __device__ static __forceinline__ void run(const uint4& a, const uint4& b, floatx16& acc) {
-    const float* af = reinterpret_cast<const float*>(&a);
-    const float* bf = reinterpret_cast<const float*>(&b);
-#pragma unroll
-    for (int s = 0; s < 4; ++s)
-      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af[s], bf[s], acc, 0, 0, 0);
-  }
-};
-template <>
-struct Mma<__half> {
-  __device__ static __forceinline__ void run(const uint4& a, const uint4& b, floatx16& acc) {
-    const halfx8 ah = *reinterpret_cast<const halfx8*>(&a);
-    const halfx8 bh = *reinterpret_cast<const halfx8*>(&b);
-    acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bh, acc, 0, 0, 0);
-  }
-};
-
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 // Offset that is out of range for every operand (operands are kept below 2 GiB), so
@@ -90,6 +69,54 @@ constexpr unsigned kOutOfRange = 0x80000000u;
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, unsigned bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
 }
+
+typedef float floatx4v __attribute__((ext_vector_type(4)));
+
+// MFMA step on a TS x TS block of outputs (the wave-split kernel's tile; the LDS-tiled
+// kernel's block when its tile is 16 columns wide).  `a` / `b` are the 16 bytes
+// the lane loaded; lanes are grouped by q = lane / TS.
+//   TS 32: q in {0,1};   fp32 4 x 32x32x2 (k = 4q + s), fp16 1 x 32x32x16 (k = 8q..)
+//   TS 16: q in {0..3};  fp32 4 x 16x16x4 (k = 4q + s), fp16 1 x 16x16x32 (k = 8q..)
+template <typename T, int TS>
+struct WaveMma;
+template <>
+struct WaveMma<float, 32> {
+  typedef floatx16 Acc;
+  static constexpr int REGS = 16;
+  __device__ static __forceinline__ void run(const u32x4& a, const u32x4& b, Acc& acc) {
+#pragma unroll
+    for (int s = 0; s < 4; ++s)
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a[s]), __uint_as_float(b[s]), acc, 0, 0, 0);
+  }
+};
+template <>
+struct WaveMma<__half, 32> {
+  typedef floatx16 Acc;
+  static constexpr int REGS = 16;
+  __device__ static __forceinline__ void run(const u32x4& a, const u32x4& b, Acc& acc) {
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(halfx8, a),
+                                                 __builtin_bit_cast(halfx8, b), acc, 0, 0, 0);
+  }
+};
+template <>
+struct WaveMma<float, 16> {
+  typedef floatx4v Acc;
+  static constexpr int REGS = 4;
+  __device__ static __forceinline__ void run(const u32x4& a, const u32x4& b, Acc& acc) {
+#pragma unroll
+    for (int s = 0; s < 4; ++s)
+      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(a[s]), __uint_as_float(b[s]), acc, 0, 0, 0);
+  }
+};
+template <>
+struct WaveMma<__half, 16> {
+  typedef floatx4v Acc;
+  static constexpr int REGS = 4;
+  __device__ static __forceinline__ void run(const u32x4& a, const u32x4& b, Acc& acc) {
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(halfx8, a),
+                                                 __builtin_bit_cast(halfx8, b), acc, 0, 0, 0);
+  }
+};
 
 // One workgroup's share of one convolution: output tile / K range number `bid` of
 // the problem.  Shared by the single-problem kernel and the grouped kernel.
@@ -107,15 +134,23 @@ __device__ __forceinline__ void igemm_tile(
     int slabs_per_split, int splits, int bid) {
   static_assert(WM * WN == 4, "four waves per workgroup");
   constexpr int WTM = BM / WM, WTN = BN / WN;
-  constexpr int TM = WTM / 32, TN = WTN / 32;
-  static_assert(TM >= 1 && TN >= 1, "wave tile at least 32x32");
+  // MFMA block: 32x32 outputs, or 16x16 (v_mfma_f32_16x16x4_f32 / 16x16x32_f16) for a tile
+  // that is only 16 columns wide (a convolution with at most 16 output channels: in a
+  // 32-wide block more than half of the MFMA work would be padding)
+  constexpr int MB = WTN % 32 == 0 ? 32 : 16;
+  constexpr int TM = WTM / MB, TN = WTN / MB;
+  static_assert(TM >= 1 && TN >= 1 && WTM % MB == 0 && WTN % MB == 0, "wave tile in whole MFMA blocks");
+  typedef typename WaveMma<T, MB>::Acc Acc;
+  constexpr int REGS = WaveMma<T, MB>::REGS;
   constexpr int VPR = ROWB / 16;       // 16-byte vectors per row per slab
   constexpr int RPP = 256 / VPR;       // rows one pass of the workgroup loads
   constexpr int AP = (BM + RPP - 1) / RPP, BP = (BN + RPP - 1) / RPP;
   constexpr bool A_PART = BM % RPP != 0, B_PART = BN % RPP != 0;  // last pass partly idle
   constexpr int LROW = ROWB + 16;      // padded LDS row, bytes
   constexpr int ESZ = (int)sizeof(T);
-  constexpr int CHUNKS = ROWB / 32;
+  constexpr int CHUNKB = (64 / MB) * 16;  // bytes of a row one MFMA step consumes (64 / MB lane groups x 16)
+  constexpr int CHUNKS = ROWB / CHUNKB;
+  static_assert(CHUNKS >= 1, "a K slab holds at least one MFMA step");
   constexpr int STAGE = (BM + BN) * LROW;  // one buffer: A rows then B rows
 
   static_assert(2 * STAGE == igemm_lds_bytes<BM, BN, ROWB>(), "LDS size");
@@ -261,16 +296,18 @@ __device__ __forceinline__ void igemm_tile(
         *reinterpret_cast<u32x4*>(base_ + (BM + p * RPP) * LROW) = rb[SET][p];               \
   }
 
-  floatx16 acc[TM][TN];
+  Acc acc[TM][TN];
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+      for (int r = 0; r < REGS; ++r) acc[i][j][r] = 0.f;
 
   const int l32 = lane & 31;
   const int lh = lane >> 5;
+  const int lrow = lane % MB;  // operand row of this lane inside an MFMA block
+  const int lq = lane / MB;    // its 16-byte group along K
 
   // Split-K: workgroup z of the grid contracts K slabs [kt_begin, kt_end) only and
   // leaves its partial sums in `partial`; a second kernel adds the splits in order.
@@ -280,16 +317,17 @@ __device__ __forceinline__ void igemm_tile(
   // One K slab from LDS buffer `buf` into the accumulators.
 #define OGLE_COMPUTE_SLAB(buf)                                                               \
   {                                                                                          \
-    const unsigned char* pa = lds + (buf) * STAGE + (wave_m * WTM + l32) * LROW + lh * 16;   \
-    const unsigned char* pb = lds + (buf) * STAGE + (BM + wave_n * WTN + l32) * LROW + lh * 16; \
+    const unsigned char* pa = lds + (buf) * STAGE + (wave_m * WTM + lrow) * LROW + lq * 16;  \
+    const unsigned char* pb = lds + (buf) * STAGE + (BM + wave_n * WTN + lrow) * LROW + lq * 16; \
     _Pragma("unroll") for (int ch = 0; ch < CHUNKS; ++ch) {                                  \
-      uint4 av[TM], bv[TN];                                                                  \
+      u32x4 av[TM], bv[TN];                                                                  \
       _Pragma("unroll") for (int i = 0; i < TM; ++i)                                         \
-        av[i] = *reinterpret_cast<const uint4*>(pa + i * 32 * LROW + ch * 32);               \
+        av[i] = *reinterpret_cast<const u32x4*>(pa + i * MB * LROW + ch * CHUNKB);           \
       _Pragma("unroll") for (int j = 0; j < TN; ++j)                                         \
-        bv[j] = *reinterpret_cast<const uint4*>(pb + j * 32 * LROW + ch * 32);               \
+        bv[j] = *reinterpret_cast<const u32x4*>(pb + j * MB * LROW + ch * CHUNKB);           \
       _Pragma("unroll") for (int i = 0; i < TM; ++i)                                         \
-        _Pragma("unroll") for (int j = 0; j < TN; ++j) Mma<T>::run(av[i], bv[j], acc[i][j]); \
+        _Pragma("unroll") for (int j = 0; j < TN; ++j)                                       \
+          WaveMma<T, MB>::run(av[i], bv[j], acc[i][j]);                                      \
     }                                                                                        \
   }
 
@@ -342,6 +380,33 @@ __device__ __forceinline__ void igemm_tile(
   const int opitch = (g.o + 3) & ~3;
   const int o2 = g.o - o1;
   float* const pdst = partial != nullptr ? partial + (long)split * g.m_total * opitch : nullptr;
+  if constexpr (MB == 16) {
+    // 16x16 blocks: register r of lane l is row 4 * (l / 16) + r, column l % 16, so the 16
+    // lanes of a group store one 64-byte run of an output row.  Partial rows are written
+    // up to their padded width (the columns past the last channel hold zeros).
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int col = n0 + wave_n * WTN + j * 16 + lrow;
+      const float bv = (pdst == nullptr && bias != nullptr && col < g.o) ? bias[col] : 0.f;
+      const bool second = col >= o1;
+      T* const dst = second ? y2 + (col - o1) : y + col;
+      const int dpitch = second ? o2 : o1;
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int r = 0; r < REGS; ++r) {
+          const int row = m0 + wave_m * WTM + i * 16 + lq * 4 + r;
+          if (row >= g.m_total) continue;
+          if (pdst != nullptr) {
+            if (col < opitch) pdst[(long)row * opitch + col] = acc[i][j][r];
+          } else if (col < g.o) {
+            dst[out_row_offset(g, row, dpitch)] = from_f32<T>(apply_epilogue(acc[i][j][r] + bv, ep));
+          }
+        }
+      }
+    }
+    return;
+  } else {
   // The staging region (reused K-loop LDS) takes JC 32-column blocks of a wave's tile at a
   // time: as many as fit, so that a row segment a wave stores is as long as possible.
   constexpr auto stage_fits = [](int jc) { return 4 * 32 * (jc * 32 + 4) * 4 <= 2 * STAGE; };
@@ -465,6 +530,7 @@ __device__ __forceinline__ void igemm_tile(
       }
     }
   }
+  }  // MB == 32
 }
 
 // Everything one convolution's workgroups need, as plain data (a kernel argument).
@@ -480,7 +546,7 @@ struct IgemmProblem {
   int tiles_n, tiles;
   float* partial;
   int slabs_per_split, splits;
-  int variant;  // mixed-group kernel only: 2 * (tile is 128x32) + (pointwise); 4..7: wave-split 32 / 16
+  int variant;  // mixed-group kernel only: 2 * (tile is 128x32) + (pointwise); 4..7: wave-split 32 / 16; 8, 9: 128x16 tile
 };
 
 template <typename T, int BM, int BN, int WM, int WN, int ROWB, bool PW>
@@ -541,9 +607,8 @@ __device__ __forceinline__ void igemm_wave_tile(
 // lane, so the register budget is that of the largest one.
 template <typename T, int ROWB>
 __global__ __launch_bounds__(256) void conv_igemm_mixed_kernel(IgemmGroup grp) {
-  constexpr int kLds = igemm_lds_bytes<128, 32, ROWB>() > igemm_lds_bytes<64, 64, ROWB>()
-                           ? igemm_lds_bytes<128, 32, ROWB>()
-                           : igemm_lds_bytes<64, 64, ROWB>();
+  constexpr int kLds = igemm_lds_bytes<128, 32, ROWB>();  // the largest of the tiles below
+  static_assert(kLds >= igemm_lds_bytes<128, 16, ROWB>() && kLds >= igemm_lds_bytes<64, 64, ROWB>(), "LDS size");
   __shared__ __attribute__((aligned(16))) unsigned char lds[kLds];
   int i = 0;
   while (i + 1 < grp.count && (int)blockIdx.x >= grp.first[i + 1]) ++i;
@@ -562,6 +627,8 @@ __global__ __launch_bounds__(256) void conv_igemm_mixed_kernel(IgemmGroup grp) {
     OGLE_MIXED_CASE(1, 64, 64, 2, 2, true)
     OGLE_MIXED_CASE(2, 128, 32, 4, 1, false)
     OGLE_MIXED_CASE(3, 128, 32, 4, 1, true)
+    OGLE_MIXED_CASE(8, 128, 16, 4, 1, false)
+    OGLE_MIXED_CASE(9, 128, 16, 4, 1, true)
 #define OGLE_MIXED_WAVE(V, PW, TS)                                                               \
   case V:                                                                                       \
     /* two steps in flight only: the group kernel's register budget is the 64x64 tile's */      \
@@ -593,53 +660,6 @@ __global__ __launch_bounds__(256) void conv_igemm_mixed_kernel(IgemmGroup grp) {
 // can keep its MFMA pipe busy because consecutive MFMAs into one accumulator issue
 // back to back.  Operands are re-read by every tile that shares them, which the L2
 // absorbs at these sizes.
-typedef float floatx4v __attribute__((ext_vector_type(4)));
-
-// MFMA step of the wave-split kernel for a TS x TS tile.  `a` / `b` are the 16 bytes
-// the lane loaded; lanes are grouped by q = lane / TS.
-//   TS 32: q in {0,1};   fp32 4 x 32x32x2 (k = 4q + s), fp16 1 x 32x32x16 (k = 8q..)
-//   TS 16: q in {0..3};  fp32 4 x 16x16x4 (k = 4q + s), fp16 1 x 16x16x32 (k = 8q..)
-template <typename T, int TS>
-struct WaveMma;
-template <>
-struct WaveMma<float, 32> {
-  typedef floatx16 Acc;
-  static constexpr int REGS = 16;
-  __device__ static __forceinline__ void run(const u32x4& a, const u32x4& b, Acc& acc) {
-#pragma unroll
-    for (int s = 0; s < 4; ++s)
-      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a[s]), __uint_as_float(b[s]), acc, 0, 0, 0);
-  }
-};
-template <>
-struct WaveMma<__half, 32> {
-  typedef floatx16 Acc;
-  static constexpr int REGS = 16;
-  __device__ static __forceinline__ void run(const u32x4& a, const u32x4& b, Acc& acc) {
-    acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(halfx8, a),
-                                                 __builtin_bit_cast(halfx8, b), acc, 0, 0, 0);
-  }
-};
-template <>
-struct WaveMma<float, 16> {
-  typedef floatx4v Acc;
-  static constexpr int REGS = 4;
-  __device__ static __forceinline__ void run(const u32x4& a, const u32x4& b, Acc& acc) {
-#pragma unroll
-    for (int s = 0; s < 4; ++s)
-      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(a[s]), __uint_as_float(b[s]), acc, 0, 0, 0);
-  }
-};
-template <>
-struct WaveMma<__half, 16> {
-  typedef floatx4v Acc;
-  static constexpr int REGS = 4;
-  __device__ static __forceinline__ void run(const u32x4& a, const u32x4& b, Acc& acc) {
-    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(halfx8, a),
-                                                 __builtin_bit_cast(halfx8, b), acc, 0, 0, 0);
-  }
-};
-
 constexpr int kWaveRedBytes = 4 * 32 * 36 * 4;  // four staged 32x32 partial tiles, padded rows
 
 // U: steps of loads in flight per register set (two sets).
@@ -926,10 +946,11 @@ __global__ __launch_bounds__(256) void splitk_reduce_group_kernel(ReduceGroup gr
 enum TileCfg {
   CFG_128x128 = 0, CFG_128x64 = 1, CFG_64x64 = 2, CFG_128x32 = 3, CFG_WAVE32 = 4, CFG_WAVE16 = 5,
   CFG_128x96 = 6, CFG_128x160 = 7,  // all output channels of a narrow, long-K problem in one tile
-  CFG_128x256 = 8                    // fp16 storage: 64x128 per wave, 64-byte K slabs
+  CFG_128x256 = 8,                   // fp16 storage: 64x128 per wave, 64-byte K slabs
+  CFG_128x16 = 9                     // at most 16 output channels: 16x16 MFMA blocks
 };
-constexpr int kCfgBM[] = {128, 128, 64, 128, 32, 16, 128, 128, 128};
-constexpr int kCfgBN[] = {128, 64, 64, 32, 32, 16, 96, 160, 256};
+constexpr int kCfgBM[] = {128, 128, 64, 128, 32, 16, 128, 128, 128, 128};
+constexpr int kCfgBN[] = {128, 64, 64, 32, 32, 16, 96, 160, 256, 16};
 constexpr int kRowBytesF16Wide = 64;  // K bytes per tile row per slab of CFG_128x256
 
 struct IgemmPlan {
@@ -989,6 +1010,8 @@ IgemmPlan plan_igemm(const OgleConvArgs& a, long m, bool allow_split) {
     const int epr2 = kRowBytesF16Wide / esz;
     p.cchunks = (a.in_c + epr2 - 1) / epr2;
     p.ktiles = a.kernel_size * a.kernel_size * p.cchunks;
+  } else if (a.out_c <= 16) {
+    p.cfg = CFG_128x16;
   } else if (a.out_c <= 32) {
     p.cfg = CFG_128x32;
   } else if (a.out_c > 64 && tiles(CFG_128x128) >= big_tiles_wanted) {
@@ -1168,7 +1191,8 @@ Prepared prepare(const OgleConvArgs& a, long m, const IgemmPlan& p) {
   out.prob.partial = p.splits > 1 ? static_cast<float*>(a.workspace_dev) : nullptr;
   out.prob.slabs_per_split = p.slabs_per_split;
   out.prob.splits = p.rows_on_xcd ? -p.splits : p.splits;
-  out.prob.variant = (p.cfg == CFG_WAVE32 ? 4 : p.cfg == CFG_WAVE16 ? 6 : p.cfg == CFG_128x32 ? 2 : 0) +
+  out.prob.variant = (p.cfg == CFG_WAVE32 ? 4 : p.cfg == CFG_WAVE16 ? 6 : p.cfg == CFG_128x32 ? 2 :
+                      p.cfg == CFG_128x16 ? 8 : 0) +
                      (is_pointwise(a) ? 1 : 0);
   if (is_wave(p.cfg)) {
     out.grid = (unsigned)(tiles_m * tiles_n);
@@ -1223,6 +1247,9 @@ Prepared prepare(const OgleConvArgs& a, long m, const IgemmPlan& p) {
       break;                                                                                 \
     case CFG_128x160:                                                                        \
       launch((K<T, 128, 160, 4, 1, ROWB, PW>), dim3(grid), dim3(256), 0, s, arg); \
+      break;                                                                                 \
+    case CFG_128x16:                                                                         \
+      launch((K<T, 128, 16, 4, 1, ROWB, PW>), dim3(grid), dim3(256), 0, s, arg);  \
       break;                                                                                 \
     default:                                                                                 \
       launch((K<T, 128, 32, 4, 1, ROWB, PW>), dim3(grid), dim3(256), 0, s, arg);  \
@@ -1328,7 +1355,7 @@ int32_t launch_conv_batch(const OgleConvArgs* args, int count, hipStream_t s,
     if (reduce_pending != nullptr && p.splits > 1) reduce_pending[i] = 1;
   }
   auto mixable = [](const Item& it) {
-    return it.cfg == CFG_64x64 || it.cfg == CFG_128x32 || is_wave(it.cfg);
+    return it.cfg == CFG_64x64 || it.cfg == CFG_128x32 || it.cfg == CFG_128x16 || is_wave(it.cfg);
   };
   std::vector<bool> done(items.size(), false);
   for (size_t a0 = 0; a0 < items.size(); ++a0) {

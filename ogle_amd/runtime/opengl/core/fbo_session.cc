@@ -277,6 +277,18 @@ void FBOSession::PlaceInputsInOutputs() {
     }
     k->set_inputs_in_place(true);
   }
+  // Every kernel but a placed node and the views on its inputs assumes dense inputs.
+  for (auto& kp : kernels_) {
+    Kernel* k = kp.get();
+    if (CheckKernelReady(k) || k->inputs_in_place()) continue;
+    bool view = !k->output_tensor_indexes_.empty();
+    for (size_t j = 0; j < k->output_tensor_indexes_.size(); ++j)
+      if (k->OutputAliasesInput(static_cast<int>(j)) < 0) view = false;
+    if (view) continue;
+    for (const Tensor* t : k->input_tensors_)
+      CHECK(t == nullptr || t->outer_stride_bytes() == 0)
+          << "node " << k->kernel_name() << " would read a tensor whose images lie apart";
+  }
 }
 
 // Issue order of a pass: file order, unless reordering was asked for.  The context defers

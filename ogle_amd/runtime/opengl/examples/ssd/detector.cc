@@ -52,6 +52,9 @@ void Detector::EnqueuePostprocess(const TensorNameList& names, int raw_width, in
   Tensor* box_preds = session_->FindTensorByName(names[1]);
   Tensor* anchors = session_->FindTensorByName(names[2]);
   CHECK(cls_logits && box_preds && anchors) << "detector outputs were not produced";
+  CHECK(cls_logits->outer_stride_bytes() == 0 && box_preds->outer_stride_bytes() == 0 &&
+        anchors->outer_stride_bytes() == 0)
+      << "the detector reads dense tensors: a head placed inside a concatenation cannot be named";
   CHECK_EQ(cls_logits->shape().size(), 3u);
   CHECK_EQ(box_preds->shape().size(), 3u);
   const int batch = box_preds->shape()[0], priors = box_preds->shape()[1];

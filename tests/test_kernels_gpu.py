@@ -229,6 +229,39 @@ def test_conv_out_image_stride_is_refused_off_the_mfma_path():
         gpu_conv(xd, wt2, None, 1, 1, image_stride=6 * 6 * 8 - 1)
 
 
+# (n, h, w, c, o, k, stride, pad): at most 16 output channels on the MFMA path, i.e. the tile
+# of 16x16 MFMA blocks: one tile row and many, ragged M, split K and not, ragged last K step
+NARROW_CASES = [
+    (16, 19, 19, 512, 12, 3, 1, 1),    # the 19x19 box head at batch 16 (split K + reduce)
+    (1, 38, 38, 128, 16, 3, 1, 1),     # all 16 columns used, M = 1444
+    (2, 9, 7, 24, 5, 3, 2, 1),         # tiny, M = 40 < one tile, C not a multiple of the K slab
+    (3, 31, 17, 64, 1, 1, 1, 0),       # pointwise, one output channel
+    (64, 10, 10, 64, 13, 1, 1, 0),     # pointwise, 50 tile rows, odd channel count
+    (1, 150, 150, 32, 8, 3, 1, 1),     # many tile rows, short K
+    (2, 5, 5, 1024, 16, 3, 1, 2),      # padding 2 (output 7x7), long K
+]
+
+
+@pytest.mark.parametrize("case", NARROW_CASES)
+@pytest.mark.parametrize("dtype", [H.F32, H.F16])
+def test_conv_narrow_tile(case, dtype):
+    n, h, w, c, o, k, s, p = case
+    r = rng(1900 + NARROW_CASES.index(case))
+    x = r.uniform(-1, 1, (n, h, w, c)).astype(np.float32)
+    wt = r.normal(0, 0.2, (o, c, k, k)).astype(np.float32)
+    b = r.uniform(-0.1, 0.1, o).astype(np.float32)
+    if dtype == H.F16:
+        x = x.astype(np.float16).astype(np.float32)
+        wt = wt.astype(np.float16).astype(np.float32)
+    variant = H.VARIANT_PW if (k == 1 and s == 1 and p == 0) else H.VARIANT_NHWC4
+    ref = O.conv2d(x, wt, b, s, p, 1, 1, O.ACT_CLIP, 0.0, 6.0, variant)
+    scale = O.conv2d_abs(x, wt, b, s, p, 1, 1)
+    for workspace in (True, False):
+        got = gpu_conv(x, wt, b, s, p, 1, 1, H.ACT_CLIP, 0.0, 6.0, variant, dtype, None, workspace)
+        assert_conv_close(got, ref, scale, FP16_RTOL if dtype == H.F16 else FP32_RTOL,
+                          "narrow %s ws=%s" % (case, workspace))
+
+
 def test_conv_shape_sweep_mfma_path():
     """Channel counts that take the implicit-GEMM kernel, ragged in every dimension."""
     r = rng(2100)
