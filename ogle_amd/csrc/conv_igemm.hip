@@ -26,6 +26,11 @@
 // Result layout of a 32x32 block: register r of lane l holds
 // row 8*(r/4) + 4*(l/32) + r%4, column l%32, so a store instruction writes two
 // 128-byte runs of one output pixel's channels.
+//
+// A tile that is 16 columns wide (at most 16 output channels) is built from 16x16
+// blocks instead: v_mfma_f32_16x16x4_f32 (lane l supplies A[l%16][l/16], four lane
+// groups take k 0..3, 4..7, 8..11, 12..15 of a 16-wide group and issue four MFMAs)
+// or v_mfma_f32_16x16x32_f16; register r of lane l is row 4*(l/16) + r, column l%16.
 #include <mutex>
 #include <vector>
 
