@@ -40,13 +40,27 @@ def build_session(batch, seed=20240005, input_seed=None):
     return s, info
 
 
+TAIL_FAMILY = "concat + detector tail (decode / score filter, top-k + NMS)"
+
+
+def detector_tail_bytes(batch, priors=1917, classes=21, topk=100):
+    """Algorithmic bytes of the detector tail per pass.  Decode + softmax-max + score filter: per
+    image the class logits and box predictions in, the decoded boxes and one (score, class) pair
+    per prior out, and the anchors once for the batch.  Top-k + NMS: per image one 28-byte record
+    per prior in (score, class, prior, rectangle) and at most `topk` 44-byte records out.  The
+    concatenations move nothing: the heads write straight into their outputs."""
+    per_image = priors * classes * 4 + priors * 16 + priors * 16 + priors * 8   # 161,028 + 30,672 + 30,672 + 15,336
+    nms = priors * 28 + topk * 44
+    return batch * (per_image + nms) + priors * 16
+
+
 def family_of(nodes, layers):
     """Kernel family of one entry of the launch plan, from the nodes it was launched for."""
     fams = set()
     for n in nodes:
         l = layers.get(n)
         if l is None:
-            fams.add("concat + detector tail (decode / score filter, top-k + NMS)")
+            fams.add(TAIL_FAMILY)
         elif n.startswith("head") or n.startswith("extra"):
             fams.add("SSD heads + extras chain (dense 3x3 and 1x1, MFMA implicit GEMM)")
         elif l["kind"] == "pw":
@@ -79,6 +93,8 @@ def per_family_roofline(sess, info, batch, passes, pass_us):
             per_label[label] = per_label.get(label, 0.0) + sum(us) / passes
             if p == 0:
                 f["launches"] += len(us)
+                if name == TAIL_FAMILY and not f["bytes"]:
+                    f["bytes"] = float(detector_tail_bytes(batch))
                 if not label.startswith("reduce:"):
                     for n in nodes:
                         if n in layers:
@@ -356,20 +372,26 @@ def cpu_baseline(seed=20240005, images=2, repeats=1):
         boxes = O.ssd_decode(loc, info["anchors"])
         return O.box_info(conf, boxes, 0.3, 300.0, 300.0)
 
-    t0 = time.perf_counter()
-    one_pass()  # warm-up (page in, thread pool); also sizes the sample
-    first = time.perf_counter() - t0
-    repeats = max(repeats, int(12.0 / max(first, 1e-3)))  # about 12 s of CPU work
-    t0 = time.perf_counter()
-    for _ in range(repeats):
+    # the reference's own protocol (nn/main.cc:76-111): 3 warm-up runs, then timed runs, here the
+    # median of at least 20 and as many more as fit in about 10 s of CPU work
+    for _ in range(3):
         one_pass()
-    dt = time.perf_counter() - t0
-    return dict(value=round(images * repeats / dt, 3), unit="images/s", cores=O.num_threads(),
-                kind="port",
-                sample="%d pass(es) of the full network + decoder over %d image(s), %.1f s of CPU work; "
+    times = []
+    t_all = time.perf_counter()
+    while len(times) < max(20, repeats) or (time.perf_counter() - t_all < 10.0 and len(times) < 2000):
+        t0 = time.perf_counter()
+        one_pass()
+        times.append(time.perf_counter() - t0)
+    dt = time.perf_counter() - t_all
+    med = float(np.median(times))
+    return dict(value=round(images / med, 3), unit="images/s", cores=O.num_threads(),
+                kind="port", protocol="3 warm-up passes, then the median of %d timed passes" % len(times),
+                ms_per_pass=dict(median=round(med * 1e3, 3), min=round(min(times) * 1e3, 3),
+                                 max=round(max(times) * 1e3, 3)),
+                sample="%d timed pass(es) of the full network + decoder over %d image(s), %.1f s of CPU work; "
                        "C restatement of the shaders' arithmetic, OpenMP over output rows "
                        "(not the reference under Mesa llvmpipe, which cannot be built here)"
-                       % (repeats, images, dt))
+                       % (len(times), images, dt))
 
 
 def profile_layers_run(args):
@@ -417,6 +439,11 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--batch", type=int, default=16)
+    ap.add_argument("--repeats", type=int, default=7,
+                    help="timed regions of --steps steps each; the median region is reported")
+    ap.add_argument("--clock-ramp", type=float, default=0.5,
+                    help="seconds of untimed replays of the pass between the warm-up steps and the "
+                         "first timed region (lets the clocks settle)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--eager", action="store_true", help="launch kernel by kernel instead of a hipGraph")
     ap.add_argument("--streams", type=int, default=4,
@@ -451,18 +478,61 @@ def main():
     # queues as they are created, and two sessions that land on one queue do not overlap.
     sess, info = build_session(args.batch)
     pool = [sess] + [build_session(args.batch, input_seed=100 + i)[0] for i in range(1, streams)]
-    # one stream: K passes (network + decode/score filter + top-k/NMS) one after the other,
-    # inputs resident, bracketed by syncs
+    from ogle_amd import session as _session
+
+    def run_single(k):
+        return sess.time_compute(0, k, graph=use_graph, with_detect=True)
+
+    def run_pipelined(k):
+        _session.Session.time_pipelined(pool, 0, k, with_detect=True)
+
+    def all_idle():
+        for s_ in pool:
+            s_.sync()
+        torch.cuda.synchronize()
+
+    def timed_regions(run, repeats):
+        """`repeats` timed regions of exactly args.steps steps each, every region bracketed by a
+        wait for all streams on both sides; wall-clock ms of each region."""
+        out = []
+        for _ in range(repeats):
+            all_idle()
+            t0 = time.perf_counter()
+            run(args.steps)
+            all_idle()
+            out.append((time.perf_counter() - t0) * 1e3)
+        return out
+
+    def spread(ms_list):
+        per = sorted(m / args.steps for m in ms_list)
+        return dict(median=round(float(np.median(per)), 4), min=round(per[0], 4), max=round(per[-1], 4),
+                    regions=len(per))
+
+    headline_run = run_single if streams == 1 else run_pipelined
+    # W untimed warm-up steps, then the clock ramp: the headline's pass is replayed until
+    # --clock-ramp seconds have gone by, so that the timed regions see settled clocks whatever
+    # the step count (20 steps of 0.6 ms are over before the clocks have moved)
     sess.time_compute(args.warmup, 0, graph=use_graph, with_detect=True)
-    sess.sync()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
+    if streams > 1:
+        _session.Session.time_pipelined(pool, args.warmup, 0, with_detect=True)
+    all_idle()
+    t_ramp = time.perf_counter()
+    ramp_steps = 0
+    while time.perf_counter() - t_ramp < args.clock_ramp:
+        headline_run(50)
+        all_idle()
+        ramp_steps += 50
+    clock_ramp_s = time.perf_counter() - t_ramp
+
+    # one stream: K passes (network + decode/score filter + top-k/NMS) one after the other,
+    # inputs resident, bracketed by syncs; the median of args.repeats such regions
+    single_ms = timed_regions(run_single, args.repeats)
     each, total_ms = sess.time_compute(0, args.steps, graph=use_graph, with_detect=True)
-    sess.sync()
-    torch.cuda.synchronize()
-    single_wall_ms = (time.perf_counter() - t0) * 1e3
+    all_idle()
+    single_wall_ms = float(np.median(single_ms))
     single = {"images_per_s": round(args.batch * args.steps / (single_wall_ms * 1e-3), 1),
               "ms_per_step": round(single_wall_ms / args.steps, 4),
+              "ms_per_step_spread": spread(single_ms),
               "event_ms_per_step": round(total_ms / args.steps, 4)}
     # the same, with the final detections (at most 100 per image) read back to the host inside
     # every step, as the reference's own timing loop does (nn/main.cc:76-111 includes GetOutputs):
@@ -479,19 +549,14 @@ def main():
         "detections_per_step": kept / args.steps,
         "note": "one pass, then wait and copy the final lists to the host, then the next pass"}
     if streams == 1:
-        wall_ms = single_wall_ms
+        region_ms = single_ms
     else:
         # the timed region of the headline: the same K passes dealt round-robin over `streams`
         # sessions (same graph and weights, own buffers and stream, own resident input), each a
         # hipGraph replay, so that one pass's launch gaps and under-filled kernels are covered by
-        # the others' work; bracketed by syncs of every stream
-        from ogle_amd import session as _session
-        _session.Session.time_pipelined(pool, args.warmup, 0, with_detect=True)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        _session.Session.time_pipelined(pool, 0, args.steps, with_detect=True)
-        torch.cuda.synchronize()
-        wall_ms = (time.perf_counter() - t0) * 1e3
+        # the others' work; bracketed by syncs of every stream; the median of args.repeats regions
+        region_ms = timed_regions(run_pipelined, args.repeats)
+    wall_ms = float(np.median(region_ms))
     ms_per_step = wall_ms / args.steps
     images_per_s = args.batch * args.steps / (wall_ms * 1e-3)
 
@@ -539,7 +604,11 @@ def main():
                     achieved=dom["gbs"] if dom["bound"] == "hbm" else dom["tflops"],
                     peak=HBM_PEAK_GBS if dom["bound"] == "hbm" else MFMA_F32_PEAK_TFLOPS,
                     unit="GB/s" if dom["bound"] == "hbm" else "TFLOP/s", frac=dom["frac"],
-                    traffic=read_traffic_summary(dom["kernel"]), launches_per_step=dom["launches"],
+                    traffic=read_traffic_summary(dom["kernel"]),
+                    traffic_source="profiles/bench_b16_per_layer_traffic.txt (two rocprofv3 --pmc runs, "
+                                   "FETCH_SIZE and WRITE_SIZE, of this script's --profile-layers leg; read "
+                                   "from that committed summary, not measured in this run)",
+                    launches_per_step=dom["launches"],
                     avg_launch_us=dom["avg_launch_us"],
                     avg_kernel_only_us=dom["avg_kernel_only_us"],
                     dispatch_gap_us=round(gap_us, 3),
@@ -563,6 +632,12 @@ def main():
         "metric": METRIC, "value": round(images_per_s, 1), "unit": "images/s",
         "single_stream": single, "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "ms_per_step_spread": spread(region_ms),
+        "value_spread": {"min": round(args.batch * args.steps / (max(region_ms) * 1e-3), 1),
+                         "max": round(args.batch * args.steps / (min(region_ms) * 1e-3), 1),
+                         "note": "value is the median of %d timed regions of %d steps each"
+                                 % (len(region_ms), args.steps)},
+        "clock_ramp_s": round(clock_ramp_s, 3), "clock_ramp_steps": ramp_steps,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": "MobileNet-v1-SSD 300x300 fp32, random init, BN folded, 21 classes, "

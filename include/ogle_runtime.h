@@ -38,12 +38,25 @@ int32_t ogle_rt_load_bytes(OgleSession* s, const void* data, size_t size);
 
 /*
  * FBOSession::Run(NamedTensorList) (fbo_session.cc:127-165).  Input i is a host
- * float buffer named names[i] of shape dims[i][0..ranks[i]) whose element order is
- * dformats[i] ("NHWC", "NCHW" or "ANY").  The first call allocates every tensor.
+ * float buffer named names[i] of LOGICAL shape dims[i][0..ranks[i]) whose element order
+ * is dformats[i]: "NHWC", "NCHW" or "ANY" (dense, the product of the dims), or one of
+ * the reference's stride-4 layouts "NHWC4", "ANY4", "HWN4C4"
+ * (tensor_format.cc:272-343), whose buffers are larger than the product of the dims.
+ * The buffer must hold ogle_rt_host_elements(dims[i], ranks[i], dformats[i]) floats:
+ * that many are read.  The first call allocates every tensor.
  */
 int32_t ogle_rt_run(OgleSession* s, int32_t n_inputs, const char* const* names,
                     const float* const* data, const int32_t* const* dims, const int32_t* ranks,
                     const char* const* dformats);
+
+/*
+ * Floats a host buffer of logical shape dims[0..rank) holds in layout `dformat`
+ * (CalcAllocatedSize1D/2D, tensor_format.cc:251-343): the product of the dims for
+ * "NHWC" / "NCHW" / "ANY"; n*h*w*4*ceil(c/4) for "NHWC4"; the last dim rounded up to 4
+ * for "ANY4"; kh*kw*ceil(o/4) rows of 4*ceil(i/4) texels of 4 for "HWN4C4" (dims OIHW).
+ * Negative status for an unknown tag or a rank the layout does not take.
+ */
+int64_t ogle_rt_host_elements(const int32_t* dims, int32_t rank, const char* dformat);
 
 /* One pass over the kernels with inputs already resident on the device. */
 int32_t ogle_rt_compute(OgleSession* s);

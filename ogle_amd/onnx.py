@@ -72,6 +72,8 @@ def _decode_tensor(buf):
             (np.frombuffer(raw, "<i8").astype(np.float32) if raw is not None else None)
     else:
         raise ConvertError("unsupported data type when converting tensor %d ('%s')" % (data_type, name))
+    if count == 0:   # a zero-sized dimension: an empty tensor, as the reference emits it
+        values = np.zeros(0, np.float32)
     if values is None or values.size < count:
         raise ConvertError("tensor '%s' holds %d values, its dims %s need %d" % (
             name, 0 if values is None else values.size, dims, count))

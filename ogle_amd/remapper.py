@@ -18,6 +18,26 @@ The fused node takes the name and the output tensor of the last node of the patt
 consumers are untouched.  Unlike the reference, a pattern is only folded when the
 intermediate tensors have no other consumer and the parameters are constants owned by
 the pattern; anything else is left as it is.
+
+Node order and tensor indices of the result follow the reference's round trip through
+its Graph class (converter/converter/core/converter.cc:33-42):
+
+  1. GraphConstructor::Convert (graph/graph_constructor.cc:144-190) gives node ids in
+     topological order, always taking the ready node that comes first in the file, so a
+     file that is already sorted keeps its order and an unsorted one is sorted;
+  2. the pass walks the ids from the last to the first; a bias it has to make is a new
+     Const node named "<conv>:<input slot>" whose id is the next free one
+     (remapper.cc:71-96), i.e. after every node of the file;
+  3. Graph::ToGraphDef (graph/graph.cc:12-54, 233-331) sorts again, always taking the
+     ready node with the smallest id, drops every node that has neither inputs nor
+     consumers and is not a graph output (the folded BatchNormalization's parameters),
+     and numbers the tensors in the order their nodes are written.
+
+A made bias therefore comes after all other constants, and its convolution (with
+everything downstream) after it.  One difference is kept on purpose: ToGraphDef only
+lists a node as a graph output when it has no output slot (graph.cc:279-285), which is
+never the case for a converted model, so the reference writes an empty output list;
+here the output names of the source model are kept.
 """
 import struct
 from collections import defaultdict
@@ -63,12 +83,87 @@ def encode_model(model):
     return dlx._sub(1, graph) + dlx._string(2, model["version"]) + dlx._string(3, model["producer_name"])
 
 
+def _topological(count, inputs_of, rank):
+    """Kahn's algorithm over nodes 0..count-1 where inputs_of(i) lists the nodes i reads
+    (once per edge) and the ready node of the smallest rank goes first: the std::set<int>
+    ready lists of GraphConstructor::Convert and of TopologicalSort in graph.cc."""
+    import heapq
+    pending = [0] * count
+    users = defaultdict(list)
+    for i in range(count):
+        for src in inputs_of(i):
+            users[src].append(i)
+            pending[i] += 1
+    ready = [(rank[i], i) for i in range(count) if pending[i] == 0]
+    heapq.heapify(ready)
+    order = []
+    while ready:
+        _, i = heapq.heappop(ready)
+        order.append(i)
+        for u in users[i]:
+            pending[u] -= 1
+            if pending[u] == 0:
+                heapq.heappush(ready, (rank[u], u))
+    return order
+
+
+def _producers(nodes):
+    producer = {}
+    for i, n in enumerate(nodes):
+        for t in n["output_index"]:
+            producer[t] = i
+    return producer
+
+
+def _sorted_as_constructed(g):
+    """The nodes in the order the reference's graph constructor creates them (their ids)."""
+    nodes = g["nodes"]
+    producer = _producers(nodes)
+    for n in nodes:
+        for t in n["input_index"]:
+            if t not in producer:
+                raise ValueError("Node '%s': Unknown input node '%s'" % (
+                    n["name"], g["tensor_names"][t] if 0 <= t < len(g["tensor_names"]) else t))
+    order = _topological(len(nodes), lambda i: [producer[t] for t in nodes[i]["input_index"]],
+                         list(range(len(nodes))))
+    if len(order) != len(nodes):
+        raise ValueError("the graph has a cycle: %d of %d nodes can be ordered" % (len(order), len(nodes)))
+    return [nodes[i] for i in order]
+
+
+def _emit(g, ids):
+    """Graph::ToGraphDef: nodes in topological order by smallest id, isolated nodes that are not
+    outputs dropped, tensors renumbered in emission order (a tensor keeps its name)."""
+    nodes = g["nodes"]
+    producer = _producers(nodes)
+    order = _topological(len(nodes), lambda i: [producer[t] for t in nodes[i]["input_index"]], ids)
+    if len(order) != len(nodes):
+        raise ValueError("the folded graph has a cycle")
+    consumed = set(t for n in nodes for t in n["input_index"])
+    targets = set(g["output_names"])
+    renumber, names, out = {}, [], []
+    for i in order:
+        n = nodes[i]
+        dead = not n["input_index"] and not any(t in consumed for t in n["output_index"])
+        if dead and n["name"] not in targets and \
+                not any(g["tensor_names"][t] in targets for t in n["output_index"]):
+            continue
+        for t in n["output_index"]:
+            renumber[t] = len(names)
+            names.append(g["tensor_names"][t])
+        out.append(n)
+    for n in out:
+        n["input_index"] = [renumber[t] for t in n["input_index"]]
+        n["output_index"] = [renumber[t] for t in n["output_index"]]
+    g["nodes"], g["tensor_names"] = out, names
+
+
 def remap(model_bytes):
     """Returns (new model bytes, number of BatchNormalization nodes folded, number of
     activations folded)."""
     model = dlx.decode_model(model_bytes)
     g = model["graph"]
-    nodes = g["nodes"]
+    nodes = g["nodes"] = _sorted_as_constructed(g)
     producer = {}
     consumers = defaultdict(list)
     for i, n in enumerate(nodes):
@@ -88,7 +183,7 @@ def remap(model_bytes):
         return i
 
     deleted = set()
-    new_consts = {}   # conv node index -> Const node to insert in front of it
+    new_consts = []   # Const nodes made by the pass, in the order they were made
     folded_bn = folded_act = 0
     for i in range(len(nodes) - 1, -1, -1):
         if i in deleted:
@@ -141,7 +236,7 @@ def remap(model_bytes):
             g["tensor_names"].append(name)
             const = dict(name=name, type="Const", input_index=[], output_index=[index], attr={})
             const["attr"][dlx.ATTR_CONST] = dlx._sub(1, dlx.encode_tensor(shift, [o], dlx.ANY, dlx.ANY4))
-            new_consts[conv_i] = const
+            new_consts.append(const)
             conv["input_index"].append(index)
         last = nodes[act] if act is not None else bn
         if act is not None:
@@ -162,15 +257,8 @@ def remap(model_bytes):
         deleted.add(bn_i)
         deleted.update(params)
         folded_bn += 1
-        # the convolution now produces the pattern's last tensor: it must not run before
-        # nodes that used to sit between it and the end of the pattern need nothing from
-        # it, and its new position stays where it was, ahead of every consumer
-    out_nodes = []
-    for i, n in enumerate(nodes):
-        if i in deleted:
-            continue
-        if i in new_consts:
-            out_nodes.append(new_consts[i])
-        out_nodes.append(n)
-    g["nodes"] = out_nodes
+    # ids: a node of the file keeps its place in construction order, a made constant follows them
+    kept = [(i, n) for i, n in enumerate(nodes) if i not in deleted]
+    g["nodes"] = [n for _, n in kept] + new_consts
+    _emit(g, [i for i, _ in kept] + [len(nodes) + j for j in range(len(new_consts))])
     return encode_model(model), folded_bn, folded_act

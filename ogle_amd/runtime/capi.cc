@@ -144,6 +144,13 @@ int32_t ogle_rt_run(OgleSession* s, int32_t n_inputs, const char* const* names,
   });
 }
 
+int64_t ogle_rt_host_elements(const int32_t* dims, int32_t rank, const char* dformat) {
+  return Guard([&]() -> int64_t {
+    opengl::IntList shape(dims, dims + rank);
+    return (int64_t)opengl::HostElements(shape, opengl::StrToFormat(dformat));
+  });
+}
+
 int32_t ogle_rt_compute(OgleSession* s) {
   return (int32_t)Guard([&]() -> int64_t {
     s->session->Compute();

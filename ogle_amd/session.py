@@ -26,7 +26,7 @@ SYMBOLS = [
     "ogle_rt_set_reorder", "ogle_rt_issue_order_name", "ogle_rt_set_device_nms",
     "ogle_rt_detect_results", "ogle_rt_graph_captured", "ogle_rt_hazard_conflicts",
     "ogle_rt_set_fuse_siblings", "ogle_rt_launch_plan", "ogle_rt_launch_plan_entry",
-    "ogle_rt_conv_hazard_conflicts",
+    "ogle_rt_conv_hazard_conflicts", "ogle_rt_host_elements",
 ]
 
 
@@ -60,6 +60,8 @@ def lib():
         l.ogle_rt_run.argtypes = [vp, i32, ctypes.POINTER(cp), ctypes.POINTER(vp),
                                   ctypes.POINTER(ctypes.POINTER(i32)), ctypes.POINTER(i32),
                                   ctypes.POINTER(cp)]
+        l.ogle_rt_host_elements.argtypes = [ctypes.POINTER(i32), i32, cp]
+        l.ogle_rt_host_elements.restype = i64
         l.ogle_rt_compute.argtypes = [vp]
         l.ogle_rt_compute_graph.argtypes = [vp]
         l.ogle_rt_sync.argtypes = [vp]
@@ -186,6 +188,13 @@ class PinnedBuffer:
         self.close()
 
 
+def host_elements(shape, dformat):
+    """Floats a host buffer of logical shape `shape` holds in layout `dformat` (the dense
+    product for NHWC / NCHW / ANY, the stride-4 padded sizes for NHWC4 / ANY4 / HWN4C4)."""
+    dims = (ctypes.c_int32 * max(len(shape), 1))(*shape)
+    return _check(lib().ogle_rt_host_elements(dims, len(shape), dformat.encode()))
+
+
 class Session:
     def __init__(self):
         self._h = lib().ogle_rt_session_create()
@@ -229,6 +238,15 @@ class Session:
         c_ranks = (ctypes.c_int32 * n)(*[len(sh) for sh in logical])
         fm = [(dformats or {}).get(nm, "NHWC" if a.ndim == 4 else "ANY") for nm, a in zip(names, arrs)]
         c_fm = (ctypes.c_char_p * n)(*[f.encode() for f in fm])
+        # the runtime reads host_elements(logical shape, tag) floats from each buffer: a dense
+        # array under a padded tag (or any other size mismatch) would be read past its end
+        for nm, a, d, sh, f in zip(names, arrs, dims, logical, fm):
+            need = host_elements(sh, f)
+            if a.size != need:
+                raise ValueError("input %r: layout %s of logical shape %s takes %d floats, the array "
+                                 "holds %d%s" % (nm, f, sh, need, a.size,
+                                                 "" if (shapes or {}).get(nm) is not None or not f.endswith("4")
+                                                 else " (pass the logical shape in `shapes`)"))
         _check(lib().ogle_rt_run(self._h, n, c_names, c_data, c_dims, c_ranks, c_fm))
 
     def compute(self, graph=False):
@@ -289,9 +307,14 @@ class Session:
         n = _check(lib().ogle_rt_launch_plan(self._h, 1 if with_detect else 0))
         out = []
         label, k = ctypes.c_char_p(), ctypes.c_int32()
-        us = (ctypes.c_float * 64)()
+        cap = 64
+        us = (ctypes.c_float * cap)()
         for i in range(n):
-            _check(lib().ogle_rt_launch_plan_entry(self._h, i, ctypes.byref(label), ctypes.byref(k), us, 64))
+            _check(lib().ogle_rt_launch_plan_entry(self._h, i, ctypes.byref(label), ctypes.byref(k), us, cap))
+            if k.value > cap:  # an entry with more device operations than the buffer: read it again
+                cap = k.value
+                us = (ctypes.c_float * cap)()
+                _check(lib().ogle_rt_launch_plan_entry(self._h, i, ctypes.byref(label), ctypes.byref(k), us, cap))
             out.append((label.value.decode(), [float(v) for v in us[:k.value]] if durations else int(k.value)))
         return out
 

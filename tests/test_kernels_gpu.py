@@ -614,6 +614,61 @@ def test_config4_heads_concat_decode():
         np.testing.assert_array_equal(res[b]["cls"], ora[b]["cls"])
 
 
+def test_config4_chained_at_batch64():
+    """BASELINE config 4 at its full batch of 64, chained: the twelve heads as one grouped call
+    -> the two concatenations -> decode + softmax-max + score filter, every stage fed with the
+    device's output of the stage before.  The head convolutions are held to a float64 im2col
+    product (the scalar oracle would take minutes at this size); concat, decode and the score
+    filter to the oracle on the device's own inputs."""
+    import ctypes
+    import torch
+    from util import pack_filter
+    r = rng(20240004)
+    batch = 64
+    keep, heads = [], []
+    args = (H.ConvArgs * 12)()
+    for mi, (m, c, a) in enumerate(C4_MAPS):
+        f = r.uniform(0, 6, (batch, m, m, c)).astype(np.float32)
+        fd = torch.from_numpy(f).cuda()
+        for hi, last in enumerate((4, 21)):
+            o = a * last
+            wt = r.normal(0, 0.01, (o, c, 3, 3)).astype(np.float32)
+            wd = pack_filter(wt, H.FILTER_OHWI)
+            y = torch.full((batch, m, m, o), float("nan"), device="cuda")
+            ar = H.conv_args(fd.data_ptr(), wd.data_ptr(), None, y.data_ptr(), batch, m, m, c, o, 3, 1, 1)
+            need = H.lib().ogle_hip_conv_workspace_bytes(ctypes.byref(ar))
+            if need:
+                ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+                ar.workspace_dev, ar.workspace_bytes = ws.data_ptr(), need
+                keep.append(ws)
+            args[mi * 2 + hi] = ar
+            keep += [fd, wd]
+            heads.append((m, a, last, f, wt, y))
+    H.check(H.lib().ogle_hip_conv2d_batch(args, 12, 0))
+    torch.cuda.synchronize()
+    locs, confs = [], []
+    for m, a, last, f, wt, y in heads:
+        got = y.cpu().numpy()
+        assert_conv_close(got, _conv3x3_f64(f, wt).astype(np.float32), _conv3x3_f64(np.abs(f), np.abs(wt)),
+                          FP32_RTOL, "C4 b64 chained head %dx%d x%d" % (m, m, last))
+        (locs if last == 4 else confs).append(got.reshape(batch, m * m * a, last))
+    loc, conf = gpu_concat(locs, 1), gpu_concat(confs, 1)
+    np.testing.assert_array_equal(loc, O.concat(locs, 1))
+    np.testing.assert_array_equal(conf, O.concat(confs, 1))
+    assert loc.shape == (batch, 1917, 4) and conf.shape == (batch, 1917, 21)
+    anchors = ssd_anchors()
+    res, boxes = gpu_detect(conf, loc, anchors, 0.3, 300.0, 300.0)
+    np.testing.assert_allclose(boxes, O.ssd_decode(loc, anchors), rtol=0, atol=1e-4)
+    ora = O.box_info(conf, boxes, 0.3, 300.0, 300.0)
+    kept = 0
+    for b in range(batch):
+        assert_same_detections(res[b], ora[b], conf[b], 0.3, "C4 b64 image %d" % b)
+        np.testing.assert_array_equal(res[b]["prior"], ora[b]["prior"])
+        np.testing.assert_array_equal(res[b]["cls"], ora[b]["cls"])
+        kept += len(ora[b]["prior"])
+    assert kept > batch  # the threshold keeps a good share of the priors at these logits
+
+
 @pytest.mark.parametrize("batch", [1, 64])
 def test_detect_kept_sets_bit_exact(batch):
     """Logits scaled so that a few percent of the priors pass the threshold."""
@@ -869,6 +924,39 @@ def test_detect_lists_in_place_then_topk_nms(batch, priors, topk, sigma):
     # in-place lists need every list
     da.kept_rect_dev = None
     assert H.lib().ogle_hip_ssd_detect(ctypes.byref(da), st) == H.ERR_INVALID_ARG
+
+
+def test_topk_nms_known_answers_on_device():
+    """The hand-built cases of tests/test_oracle.py::test_topk_nms_known_answers on the device,
+    with the answers written out (not taken from the oracle): a dropped box still drops a later
+    one (detector.cc:127-148), top-k cuts before the suppression, equal scores keep prior order."""
+    A, B, C, D = (0, 0, 100, 100), (30, 0, 100, 100), (60, 0, 100, 100), (300, 300, 50, 50)
+    cases = [  # rects, scores, topk -> surviving input positions, in sorted order
+        ([A, B, C, D], [0.9, 0.8, 0.7, 0.6], 100, [0, 3]),
+        ([C, D, A, B], [0.7, 0.6, 0.9, 0.8], 100, [2, 1]),
+        ([A, C, D], [0.9, 0.7, 0.6], 100, [0, 1, 2]),
+        ([A, B, C, D], [0.9, 0.8, 0.7, 0.6], 2, [0]),
+        ([A, B, D], [0.8, 0.8, 0.8], 100, [0, 2]),
+        ([B, A, D], [0.8, 0.8, 0.8], 100, [0, 2]),
+        ([D, B, A], [0.8, 0.8, 0.8], 2, [0, 1]),
+    ]
+    stride = 4
+    for topk in (100, 2):
+        sel = [c for c in cases if c[2] == topk]
+        batch = len(sel)
+        counts = np.array([len(c[0]) for c in sel], np.int32)
+        rect = np.zeros((batch, stride, 4), np.int32)
+        score = np.zeros((batch, stride), np.float32)
+        prior = np.tile(np.arange(stride, dtype=np.int32) * 10 + 3, (batch, 1))
+        cls = np.tile(np.arange(1, stride + 1, dtype=np.int32), (batch, 1))
+        for b, (rc, sc, _, _) in enumerate(sel):
+            rect[b, :len(rc)] = rc
+            score[b, :len(sc)] = sc
+        got = gpu_topk_nms(counts, prior, cls, score, rect, topk, 0.45)
+        for b, (_, _, _, expect) in enumerate(sel):
+            np.testing.assert_array_equal(got[b]["prior"], prior[b][expect])
+            np.testing.assert_array_equal(got[b]["cls"], cls[b][expect])
+            np.testing.assert_array_equal(got[b]["rect"], rect[b][expect])
 
 
 def test_topk_nms_rejects_bad_sizes():

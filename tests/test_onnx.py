@@ -207,6 +207,19 @@ def test_errors():
         onnx.convert(b"")
 
 
+def test_initializer_with_a_zero_dimension_is_an_empty_tensor():
+    """A tensor whose dims hold a zero has no data fields at all; it converts to an empty
+    constant (MakeTensorFromProto copies `count` = 0 values) instead of being refused."""
+    w = WRITERS["proto2"]
+    x = [w.value_info("x", [1, 4, 4, 4])]
+    model = onnx.convert(w.model([w.node("Concat", ["x", "e"], ["y"], axis=1)], x, [],
+                                 [w.tensor("e", np.zeros((0, 4), np.float32))]))
+    nodes = {n["name"]: n for n in dlx.decode_model(model)["graph"]["nodes"]}
+    (field, _, payload), = list(dlx._fields(nodes["e"]["attr"][dlx.ATTR_CONST]))
+    t = dlx.decode_tensor(payload)
+    assert t["dims"] == [0, 4] and len(t["float_data"]) == 0
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("fold", [False, True])
 def test_separable_block_onnx_to_device(fold):

@@ -311,6 +311,40 @@ def test_topk_nms_against_python_restatement():
         np.testing.assert_array_equal(O.topk_nms(scores, rects, top_k, 0.45), expect)
 
 
+def test_topk_nms_known_answers():
+    """Hand-built cases with the answer worked out on paper (detector.cc:114-148, common.cc:57-77).
+    Boxes are (x, y, w, h), 100 x 100 each.  IoU of two such boxes shifted by d along x is
+    (100 - d) / (100 + d): 0.538 for d = 30, 0.25 for d = 60."""
+    A, B, C, D = (0, 0, 100, 100), (30, 0, 100, 100), (60, 0, 100, 100), (300, 300, 50, 50)
+    # The reference's rule: B (dropped by A) still drops C although A and C overlap by 0.25 only;
+    # a textbook greedy NMS would keep C.
+    rects = np.array([A, B, C, D], np.int32)
+    scores = np.array([0.9, 0.8, 0.7, 0.6], np.float32)
+    np.testing.assert_array_equal(O.topk_nms(scores, rects, 100, 0.45), [0, 3])
+    # same boxes, input order shuffled: the sort by score decides, results are input positions
+    perm = [2, 3, 0, 1]                       # input = C, D, A, B
+    np.testing.assert_array_equal(O.topk_nms(scores[perm], rects[perm], 100, 0.45), [2, 1])
+    # without B the chain is broken and C survives
+    keep = [0, 2, 3]
+    np.testing.assert_array_equal(O.topk_nms(scores[keep], rects[keep], 100, 0.45), [0, 1, 2])
+    # the threshold is strict: IoU(A, B) = 70 / 130 exactly as the host computes it in binary32
+    thr = np.float32(np.float32(7000.0) / np.float32(13000.0))
+    np.testing.assert_array_equal(O.topk_nms(scores[:2], rects[:2], 100, float(thr)), [0, 1])
+    np.testing.assert_array_equal(O.topk_nms(scores[:2], rects[:2], 100, float(np.nextafter(thr, np.float32(0)))), [0])
+    # top-k cuts before the suppression: with k = 2 only A and B are looked at, D never appears
+    np.testing.assert_array_equal(O.topk_nms(scores, rects, 2, 0.45), [0])
+    # equal scores keep their input order (the defined choice for std::sort's ties), so the
+    # earlier of two overlapping boxes wins whichever it is
+    eq = np.array([0.8, 0.8, 0.8], np.float32)
+    np.testing.assert_array_equal(O.topk_nms(eq, np.array([A, B, D], np.int32), 100, 0.45), [0, 2])
+    np.testing.assert_array_equal(O.topk_nms(eq, np.array([B, A, D], np.int32), 100, 0.45), [0, 2])
+    np.testing.assert_array_equal(O.topk_nms(eq, np.array([D, B, A], np.int32), 2, 0.45), [0, 1])
+    # degenerate rectangles: zero area on both sides gives u <= 0 -> IoU 0, nothing is dropped
+    z = np.array([(5, 5, 0, 0), (5, 5, 0, 0)], np.int32)
+    np.testing.assert_array_equal(O.topk_nms(eq[:2], z, 100, 0.45), [0, 1])
+    assert len(O.topk_nms(np.zeros(0, np.float32), np.zeros((0, 4), np.int32), 100, 0.45)) == 0
+
+
 def test_elementwise_against_numpy():
     r = rng(90)
     a = r.normal(0, 2, (3, 5, 7, 6)).astype(np.float32)

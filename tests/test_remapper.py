@@ -53,15 +53,24 @@ def test_remap_structure_and_folded_values():
     by_name = {n["name"]: n for n in after["graph"]["nodes"]}
     # fused nodes carry the name and the output tensor of the pattern's last node
     assert by_name["c1.act"]["type"] == "Conv" and by_name["c2.bn"]["type"] == "Conv"
+    # ... under the name that tensor had (tensors are renumbered in emission order)
     old = {n["name"]: n for n in before["graph"]["nodes"]}
-    assert by_name["c1.act"]["output_index"] == old["c1.act"]["output_index"]
+    names_before, names_after = before["graph"]["tensor_names"], after["graph"]["tensor_names"]
+    assert names_after[by_name["c1.act"]["output_index"][0]] == names_before[old["c1.act"]["output_index"][0]]
+    assert [names_after[n["output_index"][0]] for n in after["graph"]["nodes"]] == names_after
     a1 = dlx.decode_conv2d_attr(by_name["c1.act"]["attr"][dlx.ATTR_CONV2D])
     assert (a1["activation_type"], a1["min"], a1["max"]) == ("Clip", 0.0, 6.0)
     assert dlx.decode_conv2d_attr(by_name["c2.bn"]["attr"][dlx.ATTR_CONV2D])["activation_type"] == ""
-    # c1 had no bias: a Const was made, in front of the node, as its third input
+    # c1 had no bias: a Const was made, as its third input.  Its id follows every node of the
+    # file, so Graph::ToGraphDef (graph.cc:12-54) writes all other constants first, then the made
+    # bias, then the convolutions, which could not start before it; the folded BatchNormalization
+    # parameters (no consumer left) are gone, and the tensor list is dense again
     assert len(by_name["c1.act"]["input_index"]) == 3 and "c1:2" in by_name
     order = [n["name"] for n in after["graph"]["nodes"]]
-    assert order.index("c1:2") < order.index("c1.act")
+    assert order == ["input", "c1.w", "c2.w", "c2.b", "c3.w", "c3.b", "c1:2",
+                     "c1.act", "c2.bn", "sum", "sum.act", "c3.bn"]
+    assert len(names_after) == len(order)
+    assert after["graph"]["output_names"] == ["c3.bn"] and after["graph"]["input_names"] == ["input"]
     # folded numbers are those of the reference's formula (the oracle restates it)
     for conv, fused in (("c1", "c1.act"), ("c2", "c2.bn"), ("c3", "c3.bn")):
         w, b, (g, bt, mu, var) = weights[conv]
@@ -72,6 +81,43 @@ def test_remap_structure_and_folded_values():
         got_b = remapper._const_tensor(tensors[node["input_index"][2]])["float_data"]
         np.testing.assert_allclose(got_w, wf, rtol=1e-6, atol=1e-7)
         np.testing.assert_allclose(got_b, bf, rtol=1e-6, atol=1e-7)
+
+
+def test_remap_sorts_an_out_of_order_graph():
+    """A file whose nodes are not in topological order (a consumer written before its producer):
+    the graph constructor orders them (graph_constructor.cc:144-190, smallest file position
+    among the ready nodes first), so the result is executable in file order and equals the
+    result for the sorted file, node for node."""
+    r = rng(30002)
+    gb, _ = residual_graph(r)
+    model = dlx.decode_model(gb.serialize())
+    nodes = model["graph"]["nodes"]
+    pos = {n["name"]: i for i, n in enumerate(nodes)}
+    # move the first convolution behind its batchnorm and the Add in front of everything
+    shuffled = list(nodes)
+    shuffled.insert(0, shuffled.pop(pos["sum"]))
+    c1 = next(i for i, n in enumerate(shuffled) if n["name"] == "c1")
+    shuffled.insert(c1 + 6, shuffled.pop(c1))
+    assert [n["name"] for n in shuffled] != [n["name"] for n in nodes]
+    model["graph"]["nodes"] = shuffled
+    out_shuffled, n_bn, n_act = remapper.remap(remapper.encode_model(model))
+    out_sorted, _, _ = remapper.remap(gb.serialize())
+    assert (n_bn, n_act) == (3, 1)
+    a, b = dlx.decode_model(out_shuffled)["graph"], dlx.decode_model(out_sorted)["graph"]
+    seen = set()
+    for n in a["nodes"]:                       # every input is produced by an earlier node
+        assert all(t in seen for t in n["input_index"]), n["name"]
+        seen.update(n["output_index"])
+    assert sorted(n["name"] for n in a["nodes"]) == sorted(n["name"] for n in b["nodes"])
+    bn = {n["name"]: n for n in b["nodes"]}
+    for n in a["nodes"]:
+        assert n["type"] == bn[n["name"]]["type"] and n["attr"] == bn[n["name"]]["attr"]
+        assert [a["tensor_names"][t] for t in n["input_index"]] == \
+            [b["tensor_names"][t] for t in bn[n["name"]]["input_index"]]
+    # a reference to a tensor nobody produces is fatal, as in the reference
+    model["graph"]["nodes"] = [n for n in shuffled if n["name"] != "c2.w"]
+    with pytest.raises(ValueError, match="Unknown input node 'c2.w'"):
+        remapper.remap(remapper.encode_model(model))
 
 
 def test_remap_leaves_shared_or_activated_patterns_alone():

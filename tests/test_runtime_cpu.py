@@ -140,6 +140,31 @@ def test_runtime_exports_every_declared_symbol():
         assert getattr(lib, name) is not None
 
 
+def test_host_elements_and_input_size_check():
+    """Sizes of the host layouts (tensor_format.cc:251-343) and the check Session.run makes with
+    them: a dense array handed over under a padded tag would be read past its end."""
+    assert session.host_elements((2, 5, 7, 3), "NHWC") == 210
+    assert session.host_elements((2, 5, 7, 3), "NCHW") == 210
+    assert session.host_elements((2, 5, 7, 3), "NHWC4") == 2 * 5 * 7 * 4
+    assert session.host_elements((2, 5, 7, 8), "NHWC4") == 2 * 5 * 7 * 8
+    assert session.host_elements((6, 1917, 21), "ANY4") == 6 * 1917 * 24
+    assert session.host_elements((5,), "ANY4") == 8
+    assert session.host_elements((5,), "ANY") == 5
+    # OIHW (13, 6, 3, 3): 9 * ceil(13/4) rows of 4 * ceil(6/4) texels of 4 lanes
+    assert session.host_elements((13, 6, 3, 3), "HWN4C4") == 9 * 4 * 8 * 4
+    with pytest.raises(RuntimeError, match="unsupported dformat"):
+        session.host_elements((1, 2), "NC4HW4")
+    with pytest.raises(RuntimeError, match="rank-4"):
+        session.host_elements((3, 3), "NHWC4")
+    s = session.Session()
+    s.load_graph(_small_graph())
+    x = np.zeros((1, 8, 8, 3), np.float32)
+    with pytest.raises(ValueError, match=r"layout NHWC4 .* takes 256 floats, the array holds 192"):
+        s.run({"input": x}, dformats={"input": "NHWC4"})
+    with pytest.raises(ValueError, match="takes 192 floats, the array holds 256"):
+        s.run({"input": np.zeros((1, 8, 8, 4), np.float32)}, shapes={"input": (1, 8, 8, 3)})
+
+
 def test_registered_op_types():
     names = session.registered_kernels()
     for op in ["Conv", "MaxPool", "AveragePool", "GlobalAveragePool", "Concat", "Decoder", "Const",

@@ -225,27 +225,25 @@ def _run_ssd(batch, seed=20240005):
     return sess, info, x
 
 
-def test_mobilenet_ssd_every_layer_matches_oracle():
-    """Full MobileNet-v1 SSD 300x300, batch 1: every conv layer is checked against the oracle
-    applied to the DEVICE's input of that layer, so each of the 47 convolutions is held to the
-    fp32 tolerance on its own (errors do not compound across the check)."""
-    sess, info, x = _run_ssd(1)
-    produced = {"input": x}
+def _check_every_layer(sess, info, x, images):
+    """Every conv layer of the network against the oracle applied to the DEVICE's input of that
+    layer, for the listed images of the batch, so each of the 47 convolutions is held to the fp32
+    tolerance on its own (errors do not compound across the check).  Returns the device's outputs
+    (those images only) by layer name and the worst normwise error."""
+    images = list(images)
+    produced = {"input": x[images]}
     prev = "input"
     feature_of = {}
     worst = 0.0
     for l in info["layers"]:
         name = l["name"]
-        if name.startswith("head"):
-            src = feature_of[int(name[4])]
-        else:
-            src = prev
+        src = feature_of[int(name[4])] if name.startswith("head") else prev
         xin = produced[src]
         w, b = info["weights"][name]
         act = O.ACT_CLIP if l["act"] else O.ACT_NONE
         variant = O.VARIANT_PW if l["kind"] == "pw" else O.VARIANT_NHWC4
         ref = O.conv2d(xin, w, b, l["stride"], l["pad"], 1, l["group"], act, 0.0, 6.0, variant)
-        got = sess.get_output(name, "NHWC")
+        got = np.ascontiguousarray(sess.get_output(name, "NHWC")[images])
         worst = max(worst, assert_conv_close(got, ref, O.conv2d_abs(xin, w, b, l["stride"], l["pad"], 1,
                                                                     l["group"]), FP32_RTOL, name))
         produced[name] = got
@@ -256,6 +254,14 @@ def test_mobilenet_ssd_every_layer_matches_oracle():
             if name.startswith("extra") and name.endswith(".conv"):
                 feature_of[int(name[5]) + 1] = name
     assert 0.0 < worst <= FP32_RTOL
+    return produced, worst
+
+
+def test_mobilenet_ssd_every_layer_matches_oracle():
+    """Full MobileNet-v1 SSD 300x300, batch 1: each of the 47 convolutions against the oracle on
+    the device's own input of that layer, then the concatenations and the anchors."""
+    sess, info, x = _run_ssd(1)
+    produced, worst = _check_every_layer(sess, info, x, [0])
     print("47 layers, worst |err| / sum|x||w| = %.3g" % worst)
     loc = sess.get_output("box_preds", "ANY")
     conf = sess.get_output("cls_logits", "ANY")
@@ -265,6 +271,29 @@ def test_mobilenet_ssd_every_layer_matches_oracle():
     np.testing.assert_array_equal(
         conf, np.concatenate([produced["head%d.conf" % i].reshape(1, -1, 21) for i in range(6)], 1))
     np.testing.assert_array_equal(sess.get_output("anchors", "ANY"), info["anchors"])
+
+
+def test_mobilenet_ssd_batch16_every_layer_matches_oracle():
+    """The headline configuration (batch 16) runs other kernels than batch 1: 64x64 LDS tiles
+    instead of the wave-split kernel, the twelve heads as one grid with their K split, outputs
+    stored an image stride apart inside the concatenations.  Each of the 47 convolutions is held
+    to the oracle on the device's own input of that layer, for the first and the last image of the
+    batch (the oracle takes those two images only), and the concatenations to the heads' outputs."""
+    sess, info, x = _run_ssd(16)
+    images = [0, 15]
+    produced, worst = _check_every_layer(sess, info, x, images)
+    print("batch 16, 47 layers x 2 images, worst |err| / sum|x||w| = %.3g" % worst)
+    loc = sess.get_output("box_preds", "ANY")
+    conf = sess.get_output("cls_logits", "ANY")
+    assert loc.shape == (16, 1917, 4) and conf.shape == (16, 1917, 21)
+    np.testing.assert_array_equal(
+        loc[images], np.concatenate([produced["head%d.loc" % i].reshape(2, -1, 4) for i in range(6)], 1))
+    np.testing.assert_array_equal(
+        conf[images], np.concatenate([produced["head%d.conf" % i].reshape(2, -1, 21) for i in range(6)], 1))
+    # and the replayed pass (hipGraph) gives what the eager pass gave
+    sess.compute(graph=True)
+    np.testing.assert_array_equal(sess.get_output("box_preds", "ANY"), loc)
+    np.testing.assert_array_equal(sess.get_output("cls_logits", "ANY"), conf)
 
 
 def test_concat_inputs_are_produced_in_place_at_batch1():

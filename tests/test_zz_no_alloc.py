@@ -58,19 +58,42 @@ def test_noalloc_matches_workspace_entry_two_calls_in_a_row():
     assert needs[0] > needs[1] > 0 and needs[0] <= H.CONV_NOALLOC_SCRATCH_BYTES, needs
 
 
+def _oversized_problem():
+    """A convolution whose split-K plan wants more scratch than the built-in array holds: SSD
+    class heads on the 19x19 map, the batch doubled until the plan is too large."""
+    import torch
+    h, c, o = 19, 512, 126
+    for n in (64, 128, 256):
+        x = torch.zeros((n, h, h, c), device="cuda")
+        w = torch.zeros((o, 3, 3, c), device="cuda")
+        y = torch.zeros((n, h, h, o), device="cuda")
+        args = H.conv_args(x.data_ptr(), w.data_ptr(), None, y.data_ptr(), n, h, h, c, o, 3, 1, 1)
+        need = H.lib().ogle_hip_conv_workspace_bytes(ctypes.byref(args))
+        if need > H.CONV_NOALLOC_SCRATCH_BYTES:
+            return args, need, (x, w, y)
+    raise AssertionError("no plan exceeds the built-in scratch: pick another shape for this test")
+
+
 def test_noalloc_refuses_oversized_and_caller_workspace():
     import torch
-    # SSD class head at batch 64 on the 19x19 map: the split-K plan wants far more than 16 MiB
-    n, h, c, o = 64, 19, 512, 126
-    x = torch.zeros((n, h, h, c), device="cuda")
-    w = torch.zeros((o, 3, 3, c), device="cuda")
-    y = torch.zeros((n, h, h, o), device="cuda")
-    args = H.conv_args(x.data_ptr(), w.data_ptr(), None, y.data_ptr(), n, h, h, c, o, 3, 1, 1)
-    need = H.lib().ogle_hip_conv_workspace_bytes(ctypes.byref(args))
-    if need > H.CONV_NOALLOC_SCRATCH_BYTES:
-        st = H.lib().ogle_hip_conv2d_noalloc(ctypes.byref(args), U.stream_ptr())
-        assert st == H.ERR_INVALID_ARG
-        assert str(need) in H.last_error() and str(H.CONV_NOALLOC_SCRATCH_BYTES) in H.last_error()
-    args.workspace_dev, args.workspace_bytes = y.data_ptr(), 16
+    args, need, keep = _oversized_problem()
+    assert need > H.CONV_NOALLOC_SCRATCH_BYTES
+    st = H.lib().ogle_hip_conv2d_noalloc(ctypes.byref(args), U.stream_ptr())
+    assert st == H.ERR_INVALID_ARG
+    assert str(need) in H.last_error() and str(H.CONV_NOALLOC_SCRATCH_BYTES) in H.last_error()
+    # a caller workspace is refused: a pointer with a size, and a size without a pointer
+    args.workspace_dev, args.workspace_bytes = keep[2].data_ptr(), 16
+    assert H.lib().ogle_hip_conv2d_noalloc(ctypes.byref(args), U.stream_ptr()) == H.ERR_INVALID_ARG
+    args.workspace_dev, args.workspace_bytes = None, 4096
     assert H.lib().ogle_hip_conv2d_noalloc(ctypes.byref(args), U.stream_ptr()) == H.ERR_INVALID_ARG
     torch.cuda.synchronize()
+    # refused calls launched nothing and left the scratch alone: two good calls right after
+    # them on the same stream still equal the workspace entry bit for bit
+    r = U.rng(4243)
+    for (n, h, w, c, o, k, s, p) in CASES[:2]:
+        x = r.uniform(-1, 1, (n, h, w, c)).astype(np.float32)
+        wt = r.normal(0, np.sqrt(2.0 / (k * k * c)), (o, c, k, k)).astype(np.float32)
+        b = r.uniform(-0.1, 0.1, o).astype(np.float32)
+        got, _ = _run("ogle_hip_conv2d_noalloc", x, wt, b, s, p, False)
+        ref, _ = _run("ogle_hip_conv2d", x, wt, b, s, p, True)
+        assert np.array_equal(got, ref), (n, h, w, c, o, k)
