@@ -160,16 +160,20 @@ def read_traffic_summary(kernel_family):
     return None
 
 
-def kernel_table(iters=50, warm=5):
+def kernel_table(iters=50, warm=5, only=None):
     """Each kernel of the path on its own, at the shapes the baseline configurations name,
     called through the C ABI on torch's current stream and timed with events on that stream.
-    FLOPs = 2 x multiply-adds; bytes = input + weights + bias + output once each."""
+    FLOPs = 2 x multiply-adds; bytes = input + weights + bias + output once each.
+    `only`: run just the rows whose name contains this text (for a profiler run of one kernel)."""
     import ctypes
     import torch
     from ogle_amd import hip as H
     L = H.lib()
     st = torch.cuda.current_stream().cuda_stream
     rows = []
+
+    def want(name):
+        return only is None or only in name
 
     def timed(fn):
         for _ in range(warm):
@@ -212,6 +216,8 @@ def kernel_table(iters=50, warm=5):
         return a, flops, nbytes, (x, wd, b, y, ws)
 
     def conv_row(name, entry, bound, *shape, peak=MFMA_F32_PEAK_TFLOPS, **kw):
+        if not want(name):
+            return
         a, flops, nbytes, keep = conv_problem(*shape, **kw)
         f = getattr(L, entry)
         row(name, timed(lambda: H.check(f(ctypes.byref(a), st))), flops, nbytes, bound, peak)
@@ -233,6 +239,11 @@ def kernel_table(iters=50, warm=5):
              32, 19, 19, 512, 1024, 1, 1, 0)
     conv_row("pointwise GEMM @C3 fp16 storage, fp32 accumulate", "ogle_hip_pwconv_gemm", "mfma",
              32, 19, 19, 512, 1024, 1, 1, 0, dtype=H.F16, peak=2500.0)
+
+    conv_row("pointwise GEMM fp16 storage, large (M=46208 K=1024 N=1024)", "ogle_hip_pwconv_gemm", "mfma",
+             128, 19, 19, 1024, 1024, 1, 1, 0, dtype=H.F16, peak=2500.0)
+    if only is not None:
+        return rows   # only the convolution rows can be picked one by one
 
     # yardstick for the two rows above: the vendor library's GEMM (torch.matmul -> hipBLASLt /
     # rocBLAS) on the same shape and types; a comparison figure, not part of the path
@@ -453,6 +464,9 @@ def main():
                     help="leave out the per-kernel leg at the single-kernel configurations")
     ap.add_argument("--skip-b1", action="store_true",
                     help="leave out the batch-1 latency leg (keeps a profiler trace to the batch-16 pass)")
+    ap.add_argument("--only-kernel", metavar="TEXT",
+                    help="run only the convolution rows of the per-kernel table whose name contains TEXT, "
+                         "--steps calls each after --warmup, and print them (for a profiler run of one kernel)")
     ap.add_argument("--profile-layers", metavar="PLAN.json",
                     help="only replay the pass --steps times as a hipGraph (after --warmup) and write the "
                          "pass's dispatch sequence to PLAN.json: run under `rocprofv3 --kernel-trace` and "
@@ -470,6 +484,10 @@ def main():
 
     if args.profile_layers:
         profile_layers_run(args)
+        return
+    if args.only_kernel:
+        print(json.dumps(dict(kernel_table=kernel_table(iters=args.steps, warm=args.warmup,
+                                                        only=args.only_kernel))))
         return
     use_graph = not args.eager
     streams = 1 if args.eager else max(1, min(args.streams, 16))

@@ -105,6 +105,10 @@ int32_t launch_conv_igemm(const OgleConvArgs& a, hipStream_t s);   // returns OG
 size_t conv_igemm_workspace_bytes(const OgleConvArgs& a);
 bool conv_igemm_takes(const OgleConvArgs& a);  // launch_conv_igemm would not return OGLE_ERR_UNSUPPORTED
 int32_t launch_conv_igemm_static_scratch(const OgleConvArgs& a, hipStream_t s);
+// fp16-storage pointwise GEMM with operands streamed straight into LDS: the tile
+// configuration it would run `a` with, or -1 if it does not take the shape.
+int f16_async_config(const OgleConvArgs& a);
+int32_t launch_pw_gemm_f16_async(const OgleConvArgs& a, hipStream_t s);
 // reduce_pending != nullptr: split-K reductions are not launched; reduce_pending[i] says
 // whether convolution i still needs launch_conv_reduce.
 int32_t launch_conv_batch(const OgleConvArgs* args, int count, hipStream_t s,

@@ -1311,12 +1311,14 @@ bool conv_igemm_takes(const OgleConvArgs& a) {
 size_t conv_igemm_workspace_bytes(const OgleConvArgs& a) {
   long m = 0;
   if (!igemm_eligible(a, &m)) return 0;
+  if (f16_async_config(a) >= 0) return 0;
   return plan_igemm(a, m, true).workspace_bytes;
 }
 
 int32_t launch_conv_igemm(const OgleConvArgs& a, hipStream_t s) {
   long m = 0;
   if (!igemm_eligible(a, &m)) return OGLE_ERR_UNSUPPORTED;
+  if (f16_async_config(a) >= 0) return launch_pw_gemm_f16_async(a, s);
   const IgemmPlan p = final_plan(a, m);
   const Prepared pr = prepare(a, m, p);
   const bool pw = is_pointwise(a);
@@ -1352,6 +1354,11 @@ int32_t launch_conv_batch(const OgleConvArgs* args, int count, hipStream_t s,
     long m = 0;
     if (!igemm_eligible(args[i], &m)) {
       const int32_t st = fallback(args[i], s);
+      if (st != OGLE_OK) return st;
+      continue;
+    }
+    if (f16_async_config(args[i]) >= 0) {  // fills the chip on its own: its own launch
+      const int32_t st = launch_pw_gemm_f16_async(args[i], s);
       if (st != OGLE_OK) return st;
       continue;
     }
@@ -1430,7 +1437,7 @@ int32_t launch_conv_reduce(const OgleConvArgs* args, int count, hipStream_t s) {
     int dtype = -1;
     for (; at < count && red.count < kMaxGroup; ++at) {
       long m = 0;
-      if (!igemm_eligible(args[at], &m)) continue;
+      if (!igemm_eligible(args[at], &m) || f16_async_config(args[at]) >= 0) continue;
       const IgemmPlan p = final_plan(args[at], m);
       if (p.splits <= 1) continue;
       if (dtype >= 0 && args[at].dtype != dtype) break;  // one storage type per grid
@@ -1498,7 +1505,7 @@ int32_t static_scratch(void** out) {
 int32_t launch_conv_igemm_static_scratch(const OgleConvArgs& a, hipStream_t s) {
   long m = 0;
   if (!igemm_eligible(a, &m)) return OGLE_ERR_UNSUPPORTED;  // the other kernels use no scratch
-  const size_t need = plan_igemm(a, m, true).workspace_bytes;
+  const size_t need = f16_async_config(a) >= 0 ? 0 : plan_igemm(a, m, true).workspace_bytes;
   if (need > (size_t)OGLE_CONV_NOALLOC_SCRATCH_BYTES) {
     set_error("conv2d_noalloc: this convolution's split-K plan needs %zu bytes of scratch, the "
               "built-in buffer holds %zu; use ogle_hip_conv2d with a caller workspace",

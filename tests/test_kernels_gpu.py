@@ -1019,6 +1019,50 @@ def test_fp16_wide_tile_large_pointwise():
                       "fp16 wide tile")
 
 
+ASYNC_F16_CASES = [
+    # n, h, w, c, o, bias, act, image stride beyond dense (elements)
+    (8, 64, 63, 264, 512, True, H.ACT_CLIP, 0),      # 256x256 tiles; ragged M; K ends inside a stage
+    (32, 19, 19, 512, 1000, True, H.ACT_RELU, 0),    # 192x256 tiles; ragged M and N (config 3's M, K)
+    (32, 19, 19, 256, 768, False, H.ACT_NONE, 64),   # no bias, images stored with a gap after each
+]
+
+
+@pytest.mark.parametrize("case", ASYNC_F16_CASES)
+def test_fp16_async_pointwise_gemm(case):
+    """fp16 storage, pointwise, at least 256 input channels and enough 256-wide tiles: the kernel
+    that streams its operands straight into LDS (256x256 / 192x256 tiles, eight waves in two
+    alternating groups).  Against a float64 product of the fp16-rounded operands; the first image
+    also against the oracle."""
+    n, h, w, c, o, with_bias, act, gap = case
+    r = rng(2800 + c)
+    x = r.uniform(0, 2, (n, h, w, c)).astype(np.float16).astype(np.float32)
+    wt = r.normal(0, np.sqrt(2 / c), (o, c, 1, 1)).astype(np.float16).astype(np.float32)
+    b = r.uniform(-0.1, 0.1, o).astype(np.float32) if with_bias else None
+    stride = h * w * o + gap if gap else 0
+    got = gpu_conv(x, wt, b, act=act, maxv=1.5, variant=H.VARIANT_PW, dtype=H.F16, image_stride=stride)
+    if gap:   # the gaps keep their NaN fill, the images are dense runs
+        got = got.reshape(n, stride)
+        assert np.isnan(got[:, h * w * o:]).all()
+        got = got[:, :h * w * o]
+    a64 = x.reshape(-1, c).astype(np.float64)
+    w64 = wt.reshape(o, c).astype(np.float64)
+    ref = a64 @ w64.T + (b if with_bias else 0.0)
+    if act == H.ACT_RELU:
+        ref = np.maximum(ref, 0)
+    elif act == H.ACT_CLIP:
+        ref = np.clip(ref, 0, 1.5)
+    ref = ref.astype(np.float32)
+    scale = np.abs(a64) @ np.abs(w64).T + (np.abs(b) if with_bias else 0.0)
+    half_ulp = 0.5 * 2.0 ** (np.floor(np.log2(np.maximum(np.abs(ref.astype(np.float64)), 2.0 ** -14))) - 10)
+    what = "fp16 async %s" % (case,)
+    assert_conv_close(got.reshape(-1, o), ref, (scale + half_ulp / FP16_RTOL).astype(np.float32), FP16_RTOL, what)
+    ora = O.conv2d(x[:1], wt, b, act={H.ACT_RELU: O.ACT_RELU, H.ACT_CLIP: O.ACT_CLIP, H.ACT_NONE: O.ACT_NONE}[act],
+                   maxv=1.5, variant=O.VARIANT_PW)
+    assert_conv_close(got.reshape(n, h, w, o)[:1], ora,
+                      (scale + half_ulp / FP16_RTOL)[:h * w].reshape(1, h, w, o).astype(np.float32), FP16_RTOL,
+                      what + " vs oracle")
+
+
 SPLIT_CASES = [
     # n, h, w, c, o1, o2, k, s, p, dtype       (output channels [0,o1) -> y, [o1,o1+o2) -> y2)
     (4, 19, 19, 128, 12, 63, 3, 1, 1, H.F32),      # SSD box + class head, 128x96 tile, element stores
