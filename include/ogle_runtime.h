@@ -240,6 +240,24 @@ int64_t ogle_rt_detect(OgleSession* s, const float* images, const int32_t* dims 
  */
 int64_t ogle_rt_detect_results(OgleSession* s, OgleDetection* out, int64_t capacity);
 
+/*
+ * ogle_rt_time_pipelined with the detector's work in every pass, and the host in the loop:
+ * every pass ends with ONE asynchronous copy of its final detection lists (a count and at
+ * most top-k records of 44 bytes per image, one device block) into page-locked host
+ * memory, recorded inside the captured graph.  The host never waits for a stream: before a
+ * session's next pass is launched it waits for the event behind that session's previous
+ * pass and reads its lists, while the other sessions' passes (and, with one session, nothing)
+ * are already enqueued.  `detections` receives the number of detections read in the timed
+ * passes.  The reference's timing loop reads its outputs back inside every run as well
+ * (nn/main.cc:76-111).  Needs top-k + NMS on the device (the default).
+ */
+int32_t ogle_rt_time_pipelined_readback(OgleSession** sessions, int32_t n, int32_t warmup,
+                                        int32_t iters, float* total_ms, int64_t* detections);
+/* The detections of the session's last pass launched by ogle_rt_time_pipelined_readback,
+ * read from the page-locked copy (waits for that pass's event if nobody has yet).  Same
+ * output convention as ogle_rt_detect. */
+int64_t ogle_rt_pipelined_results(OgleSession* s, OgleDetection* out, int64_t capacity);
+
 #ifdef __cplusplus
 }
 #endif

@@ -27,6 +27,13 @@ struct OgleSession {
   bool device_nms = true;
   std::vector<opengl::Context::LaunchRecord> plan;
   std::vector<float> plan_us;  // duration of every device operation of the plan, in order
+  // pipelined readback: the event behind the session's last pass whose final lists were
+  // copied to the detector's page-locked memory and have not been read yet
+  hipEvent_t lists_ready = nullptr;
+  bool lists_pending = false;
+  ~OgleSession() {
+    if (lists_ready != nullptr) (void)hipEventDestroy(lists_ready);
+  }
 };
 
 namespace {
@@ -534,6 +541,99 @@ int64_t ogle_rt_detect(OgleSession* s, const float* images, const int32_t* dims,
     Tensor input(Tensor::DT_FLOAT, shape, images, dlxnet::TensorProto::NHWC);
     std::vector<std::vector<opengl::BoxInfo>> result;
     s->detector->Detect(&input, raw_width, raw_height, &result);
+    return CopyDetections(result, out, capacity);
+  });
+}
+
+namespace {
+constexpr int kReadbackSlot = 2;  // graph slot: the pass, the detector's work, the copy of its lists
+
+// Waits for the session's last pass launched with the lists copy (its event only, not the
+// stream) and reads the lists from page-locked memory.
+void CollectLists(OgleSession* s, std::vector<std::vector<opengl::BoxInfo>>* out) {
+  CHECK(s->detector != nullptr && s->detector->host_copy_enabled() && s->lists_ready != nullptr)
+      << "no pass with a copy of its detection lists has been launched on this session";
+  if (s->lists_pending) {
+    const hipError_t e = hipEventSynchronize(s->lists_ready);
+    if (e != hipSuccess) LOG(FATAL) << "hipEventSynchronize: " << hipGetErrorString(e);
+    s->lists_pending = false;
+  }
+  s->detector->FinalFromHostCopy(out);
+}
+}  // namespace
+
+int32_t ogle_rt_time_pipelined_readback(OgleSession** sessions, int32_t n, int32_t warmup,
+                                        int32_t iters, float* total_ms, int64_t* detections) {
+  return (int32_t)Guard([&]() -> int64_t {
+    CHECK(sessions != nullptr && n >= 1 && n <= 16) << "1..16 sessions";
+    for (int i = 0; i < n; ++i) {
+      OgleSession* s = sessions[i];
+      CHECK(s != nullptr && s->session != nullptr) << "null session";
+      opengl::DetectorOptions opt;
+      opt.device_nms = true;  // the lists that are copied are the device's final ones
+      if (!s->detector) s->detector = opengl::Detector::Create(s->session.get(), opt);
+      CHECK(s->device_nms) << "the pipelined readback copies the device's final lists: "
+                              "ogle_rt_set_device_nms(session, 1)";
+      auto detect = [s, opt]() { s->detector->EnqueueDetect(opt.output_names, 300, 300); };
+      if (!s->session->graph_captured(kReadbackSlot)) {
+        s->detector->EnableHostCopy();
+        detect();  // first use allocates the result buffers and the page-locked copy: not under capture
+        s->context->Finish();
+        CHECK(s->detector->UsesDeviceNms() && s->detector->host_copy_enabled())
+            << "the detector's outputs do not fit the device top-k + NMS";
+        s->session->CaptureGraph(kReadbackSlot, detect);
+      }
+      if (s->lists_ready == nullptr &&
+          hipEventCreateWithFlags(&s->lists_ready, hipEventDisableTiming) != hipSuccess)
+        LOG(FATAL) << "hipEventCreate failed";
+    }
+    std::vector<std::vector<opengl::BoxInfo>> lists;
+    int64_t seen = 0;
+    auto step = [&](int i) {
+      OgleSession* s = sessions[i % n];
+      // the copy of the next pass lands where the last one's lists are: read those first
+      if (s->lists_pending) {
+        CollectLists(s, &lists);
+        for (const auto& image : lists) seen += (int64_t)image.size();
+      }
+      s->session->LaunchGraph(kReadbackSlot);
+      const hipError_t e = hipEventRecord(s->lists_ready, static_cast<hipStream_t>(s->context->stream()));
+      if (e != hipSuccess) LOG(FATAL) << "hipEventRecord: " << hipGetErrorString(e);
+      s->lists_pending = true;
+    };
+    auto drain = [&]() {
+      for (int i = 0; i < n; ++i)
+        if (sessions[i]->lists_pending) {
+          CollectLists(sessions[i], &lists);
+          for (const auto& image : lists) seen += (int64_t)image.size();
+        }
+      for (int i = 0; i < n; ++i) sessions[i]->context->Finish();
+    };
+    for (int i = 0; i < warmup; ++i) step(i);
+    drain();
+    seen = 0;
+    const auto t0 = std::chrono::steady_clock::now();
+    for (int i = 0; i < iters; ++i) step(i);
+    // the lists of every session's last pass stay unread for ogle_rt_pipelined_results:
+    // wait for them, count them, but leave them marked as the session's current lists
+    for (int i = 0; i < n; ++i) {
+      OgleSession* s = sessions[i];
+      if (!s->lists_pending) continue;
+      CollectLists(s, &lists);
+      for (const auto& image : lists) seen += (int64_t)image.size();
+    }
+    for (int i = 0; i < n; ++i) sessions[i]->context->Finish();
+    const auto t1 = std::chrono::steady_clock::now();
+    if (total_ms) *total_ms = std::chrono::duration<float, std::milli>(t1 - t0).count();
+    if (detections) *detections = seen;
+    return 0;
+  });
+}
+
+int64_t ogle_rt_pipelined_results(OgleSession* s, OgleDetection* out, int64_t capacity) {
+  return Guard([&]() -> int64_t {
+    std::vector<std::vector<opengl::BoxInfo>> result;
+    CollectLists(s, &result);
     return CopyDetections(result, out, capacity);
   });
 }

@@ -53,7 +53,7 @@ class FBOSession {
   // Records one Compute() pass into a hipGraph (once per slot) and replays it.
   // `after_pass`, if given, enqueues more work on the context's stream (a detector's
   // post-processing) that is recorded into the same graph; it must not allocate.
-  static constexpr int kGraphSlots = 2;
+  static constexpr int kGraphSlots = 3;
   void CaptureGraph(int slot = 0, const std::function<void()>& after_pass = {});
   void LaunchGraph(int slot = 0);
   bool graph_captured(int slot = 0) const { return graph_exec_[slot] != nullptr; }

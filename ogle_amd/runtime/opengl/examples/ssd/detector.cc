@@ -29,6 +29,7 @@ Detector::Detector(FBOSession* session, bool owned, const DetectorOptions& optio
 }
 
 Detector::~Detector() {
+  if (final_host_ != nullptr) (void)hipHostFree(final_host_);
   if (owns_session_) delete session_;
 }
 
@@ -134,9 +135,8 @@ void Detector::Readback() {
 namespace {
 // One BoxInfo from entry `s` of the (prior, class, score, box, rect) arrays
 // (detector.cc:211-225).
-BoxInfo MakeBoxInfo(size_t s, const std::vector<int32_t>& prior, const std::vector<int32_t>& cls,
-                    const std::vector<float>& score, const std::vector<float>& box,
-                    const std::vector<int32_t>& rect) {
+BoxInfo MakeBoxInfo(size_t s, const int32_t* prior, const int32_t* cls, const float* score,
+                    const float* box, const int32_t* rect) {
   BoxInfo info;
   const float xmin = box[s * 4 + 0], ymin = box[s * 4 + 1];
   const float xmax = box[s * 4 + 2], ymax = box[s * 4 + 3];
@@ -160,7 +160,8 @@ void Detector::GenerateBoxInfo(int image, std::vector<BoxInfo>* box_infos) const
   box_infos->clear();
   const size_t base = static_cast<size_t>(image) * priors_;
   for (int r = 0; r < count_[image]; ++r)
-    box_infos->push_back(MakeBoxInfo(base + r, prior_, class_, score_, box_, rect_));
+    box_infos->push_back(MakeBoxInfo(base + r, prior_.data(), class_.data(), score_.data(), box_.data(),
+                                     rect_.data()));
 }
 
 bool Detector::UsesDeviceNms() const {
@@ -187,24 +188,22 @@ void Detector::EnqueueTopkNms() {
   CHECK(batch_ > 0) << "EnqueuePostprocess first";
   const int topk = options_.topk;
   if (final_topk_ != topk) {
+    if (final_host_ != nullptr) {   // sized for other lists: made anew below
+      (void)hipHostFree(final_host_);
+      final_host_ = nullptr;
+    }
     final_topk_ = topk;
-    auto dev = [](IntList shape) {
-      return std::unique_ptr<Tensor>(
-          new Tensor(Tensor::DT_FLOAT, shape, Tensor::DEVICE_BUFFER, dlxnet::TensorProto::ANY4));
-    };
-    fcount_dev_ = dev({batch_});
-    fprior_dev_ = dev({batch_, topk});
-    fclass_dev_ = dev({batch_, topk});
-    fscore_dev_ = dev({batch_, topk});
-    fbox_dev_ = dev({batch_, topk, 4});
-    frect_dev_ = dev({batch_, topk, 4});
-    fcount_.resize(batch_);
-    fprior_.resize(static_cast<size_t>(batch_) * topk);
-    fclass_.resize(fprior_.size());
-    fscore_.resize(fprior_.size());
-    fbox_.resize(fprior_.size() * 4);
-    frect_.resize(fprior_.size() * 4);
+    final_dev_.reset(new Tensor(Tensor::DT_FLOAT, {static_cast<int>(FinalWords())}, Tensor::DEVICE_BUFFER,
+                                dlxnet::TensorProto::ANY));
+    final_staging_.assign(FinalWords(), 0);
   }
+  if (want_host_copy_ && final_host_ == nullptr) {
+    const hipError_t e = hipHostMalloc(&final_host_, FinalWords() * 4, hipHostMallocDefault);
+    if (e != hipSuccess) LOG(FATAL) << "hipHostMalloc(" << FinalWords() * 4 << "): " << hipGetErrorString(e);
+  }
+  // where the six lists lie inside the block
+  int32_t* const blk = static_cast<int32_t*>(final_dev_->device_ptr());
+  const size_t bt = static_cast<size_t>(batch_) * topk;
   OgleNmsArgs a{};
   a.kept_count_dev =
       lists_in_place_ ? nullptr : static_cast<const int32_t*>(count_dev_->device_ptr());
@@ -217,39 +216,60 @@ void Detector::EnqueueTopkNms() {
   a.stride = priors_;
   a.topk = topk;
   a.nms_threshold = options_.nms_threshold;
-  a.final_count_dev = static_cast<int32_t*>(fcount_dev_->device_ptr());
-  a.final_prior_dev = static_cast<int32_t*>(fprior_dev_->device_ptr());
-  a.final_class_dev = static_cast<int32_t*>(fclass_dev_->device_ptr());
-  a.final_score_dev = static_cast<float*>(fscore_dev_->device_ptr());
-  a.final_box_dev = static_cast<float*>(fbox_dev_->device_ptr());
-  a.final_rect_dev = static_cast<int32_t*>(frect_dev_->device_ptr());
+  a.final_count_dev = blk;
+  a.final_prior_dev = blk + batch_;
+  a.final_class_dev = blk + batch_ + bt;
+  a.final_score_dev = reinterpret_cast<float*>(blk + batch_ + 2 * bt);
+  a.final_box_dev = reinterpret_cast<float*>(blk + batch_ + 3 * bt);
+  a.final_rect_dev = blk + batch_ + 7 * bt;
   hipStream_t s = static_cast<hipStream_t>(session_->context()->stream());
   const int64_t before = ogle_hip_launch_count();
   const int32_t st = ogle_hip_ssd_topk_nms(&a, s);
   if (st != OGLE_OK) LOG(FATAL) << "ogle_hip_ssd_topk_nms: " << ogle_hip_last_error();
   session_->context()->LogLaunches("detector.topk_nms#Detector#", before);
+  if (final_host_ != nullptr) {
+    const hipError_t e =
+        hipMemcpyAsync(final_host_, final_dev_->device_ptr(), FinalWords() * 4, hipMemcpyDeviceToHost, s);
+    if (e != hipSuccess) LOG(FATAL) << "copy of the final lists: " << hipGetErrorString(e);
+  }
+}
+
+size_t Detector::FinalWords() const {
+  return static_cast<size_t>(batch_) * (1 + static_cast<size_t>(final_topk_) * 11);
+}
+
+void Detector::EnableHostCopy() { want_host_copy_ = true; }
+
+void Detector::ParseFinal(const int32_t* blk, std::vector<std::vector<BoxInfo>>* final_boxes) const {
+  const size_t bt = static_cast<size_t>(batch_) * final_topk_;
+  const int32_t* prior = blk + batch_;
+  const int32_t* cls = prior + bt;
+  const float* score = reinterpret_cast<const float*>(cls + bt);
+  const float* box = score + bt;
+  const int32_t* rect = reinterpret_cast<const int32_t*>(box + 4 * bt);
+  final_boxes->assign(batch_, {});
+  for (int b = 0; b < batch_; ++b) {
+    const size_t base = static_cast<size_t>(b) * final_topk_;
+    const int n = std::min(std::max(blk[b], 0), final_topk_);
+    (*final_boxes)[b].reserve(n);
+    for (int r = 0; r < n; ++r)
+      (*final_boxes)[b].push_back(MakeBoxInfo(base + r, prior, cls, score, box, rect));
+  }
+}
+
+void Detector::FinalFromHostCopy(std::vector<std::vector<BoxInfo>>* final_boxes) const {
+  CHECK(final_host_ != nullptr && final_topk_ > 0) << "EnableHostCopy, then a pass with the detector's work";
+  ParseFinal(static_cast<const int32_t*>(final_host_), final_boxes);
 }
 
 void Detector::ReadbackFinal(std::vector<std::vector<BoxInfo>>* final_boxes) {
   CHECK(final_topk_ > 0) << "EnqueueTopkNms first";
   hipStream_t s = static_cast<hipStream_t>(session_->context()->stream());
-  auto back = [&](void* dst, const Tensor* src, size_t bytes) {
-    const hipError_t e = hipMemcpyAsync(dst, src->device_ptr(), bytes, hipMemcpyDeviceToHost, s);
-    if (e != hipSuccess) LOG(FATAL) << "readback: " << hipGetErrorString(e);
-  };
-  back(fcount_.data(), fcount_dev_.get(), fcount_.size() * 4);
-  back(fprior_.data(), fprior_dev_.get(), fprior_.size() * 4);
-  back(fclass_.data(), fclass_dev_.get(), fclass_.size() * 4);
-  back(fscore_.data(), fscore_dev_.get(), fscore_.size() * 4);
-  back(fbox_.data(), fbox_dev_.get(), fbox_.size() * 4);
-  back(frect_.data(), frect_dev_.get(), frect_.size() * 4);
+  const hipError_t e = hipMemcpyAsync(final_staging_.data(), final_dev_->device_ptr(), FinalWords() * 4,
+                                      hipMemcpyDeviceToHost, s);
+  if (e != hipSuccess) LOG(FATAL) << "readback: " << hipGetErrorString(e);
   session_->context()->Finish();
-  final_boxes->assign(batch_, {});
-  for (int b = 0; b < batch_; ++b) {
-    const size_t base = static_cast<size_t>(b) * final_topk_;
-    for (int r = 0; r < fcount_[b]; ++r)
-      (*final_boxes)[b].push_back(MakeBoxInfo(base + r, fprior_, fclass_, fscore_, fbox_, frect_));
-  }
+  ParseFinal(final_staging_.data(), final_boxes);
 }
 
 // detector.cc:114-125.  std::stable_sort makes the order of equal scores defined

@@ -75,6 +75,16 @@ class Detector {
   // (asynchronous), and the readback of its final lists (synchronises).
   void EnqueueTopkNms();
   void ReadbackFinal(std::vector<std::vector<BoxInfo>>* final_boxes);
+  // Pipelined readback: once enabled, EnqueueTopkNms is followed on the stream by ONE
+  // asynchronous copy of the final lists (they are one device block: the counts, then at most
+  // topk records per image) into page-locked host memory owned by the detector.  Recorded
+  // into a captured pass it replays with it, so the host only waits for an event after the
+  // pass (not for the stream) and then reads the lists with FinalFromHostCopy, while later
+  // passes are already enqueued.  The copy lands in the same memory every pass: read it
+  // before the detector's next pass is launched.
+  void EnableHostCopy();
+  bool host_copy_enabled() const { return final_host_ != nullptr; }
+  void FinalFromHostCopy(std::vector<std::vector<BoxInfo>>* final_boxes) const;
   bool UsesDeviceNms() const;
   // Everything Detect does on the device after the network (asynchronous): the score
   // filter, and with device top-k + NMS that launch too (ReadbackFinal fetches its
@@ -104,9 +114,14 @@ class Detector {
   std::vector<float> score_, box_;
   // final lists of the device top-k + NMS: (batch, topk) each
   int final_topk_ = 0;
-  std::unique_ptr<Tensor> fcount_dev_, fprior_dev_, fclass_dev_, fscore_dev_, fbox_dev_, frect_dev_;
-  std::vector<int32_t> fcount_, fprior_, fclass_, frect_;
-  std::vector<float> fscore_, fbox_;
+  // one device block: counts (batch), then prior, class, score (batch x topk each), box and
+  // rect (batch x topk x 4 each); 4-byte elements throughout
+  std::unique_ptr<Tensor> final_dev_;
+  std::vector<int32_t> final_staging_;   // host copy made by ReadbackFinal
+  void* final_host_ = nullptr;           // page-locked copy made on the stream (EnableHostCopy)
+  bool want_host_copy_ = false;
+  size_t FinalWords() const;
+  void ParseFinal(const int32_t* block, std::vector<std::vector<BoxInfo>>* final_boxes) const;
 };
 
 float iou(const Rect& box0, const Rect& box1);

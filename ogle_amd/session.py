@@ -26,7 +26,8 @@ SYMBOLS = [
     "ogle_rt_set_reorder", "ogle_rt_issue_order_name", "ogle_rt_set_device_nms",
     "ogle_rt_detect_results", "ogle_rt_graph_captured", "ogle_rt_hazard_conflicts",
     "ogle_rt_set_fuse_siblings", "ogle_rt_launch_plan", "ogle_rt_launch_plan_entry",
-    "ogle_rt_conv_hazard_conflicts", "ogle_rt_host_elements",
+    "ogle_rt_conv_hazard_conflicts", "ogle_rt_host_elements", "ogle_rt_time_pipelined_readback",
+    "ogle_rt_pipelined_results",
 ]
 
 
@@ -107,6 +108,10 @@ def lib():
         l.ogle_rt_detect.restype = i64
         l.ogle_rt_detect_results.argtypes = [vp, ctypes.POINTER(Detection), i64]
         l.ogle_rt_detect_results.restype = i64
+        l.ogle_rt_time_pipelined_readback.argtypes = [ctypes.POINTER(vp), i32, i32, i32,
+                                                      ctypes.POINTER(ctypes.c_float), ctypes.POINTER(i64)]
+        l.ogle_rt_pipelined_results.argtypes = [vp, ctypes.POINTER(Detection), i64]
+        l.ogle_rt_pipelined_results.restype = i64
         l.ogle_rt_reserialize.argtypes = [vp, ctypes.c_size_t, vp, i64]
         l.ogle_rt_reserialize.restype = i64
         l.ogle_rt_model_debug_string.argtypes = [vp, ctypes.c_size_t, vp, i64]
@@ -401,6 +406,26 @@ class Session:
             per_image[d.image].append(dict(prior=d.prior, cls=d.class_id, score=d.score,
                                            rect=(d.x, d.y, d.width, d.height), cx=d.cx, cy=d.cy))
         return per_image
+
+    @staticmethod
+    def time_pipelined_readback(sessions, warmup, iters):
+        """`iters` passes dealt round-robin over `sessions`, each pass a hipGraph replay on its
+        session's stream that ends with one asynchronous copy of its final detection lists to
+        page-locked host memory; before a session's next pass is launched the host waits for the
+        event behind its previous pass and reads the lists.  Returns (total ms, detections read
+        in the timed passes)."""
+        handles = (ctypes.c_void_p * len(sessions))(*[s._h for s in sessions])
+        total, seen = ctypes.c_float(0), ctypes.c_int64(0)
+        _check(lib().ogle_rt_time_pipelined_readback(handles, len(sessions), warmup, iters,
+                                                     ctypes.byref(total), ctypes.byref(seen)))
+        return float(total.value), int(seen.value)
+
+    def pipelined_results(self, batch, capacity=4096):
+        """Detections of the session's last pass of time_pipelined_readback, from the page-locked
+        copy of its lists."""
+        buf = (Detection * capacity)()
+        n = _check(lib().ogle_rt_pipelined_results(self._h, buf, capacity))
+        return self._per_image(buf, n, capacity, batch)
 
     def detect_results(self, batch, capacity=4096):
         """Detections of the detector work last enqueued by time_compute(with_detect=True)."""

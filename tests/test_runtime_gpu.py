@@ -560,6 +560,47 @@ def test_pipelined_sessions_keep_their_own_results():
         pb.close()
 
 
+def test_pipelined_readback_lists_equal_detect_results():
+    """Passes whose final detection lists are copied to page-locked host memory inside the
+    captured graph, the host waiting only for the event behind a session's previous pass: the
+    lists read that way equal what the synchronous readback of the same session gives and what
+    Detector::Detect computes eagerly, for one session alone (every pass waits for the one
+    before) and for three sessions with different inputs in flight together, replay after replay
+    and after an input change."""
+    batch = 3
+    g, _ = models.mobilenet_v1_ssd(batch, seed=41, head_std=0.05)
+    inputs = [rng(90 + i).uniform(-1, 1, (batch, 300, 300, 3)).astype(np.float32) for i in range(3)]
+    sessions, eager = [], []
+    for x in inputs:
+        s = session.Session()
+        s.load_graph(g)
+        eager.append(s.detect(x, 300, 300, 0.3, 0.45, 100))
+        sessions.append(s)
+    assert all(sum(len(e) for e in d) > 0 for d in eager)
+    per_pass = [sum(len(e) for e in d) for d in eager]
+    # one session: 5 timed passes, every one's lists read by the host
+    ms, seen = session.Session.time_pipelined_readback(sessions[:1], 2, 5)
+    assert ms > 0 and seen == 5 * per_pass[0]
+    assert sessions[0].pipelined_results(batch) == eager[0]
+    assert sessions[0].detect_results(batch) == eager[0]
+    # three sessions in flight: 7 passes dealt round-robin (3 + 2 + 2)
+    ms, seen = session.Session.time_pipelined_readback(sessions, 3, 7)
+    assert seen == 3 * per_pass[0] + 2 * per_pass[1] + 2 * per_pass[2]
+    for s, e in zip(sessions, eager):
+        assert s.pipelined_results(batch) == e
+        assert s.detect_results(batch) == e
+    # new inputs: the replayed copy follows them
+    sessions[0].run({"input": inputs[1]})
+    sessions[1].run({"input": inputs[2]})
+    session.Session.time_pipelined_readback(sessions[:2], 1, 4)
+    assert sessions[0].pipelined_results(batch) == eager[1]
+    assert sessions[1].pipelined_results(batch) == eager[2]
+    # the host loop of the reference is not what is copied: refused with the host top-k + NMS
+    sessions[2].set_device_nms(False)
+    with pytest.raises(RuntimeError, match="ogle_rt_set_device_nms"):
+        session.Session.time_pipelined_readback(sessions[2:], 1, 1)
+
+
 def test_batch16_images_match_their_batch1_passes():
     """The headline configuration (batch 16) takes other tile shapes, K splits and issue order than
     batch 1.  Every image is independent through every kernel, so image i of a batch-16 pass must
