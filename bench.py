@@ -235,6 +235,13 @@ def kernel_table(iters=50, warm=5, only=None):
              16, 150, 150, 64, 64, 3, 2, 1, g=64, act=H.ACT_CLIP, maxv=6.0)
     conv_row("depthwise 3x3 @C5 b16 block3 (75x75x128)", "ogle_hip_dwconv2d", "hbm",
              16, 75, 75, 128, 128, 3, 1, 1, g=128, act=H.ACT_CLIP, maxv=6.0)
+    # pointwise layers of the headline pass (C5 at batch 16)
+    conv_row("pointwise @C5 b16 block2 (M=90000 K=64 N=128)", "ogle_hip_pwconv_gemm", "mfma",
+             16, 75, 75, 64, 128, 1, 1, 0, act=H.ACT_CLIP, maxv=6.0)
+    conv_row("pointwise @C5 b16 block8 (M=5776 K=512 N=512)", "ogle_hip_pwconv_gemm", "mfma",
+             16, 19, 19, 512, 512, 1, 1, 0, act=H.ACT_CLIP, maxv=6.0)
+    conv_row("pointwise @C5 b16 block13 (M=1600 K=1024 N=1024)", "ogle_hip_pwconv_gemm", "mfma",
+             16, 10, 10, 1024, 1024, 1, 1, 0, act=H.ACT_CLIP, maxv=6.0)
     conv_row("pointwise GEMM @C3 fp32 (M=11552 K=512 N=1024)", "ogle_hip_pwconv_gemm", "mfma",
              32, 19, 19, 512, 1024, 1, 1, 0)
     conv_row("pointwise GEMM @C3 fp16 storage, fp32 accumulate", "ogle_hip_pwconv_gemm", "mfma",

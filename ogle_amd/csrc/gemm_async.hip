@@ -34,6 +34,13 @@
 //
 // Eight waves per workgroup, two per SIMD, in two groups that alternate between reading
 // operands and issuing MFMAs (see the loop), 256 x 256 or 192 x 256 outputs per workgroup.
+//
+// The kernel is written for either storage type, but only fp16 storage is routed here: with
+// fp32 operands (v_mfma_f32_32x32x2_f32 does a sixteenth of the work per operand byte and per
+// cycle) 128 x 128 ... 256 x 256 tiles of this form measured 70-111 TFLOP/s on the network's
+// pointwise layers, alone and with two or four launches in flight, against 88-115 TFLOP/s for
+// the LDS-tiled kernel with its small 64 x 64 tiles, which spread far better over 256 compute
+// units at those sizes.
 #include "common.h"
 
 #pragma clang diagnostic ignored "-Winline-asm"
@@ -97,9 +104,10 @@ constexpr int async_lds_bytes() {
   return NST * (BM + BN) * kStageRowBytes + BN * 4 + spare * 1024;
 }
 
-template <int BM, int BN, int WM, int WN, int NST>
-__global__ __launch_bounds__(64 * WM * WN, 1) void pw_gemm_f16_async_kernel(AsyncProblem p) {
+template <typename T, int BM, int BN, int WM, int WN, int NST>
+__global__ __launch_bounds__(64 * WM * WN, 1) void pw_gemm_async_kernel(AsyncProblem p) {
   constexpr int NW = WM * WN;
+  constexpr unsigned ESZ = sizeof(T);
   constexpr int KS = kStageRowBytes;
   constexpr int WTM = BM / WM, WTN = BN / WN;
   constexpr int TM = WTM / 32, TN = WTN / 32;       // 32x32 MFMA blocks per wave: pixels, channels
@@ -135,7 +143,7 @@ __global__ __launch_bounds__(64 * WM * WN, 1) void pw_gemm_f16_async_kernel(Asyn
 
   const u32x4 dx = make_desc(p.x, p.x_bytes);
   const u32x4 dw = make_desc(p.w, p.w_bytes);
-  const unsigned krow = (unsigned)p.k * 2u;         // bytes per operand row
+  const unsigned krow = (unsigned)p.k * ESZ;        // bytes per operand row
 
   // The pieces this wave fetches each stage: piece c = wave + NW * i covers tile rows
   // [16 c, 16 c + 16); this lane's row of it and the K group it fetches.
@@ -157,7 +165,7 @@ __global__ __launch_bounds__(64 * WM * WN, 1) void pw_gemm_f16_async_kernel(Asyn
       g_off[i] = kOutOfRange;   // a spare slot
     }
   }
-  const int stages = (p.k * 2 + KS - 1) / KS;
+  const int stages = (int)((krow + KS - 1) / KS);
 
   auto request_stage = [&](int s) {
     const unsigned kb = (unsigned)s * KS;
@@ -204,27 +212,44 @@ __global__ __launch_bounds__(64 * WM * WN, 1) void pw_gemm_f16_async_kernel(Asyn
     *reinterpret_cast<float4*>(bias_lds + tid * 4) = bv;
   }
 
-  halfx8 xv[2][TM], wv[2][TN];
+  u32x4 xv[2][TM], wv[2][TN];
   auto read_stage = [&](int s) {
     const unsigned char* buf = lds + (s % NST) * STAGE;
 #pragma unroll
     for (int ch = 0; ch < 2; ++ch) {
 #pragma unroll
       for (int b = 0; b < TM; ++b)
-        xv[ch][b] = *reinterpret_cast<const halfx8*>(buf + rd_x + b * 32 * KS + rd_k[ch]);
+        xv[ch][b] = *reinterpret_cast<const u32x4*>(buf + rd_x + b * 32 * KS + rd_k[ch]);
 #pragma unroll
       for (int a = 0; a < TN; ++a)
-        wv[ch][a] = *reinterpret_cast<const halfx8*>(buf + rd_w + a * 32 * KS + rd_k[ch]);
+        wv[ch][a] = *reinterpret_cast<const u32x4*>(buf + rd_w + a * 32 * KS + rd_k[ch]);
     }
   };
+  // fp16: a lane's 16 bytes are the 8 halves one v_mfma_f32_32x32x16_f16 wants (k = 8 * (l / 32) ..+7).
+  // fp32: they are 4 floats, one v_mfma_f32_32x32x2_f32 each (the contraction sums over k in any
+  // order: lanes 0-31 supply k 0..3 of an 8-wide group, lanes 32-63 k 4..7).
   auto multiply_stage = [&]() {
 #pragma unroll
-    for (int ch = 0; ch < 2; ++ch)
+    for (int ch = 0; ch < 2; ++ch) {
+      if constexpr (sizeof(T) == 2) {
 #pragma unroll
-      for (int a = 0; a < TN; ++a)
+        for (int a = 0; a < TN; ++a)
 #pragma unroll
-        for (int b = 0; b < TM; ++b)
-          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wv[ch][a], xv[ch][b], acc[a][b], 0, 0, 0);
+          for (int b = 0; b < TM; ++b)
+            acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(halfx8, wv[ch][a]),
+                                                               __builtin_bit_cast(halfx8, xv[ch][b]),
+                                                               acc[a][b], 0, 0, 0);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+#pragma unroll
+          for (int a = 0; a < TN; ++a)
+#pragma unroll
+            for (int b = 0; b < TM; ++b)
+              acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(wv[ch][a][e]),
+                                                               __uint_as_float(xv[ch][b][e]), acc[a][b], 0, 0, 0);
+      }
+    }
   };
   // A barrier the instruction scheduler does not move anything across: the two halves of
   // the loop body must stay on their own sides of it.
@@ -269,14 +294,16 @@ __global__ __launch_bounds__(64 * WM * WN, 1) void pw_gemm_f16_async_kernel(Asyn
   // conversion on the way in (8 bytes per quad), 16 bytes per lane on the way out with
   // consecutive lanes on consecutive channels of one pixel, i.e. whole 128-byte runs per row.
   __syncthreads();   // every wave has finished reading the stage buffers that are reused here
-  constexpr int ROWP = WTN * 2 + 16;            // staged row: the wave's channels as halves, padded
-  constexpr int SEGS = WTN * 2 / 16;            // 16-byte segments (lanes) per row
+  constexpr int ROWP = WTN * (int)ESZ + 16;     // staged row: the wave's channels in storage type, padded
+  constexpr int SEGS = WTN * (int)ESZ / 16;     // 16-byte segments (lanes) per row
   constexpr int RPI = 64 / SEGS;                // rows one store instruction covers
+  constexpr int EPS = 16 / (int)ESZ;            // elements per 16-byte segment
   static_assert(NW * 32 * ROWP <= NST * STAGE, "epilogue staging exceeds the stage buffers");
+  static_assert(SEGS <= 64 && 64 % SEGS == 0 && 32 % RPI == 0, "staged rows divide among the lanes");
   unsigned char* const stg = lds + wave * (32 * ROWP);
-  __half* const y = static_cast<__half*>(p.y);
+  T* const y = static_cast<T*>(p.y);
   const int seg = lane % SEGS, rsub = lane / SEGS;
-  const int ocol = n0 + wave_n * WTN + seg * 8;
+  const int ocol = n0 + wave_n * WTN + seg * EPS;
 #pragma unroll
   for (int b = 0; b < TM; ++b) {
 #pragma unroll
@@ -285,12 +312,17 @@ __global__ __launch_bounds__(64 * WM * WN, 1) void pw_gemm_f16_async_kernel(Asyn
       for (int q = 0; q < 4; ++q) {
         const int oc = a * 32 + q * 8 + lh * 4;   // channel inside the wave's tile
         const float4 bv = *reinterpret_cast<const float4*>(bias_lds + wave_n * WTN + oc);
-        halfx4 out;
-        out[0] = (_Float16)apply_epilogue(acc[a][b][q * 4 + 0] + bv.x, p.ep);
-        out[1] = (_Float16)apply_epilogue(acc[a][b][q * 4 + 1] + bv.y, p.ep);
-        out[2] = (_Float16)apply_epilogue(acc[a][b][q * 4 + 2] + bv.z, p.ep);
-        out[3] = (_Float16)apply_epilogue(acc[a][b][q * 4 + 3] + bv.w, p.ep);
-        *reinterpret_cast<halfx4*>(stg + l32 * ROWP + oc * 2) = out;
+        const float o0 = apply_epilogue(acc[a][b][q * 4 + 0] + bv.x, p.ep);
+        const float o1 = apply_epilogue(acc[a][b][q * 4 + 1] + bv.y, p.ep);
+        const float o2 = apply_epilogue(acc[a][b][q * 4 + 2] + bv.z, p.ep);
+        const float o3 = apply_epilogue(acc[a][b][q * 4 + 3] + bv.w, p.ep);
+        if constexpr (sizeof(T) == 2) {
+          halfx4 out;
+          out[0] = (_Float16)o0; out[1] = (_Float16)o1; out[2] = (_Float16)o2; out[3] = (_Float16)o3;
+          *reinterpret_cast<halfx4*>(stg + l32 * ROWP + oc * 2) = out;
+        } else {
+          *reinterpret_cast<float4*>(stg + l32 * ROWP + oc * 4) = make_float4(o0, o1, o2, o3);
+        }
       }
     }
 #pragma unroll
@@ -314,23 +346,25 @@ __global__ __launch_bounds__(64 * WM * WN, 1) void pw_gemm_f16_async_kernel(Asyn
 
 enum { kTile256 = 0, kTile192 = 1 };   // 256 x 256 or 192 x 256 outputs per workgroup
 
-template <int BM, int BN, int WM, int WN, int NST>
-int32_t launch_tile(const AsyncProblem& p, hipStream_t s) {
+template <typename T, int BM, int BN, int WM, int WN, int NST>
+int32_t launch_tile(AsyncProblem p, hipStream_t s) {
   constexpr int kLds = async_lds_bytes<BM, BN, WM, WN, NST>();
-  auto kernel = pw_gemm_f16_async_kernel<BM, BN, WM, WN, NST>;
+  auto kernel = pw_gemm_async_kernel<T, BM, BN, WM, WN, NST>;
   static bool configured = false;  // per process; the attribute is a property of the function
   if (!configured) {
     const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                              hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
     if (e != hipSuccess) {
-      set_error("pw_gemm_f16_async: cannot reserve %d bytes of LDS: %s", kLds, hipGetErrorString(e));
+      set_error("pw_gemm_async: cannot reserve %d bytes of LDS: %s", kLds, hipGetErrorString(e));
       return OGLE_ERR_LAUNCH;
     }
     configured = true;
   }
+  p.tiles_m = (p.m + BM - 1) / BM;
+  p.tiles_n = (p.n + BN - 1) / BN;
   const unsigned grid = 8u * (unsigned)((p.tiles_m + 7) / 8) * (unsigned)p.tiles_n;
   launch(kernel, dim3(grid), dim3(64 * WM * WN), (unsigned)kLds, s, p);
-  return check_launch("pw_gemm_f16_async");
+  return check_launch("pw_gemm_async");
 }
 
 }  // namespace
@@ -371,16 +405,17 @@ int32_t launch_pw_gemm_f16_async(const OgleConvArgs& a, hipStream_t s) {
   p.m = (int)((long)a.n * a.out_h * a.out_w);
   p.n = a.out_c;
   p.k = a.in_c;
-  p.x_bytes = (unsigned)((long)p.m * p.k * 2);
-  p.w_bytes = (unsigned)((long)p.n * p.k * 2);
-  const int bm = cfg == kTile192 ? 192 : 256;
-  p.tiles_m = (p.m + bm - 1) / bm;
-  p.tiles_n = (p.n + 255) / 256;
+  const long esz = a.dtype == OGLE_F16 ? 2 : 4;
+  p.x_bytes = (unsigned)((long)p.m * p.k * esz);
+  p.w_bytes = (unsigned)((long)p.n * p.k * esz);
   p.hw = a.out_h * a.out_w;
   p.oimg = a.out_image_stride == (long)p.hw * a.out_c ? 0 : a.out_image_stride;
   p.ep = make_epilogue(a.act, a.min_value, a.max_value, a.act_variant);
-  if (cfg == kTile192) return launch_tile<192, 256, 2, 4, 4>(p, s);
-  return launch_tile<256, 256, 2, 4, 4>(p, s);
+  switch (cfg) {
+    case kTile192: return launch_tile<__half, 192, 256, 2, 4, 4>(p, s);
+    case kTile256: return launch_tile<__half, 256, 256, 2, 4, 4>(p, s);
+    default: return OGLE_ERR_UNSUPPORTED;
+  }
 }
 
 }  // namespace ogle
