@@ -10,6 +10,11 @@ The graph is a .dlx model loaded into the C++ FBOSession; the pass is replayed a
 Printed JSON (one line): images/s at batch 16 (`value`), p50 latency at batch 1, the roofline
 of the dominant kernel family measured with HIP events on the session's stream inside this
 process, a per-family table, and the CPU restatement timed on the host cores.
+
+Timing protocol: --warmup untimed steps, then untimed replays until --clock-ramp seconds have
+gone by (the clocks of an idle GPU take longer to settle than 20 steps last), then --repeats
+timed regions of exactly --steps steps each, every region bracketed by a wait for all streams;
+`ms_per_step` / `value` are the median region, the extremes are reported beside them.
 """
 import argparse
 import json
@@ -43,15 +48,19 @@ def build_session(batch, seed=20240005, input_seed=None):
 TAIL_FAMILY = "concat + detector tail (decode / score filter, top-k + NMS)"
 
 
-def detector_tail_bytes(batch, priors=1917, classes=21, topk=100):
-    """Algorithmic bytes of the detector tail per pass.  Decode + softmax-max + score filter: per
-    image the class logits and box predictions in, the decoded boxes and one (score, class) pair
-    per prior out, and the anchors once for the batch.  Top-k + NMS: per image one 28-byte record
-    per prior in (score, class, prior, rectangle) and at most `topk` 44-byte records out.  The
-    concatenations move nothing: the heads write straight into their outputs."""
+def detector_tail_parts(batch, priors=1917, classes=21, topk=100):
+    """Algorithmic bytes of the detector tail per pass, by launch.  Decode + softmax-max + score
+    filter: per image the class logits and box predictions in, the decoded boxes and one
+    (score, class) pair per prior out, and the anchors once for the batch.  Top-k + NMS: per image
+    one 28-byte record per prior in (score, class, prior, rectangle) and at most `topk` 44-byte
+    records out.  The concatenations move nothing: the heads write straight into their outputs."""
     per_image = priors * classes * 4 + priors * 16 + priors * 16 + priors * 8   # 161,028 + 30,672 + 30,672 + 15,336
-    nms = priors * 28 + topk * 44
-    return batch * (per_image + nms) + priors * 16
+    return {"detector.score_filter": batch * per_image + priors * 16,
+            "detector.topk_nms": batch * (priors * 28 + topk * 44)}
+
+
+def detector_tail_bytes(batch):
+    return sum(detector_tail_parts(batch).values())
 
 
 def family_of(nodes, layers):
@@ -428,6 +437,7 @@ def profile_layers_run(args):
                         "network + decode/score filter + top-k/NMS"
                         % (args.batch, "kernel-by-kernel launches" if args.eager else "hipGraph replay"),
                batch=args.batch, replays=args.steps, dispatches_per_pass=sum(k for _, k in plan),
+               tail_bytes=detector_tail_parts(args.batch),
                plan=plan, calibration=dict(kernel="convert_kernel<float, float>", kib_per_launch=copy_bytes // 1024),
                layers={l["name"]: dict(kind=l["kind"], flops_per_image=l["flops_per_image"],
                                        act_bytes_per_image=l["act_bytes_per_image"],

@@ -350,15 +350,21 @@ template <typename T, int BM, int BN, int WM, int WN, int NST>
 int32_t launch_tile(AsyncProblem p, hipStream_t s) {
   constexpr int kLds = async_lds_bytes<BM, BN, WM, WN, NST>();
   auto kernel = pw_gemm_async_kernel<T, BM, BN, WM, WN, NST>;
-  static bool configured = false;  // per process; the attribute is a property of the function
-  if (!configured) {
+  // more than 64 KB of dynamic LDS has to be asked for once per device and kernel
+  static bool configured[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
+    set_error("pw_gemm_async: no current device");
+    return OGLE_ERR_NO_DEVICE;
+  }
+  if (!configured[dev]) {
     const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                              hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
     if (e != hipSuccess) {
       set_error("pw_gemm_async: cannot reserve %d bytes of LDS: %s", kLds, hipGetErrorString(e));
       return OGLE_ERR_LAUNCH;
     }
-    configured = true;
+    configured[dev] = true;
   }
   p.tiles_m = (p.m + BM - 1) / BM;
   p.tiles_n = (p.n + BN - 1) / BN;

@@ -90,6 +90,7 @@ def summarize(trace_path, plan):
                                         for x in nodes if x in layers)
         nbytes = 0 if is_reduce else sum((layers[x]["act_bytes_per_image"] * batch + layers[x]["weight_bytes"])
                                          * share.get(x, 1.0) for x in nodes if x in layers)
+        nbytes += sum(plan.get("tail_bytes", {}).get(x, 0) for x in nodes)   # the detector's launches
         f = family_of(nodes, layers)
         bound = "hbm" if f in ("depthwise", "stem", "tail") else "mfma"
         if is_reduce:
@@ -154,7 +155,7 @@ def render_traffic(fetch_path, write_path, plan):
     w("    WRITE_SIZE read %.1f KiB for the copy -> scale %.4f" % (wraw, wscale))
     w("Values below are scaled and averaged over %d passes; algorithmic = input + weights + bias + output"
       % plan["replays"])
-    w("once each (0 for reductions, concat and the detector tail, whose bytes are all overhead here).")
+    w("once each (0 for reductions and concat, whose bytes are all overhead here; the detector's two launches: their lists).")
     w("")
     w("%-44s %-46s %10s %10s %10s %7s" % ("node(s)", "kernel", "fetch MB", "write MB", "algo MB", "ratio"))
     fam, at = {}, 0
@@ -163,6 +164,7 @@ def render_traffic(fetch_path, write_path, plan):
         nodes = [m[0] for m in re.findall(r"([^#+\[\]:]+)#([A-Za-z0-9_]+)#", label)]
         algo = 0 if is_reduce else sum(layers[x]["act_bytes_per_image"] * batch + layers[x]["weight_bytes"]
                                        for x in nodes if x in layers)
+        algo += sum(plan.get("tail_bytes", {}).get(x, 0) for x in nodes)
         f = family_of(nodes, layers)
         name = ("reduce:" if is_reduce else "") + "+".join(nodes)
         if len(name) > 43:
