@@ -508,9 +508,9 @@ def main():
         return
     use_graph = not args.eager
     streams = 1 if args.eager else max(1, min(args.streams, 16))
-    # Every session of the pipelined leg is created here, one after the other, before any
-    # other stream exists in the process: the runtime maps streams to its four hardware
-    # queues as they are created, and two sessions that land on one queue do not overlap.
+    # The sessions of the pipelined leg.  The first four sessions of a process take their
+    # streams from a pool the runtime created in one go, so they sit on different hardware
+    # queues (two sessions that share a queue do not overlap) wherever they are created.
     sess, info = build_session(args.batch)
     pool = [sess] + [build_session(args.batch, input_seed=100 + i)[0] for i in range(1, streams)]
     from ogle_amd import session as _session

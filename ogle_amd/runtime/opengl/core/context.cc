@@ -6,6 +6,9 @@
 
 #include <cstdlib>
 #include <cstring>
+#include <deque>
+#include <map>
+#include <mutex>
 #include <vector>
 
 namespace opengl {
@@ -18,11 +21,52 @@ namespace opengl {
 
 Context::Context() {}
 
+namespace {
+// The HIP runtime spreads streams over its few hardware queues as they are created, and work on
+// two streams that share a queue does not overlap.  Streams made one at a time, with the
+// application creating streams of its own in between, can therefore end up on one queue (four
+// sessions created three unrelated streams apart replay their passes at 24 k images/s instead of
+// 29.5 k).  So the first kPooledStreams streams that contexts ask for on a device are created
+// together, in one go, and handed out in that order; a context hands its stream back when it is
+// destroyed.  Contexts beyond the pool get a stream of their own.
+constexpr int kPooledStreams = 4;
+struct StreamPool {
+  std::mutex mu;
+  std::map<int, std::deque<hipStream_t>> idle;   // per device, in creation order
+  std::map<int, bool> created;
+};
+StreamPool& Pool() {
+  static StreamPool* pool = new StreamPool;   // never destroyed: streams outlive static teardown
+  return *pool;
+}
+}  // namespace
+
 void* Context::stream() {
   if (stream_ == nullptr) {
-    hipStream_t s = nullptr;
-    OGLE_HIP_CALL(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
-    stream_ = s;
+    int device = 0;
+    OGLE_HIP_CALL(hipGetDevice(&device));
+    StreamPool& pool = Pool();
+    std::lock_guard<std::mutex> lock(pool.mu);
+    if (!pool.created[device]) {
+      for (int i = 0; i < kPooledStreams; ++i) {
+        hipStream_t s = nullptr;
+        OGLE_HIP_CALL(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+        pool.idle[device].push_back(s);
+      }
+      pool.created[device] = true;
+    }
+    std::deque<hipStream_t>& idle = pool.idle[device];
+    if (!idle.empty()) {
+      stream_ = idle.front();
+      idle.pop_front();
+      stream_pooled_ = true;
+    } else {
+      hipStream_t s = nullptr;
+      OGLE_HIP_CALL(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+      stream_ = s;
+      stream_pooled_ = false;
+    }
+    stream_device_ = device;
   }
   return stream_;
 }
@@ -297,7 +341,17 @@ void Context::Flush() {
 
 Context::~Context() {
   if (workspace_ != nullptr) (void)hipFree(workspace_);
-  if (stream_ != nullptr) (void)hipStreamDestroy(static_cast<hipStream_t>(stream_));
+  if (stream_ != nullptr) {
+    hipStream_t s = static_cast<hipStream_t>(stream_);
+    if (stream_pooled_) {
+      (void)hipStreamSynchronize(s);   // the next owner starts on an idle stream
+      StreamPool& pool = Pool();
+      std::lock_guard<std::mutex> lock(pool.mu);
+      pool.idle[stream_device_].push_front(s);
+    } else {
+      (void)hipStreamDestroy(s);
+    }
+  }
 }
 
 Program* Context::CreateProgram(const std::string& kernel_fname, const std::string& build_options) {

@@ -30,7 +30,9 @@ class Context {
   ~Context();
 
   // The HIP stream every kernel of this context is launched on (a hipStream_t),
-  // created on first use so that graph loading and validation need no device.
+  // taken on first use so that graph loading and validation need no device.  The first four
+  // contexts alive on a device share a pool of streams that were created together, which
+  // keeps them on different hardware queues whatever other streams the process creates.
   void* stream();
 
   // Looks `kernel_fname` (a shader stem such as "conv2d_pw") up in the HIP kernel
@@ -113,6 +115,8 @@ class Context {
 
  private:
   void* stream_ = nullptr;
+  bool stream_pooled_ = false;
+  int stream_device_ = 0;
   void* workspace_ = nullptr;
   size_t workspace_bytes_ = 0;
   size_t workspace_used_ = 0;

@@ -871,3 +871,36 @@ def test_convolution_only_forces_out_what_it_conflicts_with():
     sess.compute(graph=True)
     for n, v in eager.items():
         np.testing.assert_array_equal(sess.get_output(n, "NHWC"), v)
+
+
+def test_sessions_take_their_streams_from_one_pool():
+    """The first four sessions alive on the device get streams that were created together (so
+    they sit on different hardware queues whatever streams the application creates in between);
+    a closed session's stream goes to the next session; further sessions get streams of their
+    own.  Outputs do not depend on which stream a session got."""
+    import gc
+    import torch
+    gc.collect()   # sessions of earlier tests give their streams back
+    g, info = models.mobilenet_v1_ssd(1, seed=5)
+    x = rng(7).uniform(-1, 1, (1, 300, 300, 3)).astype(np.float32)
+    made, other = [], []
+    for _ in range(4):
+        s = session.Session()
+        s.load_graph(g)
+        made.append(s)
+        other.append(torch.cuda.Stream())   # an unrelated stream between two sessions
+    streams = [int(s.stream or 0) for s in made]
+    assert all(streams) and len(set(streams)) == 4
+    fifth = session.Session()
+    fifth.load_graph(g)
+    assert int(fifth.stream) not in streams
+    made[1].run({"input": x})
+    ref = made[1].get_output("cls_logits", "ANY")
+    made[1].close()
+    again = session.Session()
+    again.load_graph(g)
+    assert int(again.stream) == streams[1]
+    again.run({"input": x})
+    np.testing.assert_array_equal(again.get_output("cls_logits", "ANY"), ref)
+    fifth.run({"input": x})
+    np.testing.assert_array_equal(fifth.get_output("cls_logits", "ANY"), ref)
