@@ -91,6 +91,29 @@ __device__ __forceinline__ float from_f32<float>(float v) { return v; }
 template <>
 __device__ __forceinline__ __half from_f32<__half>(float v) { return __float2half_rn(v); }
 
+
+// Result stores.  A kernel's results are written through to memory (system scope) while it
+// runs.  Left dirty in the L2s they are all written back at the end of the kernel, when
+// nothing is left to overlap the write-back with; measured on MI355X the depthwise layers
+// of the network are 7 % faster this way, the fp16 GEMM of 12 GFLOP 13 %, a whole batch-16
+// pass 1.5 %.  (Non-temporal stores were slower than plain ones.)
+constexpr int kResultStoreAux = 17;   // raw buffer stores: sc0 | sc1
+__device__ __forceinline__ void store_result16(void* dst, float4 v) {
+  typedef float f32x4_t __attribute__((ext_vector_type(4)));
+  const f32x4_t t = {v.x, v.y, v.z, v.w};
+  asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(dst), "v"(t) : "memory");
+}
+__device__ __forceinline__ void store_result16(void* dst, uint4 v) {
+  typedef unsigned u32x4_t __attribute__((ext_vector_type(4)));
+  const u32x4_t t = {v.x, v.y, v.z, v.w};
+  asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(dst), "v"(t) : "memory");
+}
+__device__ __forceinline__ void store_result8(void* dst, uint2 v) {
+  typedef unsigned u32x2_t __attribute__((ext_vector_type(2)));
+  const u32x2_t t = {v.x, v.y};
+  asm volatile("global_store_dwordx2 %0, %1, off sc0 sc1" ::"v"(dst), "v"(t) : "memory");
+}
+
 // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.
 // Remaps the linear workgroup id so that consecutive logical ids land on the
 // same XCD, keeping tiles that share operands in one L2.

@@ -108,10 +108,10 @@ __device__ __forceinline__ float stem_load(__amdgpu_buffer_rsrc_t r, unsigned by
 template <typename T>
 __device__ __forceinline__ void stem_store(__amdgpu_buffer_rsrc_t r, unsigned byte_off, float v) {
   if constexpr (sizeof(T) == 4) {
-    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), r, (int)byte_off, 0, 0);
+    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), r, (int)byte_off, 0, kResultStoreAux);
   } else {
     __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(unsigned short, __float2half_rn(v)), r,
-                                          (int)byte_off, 0, 0);
+                                          (int)byte_off, 0, kResultStoreAux);
   }
 }
 
@@ -284,7 +284,7 @@ __global__ __launch_bounds__(256) void conv_stem_rgb_mfma(
         const int dr = (r >> 2) * 8 + (r & 3);
         __builtin_amdgcn_raw_buffer_store_b32(
             __builtin_bit_cast(unsigned, apply_epilogue(acc[r] + bias_v, ep)), ry,
-            (int)(off0 + (unsigned)(dr * o) * 4u), 0, 0);
+            (int)(off0 + (unsigned)(dr * o) * 4u), 0, kResultStoreAux);
       }
     }
   }

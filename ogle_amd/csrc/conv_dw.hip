@@ -200,7 +200,7 @@ __global__ __launch_bounds__(256) void dwconv3x3_rows(
 #pragma unroll
           for (int v = 0; v < V; ++v) out[v] = apply_epilogue(acc[q][v], ep);
           const unsigned off = ox0 + q < ow ? out_off + (unsigned)(q * c) * ESZ : kOut;
-          __builtin_amdgcn_raw_buffer_store_b128(Vec<T>::pack(out), ry, (int)off, 0, 0);
+          __builtin_amdgcn_raw_buffer_store_b128(Vec<T>::pack(out), ry, (int)off, 0, kResultStoreAux);
         }
         out_off += out_row_bytes;
       }

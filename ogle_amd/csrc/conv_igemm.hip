@@ -456,7 +456,7 @@ __device__ __forceinline__ void igemm_tile(
               v.w = apply_epilogue(v.w + bias4.w, ep);
             }
             const long at = pdst != nullptr ? (long)grow * dpitch : out_row_offset(g, grow, dpitch);
-            *reinterpret_cast<float4*>(dbase + at + dcol) = v;
+            store_result16(dbase + at + dcol, v);
           }
         }
       }
@@ -504,7 +504,7 @@ __device__ __forceinline__ void igemm_tile(
               for (int q = 0; q < 4; ++q)
                 h[q] = __floats2half2_rn(apply_epilogue(f[2 * q] + bias8[2 * q], ep),
                                          apply_epilogue(f[2 * q + 1] + bias8[2 * q + 1], ep));
-              *reinterpret_cast<uint4*>(reinterpret_cast<__half*>(y) + out_row_offset(g, grow, g.o) + col) = packed;
+              store_result16(reinterpret_cast<__half*>(y) + out_row_offset(g, grow, g.o) + col, packed);
             }
           }
         }
@@ -828,13 +828,13 @@ __device__ __forceinline__ void igemm_wave_tile(
   T* dst = y + out_row_offset(g, grow, g.o) + gcol;
   if ((g.o & 3) == 0 && (g.oimg & 3) == 0) {
     if constexpr (sizeof(T) == 4) {
-      *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+      store_result16(dst, make_float4(v[0], v[1], v[2], v[3]));
     } else {
       const __half2 lo = __floats2half2_rn(v[0], v[1]), hi = __floats2half2_rn(v[2], v[3]);
       uint2 packed;
       packed.x = *reinterpret_cast<const unsigned*>(&lo);
       packed.y = *reinterpret_cast<const unsigned*>(&hi);
-      *reinterpret_cast<uint2*>(dst) = packed;
+      store_result8(dst, packed);
     }
   } else {
 #pragma unroll
@@ -914,7 +914,7 @@ __device__ __forceinline__ void splitk_reduce_block(const ReduceProblem& r, int 
     at = b * r.oimg + (row - b * r.hw) * r.o;
   }
   if (sizeof(T) == 4 && r.y2 == nullptr && (r.o & 3) == 0 && (r.oimg & 3) == 0) {
-    *reinterpret_cast<float4*>(static_cast<float*>(r.y) + at + col) = make_float4(v[0], v[1], v[2], v[3]);
+    store_result16(static_cast<float*>(r.y) + at + col, make_float4(v[0], v[1], v[2], v[3]));
     return;
   }
 #pragma unroll

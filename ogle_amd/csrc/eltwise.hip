@@ -23,7 +23,7 @@ struct Vec4<float> {
     v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
   }
   __device__ static __forceinline__ void store(float* p, const float v[4]) {
-    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+    store_result16(p, make_float4(v[0], v[1], v[2], v[3]));
   }
 };
 template <>
@@ -39,7 +39,7 @@ struct Vec4<__half> {
     uint2 t;
     t.x = *reinterpret_cast<const unsigned*>(&lo);
     t.y = *reinterpret_cast<const unsigned*>(&hi);
-    *reinterpret_cast<uint2*>(p) = t;
+    store_result8(p, t);
   }
 };
 

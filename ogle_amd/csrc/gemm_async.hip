@@ -338,7 +338,7 @@ __global__ __launch_bounds__(64 * WM * WN, 1) void pw_gemm_async_kernel(AsyncPro
           const int img = m / p.hw;
           row_at = (long)img * p.oimg + (long)(m - img * p.hw) * p.n;
         }
-        *reinterpret_cast<u32x4*>(y + row_at + ocol) = v;
+        store_result16(y + row_at + ocol, make_uint4(v[0], v[1], v[2], v[3]));
       }
     }
   }

@@ -66,7 +66,7 @@ __global__ __launch_bounds__(256) void pool_kernel(const T* __restrict__ x, T* _
     }
     T* q = y + (((long)b * oh + oy) * ow + ox) * c + cg * V;
     if constexpr (V == 4 && sizeof(T) == 4) {
-      *reinterpret_cast<float4*>(q) = make_float4(v[0], v[1], v[2], v[3]);
+      store_result16(q, make_float4(v[0], v[1], v[2], v[3]));
     } else {
 #pragma unroll
       for (int j = 0; j < V; ++j) q[j] = from_f32<T>(v[j]);
@@ -170,7 +170,7 @@ __global__ __launch_bounds__(256) void pool_small_kernel(
   out.z = __float_as_uint(v[2]); out.w = __float_as_uint(v[3]);
   const unsigned off = ((b * (unsigned)oh + (unsigned)oy) * (unsigned)ow + (unsigned)ox) *
                            (unsigned)c * 4u + cg * 16u;
-  __builtin_amdgcn_raw_buffer_store_b128(out, ry, (int)off, 0, 0);
+  __builtin_amdgcn_raw_buffer_store_b128(out, ry, (int)off, 0, kResultStoreAux);
 }
 
 // Global average pooling with large windows: one workgroup per (image, 64
