@@ -200,8 +200,13 @@ __global__ __launch_bounds__(64 * WM * WN, 1) void pw_gemm_async_kernel(AsyncPro
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
 
+  // Two groups of waves (see the loop below).  Group 1 requests NST - 1 stages ahead of the
+  // one it reads, group 0 one stage less.
+  static_assert(NST >= 4 && NW % 2 == 0, "ping-pong needs two wave groups and four stages");
+  const int grp = wave / (NW / 2);
 #pragma unroll
-  for (int s = 0; s < NST - 1; ++s) request_stage(s);
+  for (int s = 0; s < NST - 2; ++s) request_stage(s);
+  if (grp == 1) request_stage(NST - 2);
 
   // the tile's bias values wait in LDS behind the stage ring for the epilogue
   float* const bias_lds = reinterpret_cast<float*>(lds + NST * STAGE);
@@ -251,36 +256,60 @@ __global__ __launch_bounds__(64 * WM * WN, 1) void pw_gemm_async_kernel(AsyncPro
       }
     }
   };
-  // A barrier the instruction scheduler does not move anything across: the two halves of
-  // the loop body must stay on their own sides of it.
+  // A barrier without the fence of __syncthreads(): it waits for no memory operation of the
+  // wave, so operand reads issued before it may still be in flight behind it.  Neither the
+  // compiler nor the instruction scheduler moves anything across it.
 #define OGLE_PHASE_BARRIER()              \
   __builtin_amdgcn_sched_barrier(0);      \
-  __syncthreads();                        \
+  asm volatile("" ::: "memory");          \
+  __builtin_amdgcn_s_barrier();           \
+  asm volatile("" ::: "memory");          \
   __builtin_amdgcn_sched_barrier(0)
 
   // Two groups of waves, one wave of each on every SIMD, take turns: while one group reads
   // its operands of a stage from LDS and requests a further stage ("memory phase"), the
   // other issues the MFMAs of the stage it read before ("compute phase"); a barrier ends
-  // every phase, so the MFMA pipe always has one wave feeding it and the LDS latency of the
-  // other is hidden behind it.  Group 1 runs half a step behind group 0.
-  //   group 0:  M0 | C0 | M1 | C1 | ...
-  //   group 1:   - | M0 | C0 | M1 | ...
-  // Before a wave's memory phase of stage s: its own pieces of stage s + 1 have landed
-  // (waited for here; those of stage s one phase earlier), every wave's pieces of stage s
-  // were waited for in its previous memory phase, at least one barrier ago, and stage s - 1
-  // has been read by both groups, so its buffer takes stage s + NST - 1.
-  static_assert(NST >= 4 && NW % 2 == 0, "ping-pong needs two wave groups and four stages");
-  const int grp = wave / (NW / 2);
-  wait_loads_outstanding<LPW * (NST - 2)>();
+  // every phase.  Group 1 runs one phase behind group 0:
+  //   phase      2s      2s+1    2s+2
+  //   group 0:   M(s)    C(s)    M(s+1)
+  //   group 1:   C(s-1)  M(s)    C(s)
+  // The barriers do not wait for the LDS reads of a memory phase: their data arrive while the
+  // first MFMAs of the compute phase that follows are issued (every value read is consumed
+  // by an MFMA of that phase, so at its end the reads are complete).  What keeps the ring
+  // consistent:
+  //  - a stage is read after it has landed: before the barrier that ends phase 2s - 1 every
+  //    wave waits for its own pieces of stage s, which group 0 reads in phase 2s and group 1
+  //    in phase 2s + 1;
+  //  - a buffer is overwritten after it has been read: stage s has been read completely at
+  //    the end of phase 2s + 1 by group 0 and of phase 2s + 2 by group 1, so the request that
+  //    reuses its buffer (for stage s + NST) is issued in phase 2s + 3 or later: group 1 does
+  //    that in M(s + 1), i.e. it requests NST - 1 stages ahead; group 0's first memory phase
+  //    late enough is M(s + 2), so it requests NST - 2 stages ahead.
+  if (grp == 0) {
+    wait_loads_outstanding<LPW * (NST - 3)>();   // own pieces of stage 0
+  } else {
+    wait_loads_outstanding<LPW * (NST - 2)>();   // the same, with one more stage in flight
+  }
   OGLE_PHASE_BARRIER();
-  if (grp == 1) { OGLE_PHASE_BARRIER(); }
-  for (int s = 0; s < stages; ++s) {
-    wait_loads_outstanding<LPW * (NST - 3)>();
-    read_stage(s);
-    request_stage(s + NST - 1);
+  if (grp == 0) {
+    for (int s = 0; s < stages; ++s) {
+      read_stage(s);
+      request_stage(s + NST - 2);
+      OGLE_PHASE_BARRIER();
+      multiply_stage();
+      wait_loads_outstanding<LPW * (NST - 3)>();   // own pieces of stage s + 1
+      OGLE_PHASE_BARRIER();
+    }
+  } else {
     OGLE_PHASE_BARRIER();
-    multiply_stage();
-    if (grp == 0 || s + 1 < stages) { OGLE_PHASE_BARRIER(); }
+    for (int s = 0; s < stages; ++s) {
+      read_stage(s);
+      request_stage(s + NST - 1);
+      wait_loads_outstanding<LPW * (NST - 2)>();   // own pieces of stage s + 1
+      OGLE_PHASE_BARRIER();
+      multiply_stage();
+      if (s + 1 < stages) { OGLE_PHASE_BARRIER(); }
+    }
   }
 #undef OGLE_PHASE_BARRIER
   // the zero-filled requests past the last stage still write LDS: they must have landed
