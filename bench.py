@@ -582,7 +582,25 @@ def main():
     single["with_detection_readback"] = {
         "images_per_s": round(args.batch / (rb_ms * 1e-3), 1), "ms_per_step": round(rb_ms, 4),
         "detections_per_step": kept / args.steps,
-        "note": "one pass, then wait and copy the final lists to the host, then the next pass"}
+        "note": "one pass, then wait for the stream and copy the final lists to the host (pageable copies, the "
+                "lists unpacked into Python objects), then the next pass; driven from Python step by step"}
+    if use_graph:
+        # the same serial loop inside the runtime: the pass ends with one copy of the final
+        # lists to page-locked memory (part of the replayed graph), the host waits for the
+        # event behind the pass, reads the lists, and only then launches the next pass
+        def run_serial_readback(k):
+            return _session.Session.time_pipelined_readback([sess], 0, k)[0]
+        _session.Session.time_pipelined_readback([sess], max(args.warmup, 3), max(args.warmup, 3))
+        srb = timed_regions(run_serial_readback, args.repeats)
+        srb_ms = float(np.median(srb))
+        _, seen = _session.Session.time_pipelined_readback([sess], 0, args.steps)
+        single["serial_readback"] = {
+            "images_per_s": round(args.batch * args.steps / (srb_ms * 1e-3), 1),
+            "ms_per_step": round(srb_ms / args.steps, 4), "ms_per_step_spread": spread(srb),
+            "detections_per_step": seen / args.steps,
+            "note": "one session, one pass at a time, the host holds every pass's final lists before it launches "
+                    "the next (nn/main.cc:76-111 times Run + GetOutputs the same way): the lists are copied to "
+                    "page-locked memory inside the replayed graph and the host waits for one event per pass"}
     if streams == 1:
         region_ms = single_ms
     else:
