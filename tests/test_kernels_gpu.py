@@ -1024,6 +1024,7 @@ ASYNC_F16_CASES = [
     (8, 64, 63, 264, 512, True, H.ACT_CLIP, 0),      # 256x256 tiles; ragged M; K ends inside a stage
     (32, 19, 19, 512, 1000, True, H.ACT_RELU, 0),    # 192x256 tiles; ragged M and N (config 3's M, K)
     (32, 19, 19, 256, 768, False, H.ACT_NONE, 64),   # no bias, images stored with a gap after each
+    (36, 19, 19, 2048, 512, True, H.ACT_RELU, 0),    # a long contraction: the stage ring turns 16 times
 ]
 
 
