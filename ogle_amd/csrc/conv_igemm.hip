@@ -151,12 +151,18 @@ __device__ __forceinline__ void igemm_tile(
   constexpr int RPP = 256 / VPR;       // rows one pass of the workgroup loads
   constexpr int AP = (BM + RPP - 1) / RPP, BP = (BN + RPP - 1) / RPP;
   constexpr bool A_PART = BM % RPP != 0, B_PART = BN % RPP != 0;  // last pass partly idle
-  constexpr int LROW = ROWB + 16;      // padded LDS row, bytes
+  // LDS rows.  fp32 slabs under 32x32 MFMA blocks: 64-byte rows whose four 16-byte K groups
+  // are permuted by (row >> 2) & 3, which keeps both the operand reads and the staging
+  // writes free of bank conflicts (a 16-byte LDS access is served 16 lanes per cycle: those
+  // with the same lane / 32 and the same parity of (lane >> 2) & 7; they must fall into 16
+  // different 16-byte columns of a 256-byte window).  Otherwise rows padded by 16 bytes.
+  constexpr bool SWZ = ROWB == 64 && MB == 32;
+  constexpr int LROW = SWZ ? ROWB : ROWB + 16;   // LDS row pitch, bytes
   constexpr int ESZ = (int)sizeof(T);
   constexpr int CHUNKB = (64 / MB) * 16;  // bytes of a row one MFMA step consumes (64 / MB lane groups x 16)
   constexpr int CHUNKS = ROWB / CHUNKB;
   static_assert(CHUNKS >= 1, "a K slab holds at least one MFMA step");
-  constexpr int STAGE = (BM + BN) * LROW;  // one buffer: A rows then B rows
+  constexpr int STAGE = (BM + BN) * (ROWB + 16);  // one buffer: A rows then B rows
 
   static_assert(2 * STAGE == igemm_lds_bytes<BM, BN, ROWB>(), "LDS size");
 
@@ -292,7 +298,8 @@ __device__ __forceinline__ void igemm_tile(
   // Writes ra / rb into LDS buffer `buf`.
 #define OGLE_STORE_SLAB(buf, SET)                                                            \
   {                                                                                          \
-    unsigned char* base_ = lds + (buf) * STAGE + vrow * LROW + vcol * 16;                    \
+    unsigned char* base_ = lds + (buf) * STAGE + vrow * LROW +                               \
+                           (SWZ ? (vcol ^ ((vrow >> 2) & 3)) : vcol) * 16;                   \
     _Pragma("unroll") for (int p = 0; p < AP; ++p)                                           \
       if (!A_PART || p * RPP + vrow < BM)                                                    \
         *reinterpret_cast<u32x4*>(base_ + p * RPP * LROW) = ra[SET][p];                      \
@@ -322,14 +329,17 @@ __device__ __forceinline__ void igemm_tile(
   // One K slab from LDS buffer `buf` into the accumulators.
 #define OGLE_COMPUTE_SLAB(buf)                                                               \
   {                                                                                          \
-    const unsigned char* pa = lds + (buf) * STAGE + (wave_m * WTM + lrow) * LROW + lq * 16;  \
-    const unsigned char* pb = lds + (buf) * STAGE + (BM + wave_n * WTN + lrow) * LROW + lq * 16; \
+    const unsigned char* pa = lds + (buf) * STAGE + (wave_m * WTM + lrow) * LROW;            \
+    const unsigned char* pb = lds + (buf) * STAGE + (BM + wave_n * WTN + lrow) * LROW;       \
     _Pragma("unroll") for (int ch = 0; ch < CHUNKS; ++ch) {                                  \
+      /* this lane's 16-byte K group of the step (rows 32 apart share the permutation) */    \
+      const int kof = SWZ ? (((ch * (CHUNKB / 16) + lq) ^ ((lrow >> 2) & 3)) * 16)           \
+                          : lq * 16 + ch * CHUNKB;                                           \
       u32x4 av[TM], bv[TN];                                                                  \
       _Pragma("unroll") for (int i = 0; i < TM; ++i)                                         \
-        av[i] = *reinterpret_cast<const u32x4*>(pa + i * MB * LROW + ch * CHUNKB);           \
+        av[i] = *reinterpret_cast<const u32x4*>(pa + i * MB * LROW + kof);                   \
       _Pragma("unroll") for (int j = 0; j < TN; ++j)                                         \
-        bv[j] = *reinterpret_cast<const u32x4*>(pb + j * MB * LROW + ch * CHUNKB);           \
+        bv[j] = *reinterpret_cast<const u32x4*>(pb + j * MB * LROW + kof);                   \
       _Pragma("unroll") for (int i = 0; i < TM; ++i)                                         \
         _Pragma("unroll") for (int j = 0; j < TN; ++j)                                       \
           WaveMma<T, MB>::run(av[i], bv[j], acc[i][j]);                                      \
