@@ -151,13 +151,17 @@ __device__ __forceinline__ void igemm_tile(
   constexpr int RPP = 256 / VPR;       // rows one pass of the workgroup loads
   constexpr int AP = (BM + RPP - 1) / RPP, BP = (BN + RPP - 1) / RPP;
   constexpr bool A_PART = BM % RPP != 0, B_PART = BN % RPP != 0;  // last pass partly idle
-  // LDS rows.  fp32 slabs under 32x32 MFMA blocks: 64-byte rows whose four 16-byte K groups
-  // are permuted by (row >> 2) & 3, which keeps both the operand reads and the staging
-  // writes free of bank conflicts (a 16-byte LDS access is served 16 lanes per cycle: those
-  // with the same lane / 32 and the same parity of (lane >> 2) & 7; they must fall into 16
-  // different 16-byte columns of a 256-byte window).  Otherwise rows padded by 16 bytes.
-  constexpr bool SWZ = ROWB == 64 && MB == 32;
+  // LDS rows.  Under 32x32 MFMA blocks a row is exactly its slab bytes and its 16-byte K groups
+  // are permuted by a function of the row: (row >> 2) & 3 for 64-byte rows, (row >> 1) & 7 for
+  // 128-byte rows.  That keeps both the operand reads and the staging writes free of bank
+  // conflicts (a 16-byte LDS access is served 16 lanes per cycle: those with the same
+  // lane / 32 and the same parity of (lane >> 2) & 7; they must fall into 16 different 16-byte
+  // columns of a 256-byte window; found by exhaustive search over XOR functions of the row
+  // bits against that model, confirmed by SQ_LDS_BANK_CONFLICT: 1.58 M -> 0.05 M cycles per
+  // launch of a 19x19x512 -> 512 pointwise layer at batch 16).  Otherwise rows padded by 16 bytes.
+  constexpr bool SWZ = MB == 32 && (ROWB == 64 || ROWB == 128);
   constexpr int LROW = SWZ ? ROWB : ROWB + 16;   // LDS row pitch, bytes
+  auto row_perm = [](int row) { return ROWB == 64 ? (row >> 2) & 3 : (row >> 1) & 7; };
   constexpr int ESZ = (int)sizeof(T);
   constexpr int CHUNKB = (64 / MB) * 16;  // bytes of a row one MFMA step consumes (64 / MB lane groups x 16)
   constexpr int CHUNKS = ROWB / CHUNKB;
@@ -299,7 +303,7 @@ __device__ __forceinline__ void igemm_tile(
 #define OGLE_STORE_SLAB(buf, SET)                                                            \
   {                                                                                          \
     unsigned char* base_ = lds + (buf) * STAGE + vrow * LROW +                               \
-                           (SWZ ? (vcol ^ ((vrow >> 2) & 3)) : vcol) * 16;                   \
+                           (SWZ ? (vcol ^ row_perm(vrow)) : vcol) * 16;                      \
     _Pragma("unroll") for (int p = 0; p < AP; ++p)                                           \
       if (!A_PART || p * RPP + vrow < BM)                                                    \
         *reinterpret_cast<u32x4*>(base_ + p * RPP * LROW) = ra[SET][p];                      \
@@ -333,7 +337,7 @@ __device__ __forceinline__ void igemm_tile(
     const unsigned char* pb = lds + (buf) * STAGE + (BM + wave_n * WTN + lrow) * LROW;       \
     _Pragma("unroll") for (int ch = 0; ch < CHUNKS; ++ch) {                                  \
       /* this lane's 16-byte K group of the step (rows 32 apart share the permutation) */    \
-      const int kof = SWZ ? (((ch * (CHUNKB / 16) + lq) ^ ((lrow >> 2) & 3)) * 16)           \
+      const int kof = SWZ ? (((ch * (CHUNKB / 16) + lq) ^ row_perm(lrow)) * 16)              \
                           : lq * 16 + ch * CHUNKB;                                           \
       u32x4 av[TM], bv[TN];                                                                  \
       _Pragma("unroll") for (int i = 0; i < TM; ++i)                                         \
