@@ -151,17 +151,22 @@ __device__ __forceinline__ void igemm_tile(
   constexpr int RPP = 256 / VPR;       // rows one pass of the workgroup loads
   constexpr int AP = (BM + RPP - 1) / RPP, BP = (BN + RPP - 1) / RPP;
   constexpr bool A_PART = BM % RPP != 0, B_PART = BN % RPP != 0;  // last pass partly idle
-  // LDS rows.  Under 32x32 MFMA blocks a row is exactly its slab bytes and its 16-byte K groups
-  // are permuted by a function of the row: (row >> 2) & 3 for 64-byte rows, (row >> 1) & 7 for
-  // 128-byte rows.  That keeps both the operand reads and the staging writes free of bank
-  // conflicts (a 16-byte LDS access is served 16 lanes per cycle: those with the same
-  // lane / 32 and the same parity of (lane >> 2) & 7; they must fall into 16 different 16-byte
-  // columns of a 256-byte window; found by exhaustive search over XOR functions of the row
-  // bits against that model, confirmed by SQ_LDS_BANK_CONFLICT: 1.58 M -> 0.05 M cycles per
-  // launch of a 19x19x512 -> 512 pointwise layer at batch 16).  Otherwise rows padded by 16 bytes.
-  constexpr bool SWZ = MB == 32 && (ROWB == 64 || ROWB == 128);
+  // LDS rows.  A row is exactly its slab bytes and its 16-byte K groups are permuted by a
+  // function of the row: (row >> 1) & 7 for 128-byte rows; for 64-byte rows (row >> 2) & 3
+  // under 32x32 MFMA blocks and 2 * ((row >> 2) & 1) under 16x16 blocks.  That keeps both the
+  // operand reads and the staging writes free of bank conflicts (a 16-byte LDS access is
+  // served 16 lanes per cycle: those with the same lane / 32 and the same parity of
+  // (lane >> 2) & 7; they must fall into 16 different 16-byte columns of a 256-byte window;
+  // found by exhaustive search over XOR functions of the row bits against that model,
+  // confirmed by SQ_LDS_BANK_CONFLICT: 1.58 M -> 0.05 M cycles per launch of a
+  // 19x19x512 -> 512 pointwise layer at batch 16; rows padded by 16 bytes, as before, cost the
+  // writes three times and the 16x16 reads twice the conflict-free cycles).  Other slab
+  // widths: rows padded by 16 bytes.
+  constexpr bool SWZ = ROWB == 64 || ROWB == 128;
   constexpr int LROW = SWZ ? ROWB : ROWB + 16;   // LDS row pitch, bytes
-  auto row_perm = [](int row) { return ROWB == 64 ? (row >> 2) & 3 : (row >> 1) & 7; };
+  auto row_perm = [](int row) {
+    return ROWB == 128 ? (row >> 1) & 7 : MB == 32 ? (row >> 2) & 3 : ((row >> 2) & 1) << 1;
+  };
   constexpr int ESZ = (int)sizeof(T);
   constexpr int CHUNKB = (64 / MB) * 16;  // bytes of a row one MFMA step consumes (64 / MB lane groups x 16)
   constexpr int CHUNKS = ROWB / CHUNKB;
